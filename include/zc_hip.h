@@ -1,0 +1,171 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of ZeroCool's mixture-of-experts
+ * layer path.  Plain pointers and sizes only; every data pointer is a DEVICE
+ * pointer unless the parameter name says host.  Each entry point replaces one
+ * piece of the reference's operator layer (include/engine/metal.hpp,
+ * src/engine/metal.mm), cited beside it.
+ *
+ * Execution model (metal.hpp:45-47): calls only ENQUEUE work on the context's
+ * stream; results are defined after zc_hip_finish() or after zc_hip_wait() on a
+ * ticket taken later.  Errors: every call returns a zc_status; the text is in
+ * zc_hip_last_error() (thread local).  The C++ shim turns the status back into
+ * the reference's exception classes.
+ */
+#ifndef ZC_HIP_H
+#define ZC_HIP_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    ZC_OK = 0,
+    ZC_INVALID_ARGUMENT = 1, /* std::invalid_argument in the reference */
+    ZC_RUNTIME_ERROR = 2,    /* std::runtime_error ("HIP execution: …", "invalid router output") */
+    ZC_LOGIC_ERROR = 3,      /* std::logic_error (protocol misuse) */
+    ZC_OUT_OF_RANGE = 4,     /* std::out_of_range */
+    ZC_BUDGET_EXCEEDED = 5   /* "engine memory budget exceeded", metal.mm:395 */
+} zc_status;
+
+typedef struct zc_hip_ctx zc_hip_ctx;
+
+/* metal.hpp:8-13 (Linear) with bindings resolved to device addresses.
+ * quantized: affine Q4/Q8 (qwen.metal:46-62, 112-125); otherwise a plain matrix of
+ * dtype 0 = BF16, 1 = F32 (qwen.metal:23-27). */
+typedef struct {
+    const void* weight;
+    const void* scales;
+    const void* biases;
+    uint32_t input, output, group, dtype;
+    uint32_t quantized, bits;
+} zc_linear;
+
+/* Shapes the reference hard-codes (storage.hpp:26-27) become parameters. */
+typedef struct {
+    uint32_t hidden, experts, topk, inter, group;
+    uint32_t bits_gate_up, bits_down;               /* routed experts */
+    uint32_t shared_bits_gate_up, shared_bits_down; /* shared expert */
+} zc_moe_config;
+
+/* One layer's weights: what Model::moe reads through Resident and the expert
+ * store (model.cpp:433-434, 483-485, 508-513).  A record is
+ * [gate W,S,B | up W,S,B | down W,S,B] (metal.mm:1124-1129). */
+typedef struct {
+    const void* router;          /* [E][H] BF16 */
+    const float* router_offsets; /* [E] fp32 added to the logits, or NULL (benchmark load skew) */
+    const void* shared_gate;     /* [1][H] BF16, shared_expert_gate */
+    const void* shared_record;   /* shared expert record */
+    const void* expert_records;  /* E records, record_stride bytes apart */
+    uint64_t record_stride;
+} zc_moe_layer;
+
+const char* zc_hip_last_error(void);
+const char* zc_hip_version(void);
+
+/* Metal::Metal / ~Metal (metal.mm:291-355), Metal::budget (metal.hpp:70). budget 0 = unlimited. */
+zc_status zc_hip_create(int device, uint64_t budget_bytes, zc_hip_ctx** out);
+zc_status zc_hip_destroy(zc_hip_ctx* ctx);
+/* Metal::allocate / zeros / upload (metal.hpp:61-65); download stands in for reading Buffer::data. */
+zc_status zc_hip_alloc(zc_hip_ctx* ctx, uint64_t bytes, void** out);
+zc_status zc_hip_free(zc_hip_ctx* ctx, void* ptr);
+zc_status zc_hip_memset(zc_hip_ctx* ctx, void* dst, int byte, uint64_t bytes);
+zc_status zc_hip_upload(zc_hip_ctx* ctx, void* dst, const void* host_src, uint64_t bytes);
+zc_status zc_hip_download(zc_hip_ctx* ctx, void* host_dst, const void* src, uint64_t bytes);
+/* Metal::copy (metal.hpp:66-68) */
+zc_status zc_hip_copy(zc_hip_ctx* ctx, void* dst, const void* src, uint64_t bytes);
+/* Metal::allocated / peak (metal.hpp:127-128) */
+uint64_t zc_hip_allocated(const zc_hip_ctx* ctx);
+uint64_t zc_hip_peak(const zc_hip_ctx* ctx);
+/* Metal::submit / wait / finish (metal.hpp:105-108): a ticket is done when all work
+ * enqueued before it has run. */
+zc_status zc_hip_submit(zc_hip_ctx* ctx, uint64_t* ticket);
+zc_status zc_hip_wait(zc_hip_ctx* ctx, uint64_t ticket);
+zc_status zc_hip_finish(zc_hip_ctx* ctx);
+/* The raw hipStream_t the context enqueues on (for event timing by the caller). */
+void* zc_hip_stream(zc_hip_ctx* ctx);
+
+/* Metal::linear_into (metal.mm:775-827): quantized -> q4_mm/q8_mm arithmetic;
+ * plain -> plain_mm (qwen.metal:499-506). out[tokens][output]. */
+zc_status zc_hip_linear_into(zc_hip_ctx* ctx, const zc_linear* layer, const float* x,
+                             uint32_t tokens, float* out, int float_output);
+/* The router branch of linear_into (metal.mm:818-822; qwen.metal:512-534). */
+zc_status zc_hip_router_logits(zc_hip_ctx* ctx, const void* w_bf16, const float* x, uint32_t tokens,
+                               uint32_t hidden, uint32_t experts, const float* offsets, float* logits);
+/* Metal::gated_linear (metal.mm:845-880; qwen.metal:71-81, 134-144). rows may be NULL.
+ * x_rows is the number of rows x holds (bounds for the gather). */
+zc_status zc_hip_gated_linear(zc_hip_ctx* ctx, const zc_linear* gate, const zc_linear* up,
+                              const float* x, uint32_t x_rows, uint32_t tokens,
+                              const int32_t* rows, float* out);
+/* Metal::route (metal.mm:261-266; qwen.metal:742-795) */
+zc_status zc_hip_route(zc_hip_ctx* ctx, const float* logits, uint32_t tokens, uint32_t experts,
+                       uint32_t topk, int32_t* ids, float* weights);
+/* The positions/selected lists Model::moe builds on the CPU (model.cpp:449-479), built on
+ * the device: offsets[E+1], slots[tokens*topk] (flat p = t*topk+k, ascending inside each
+ * expert), selected[E] (ascending ids of non-empty experts), count[1], status[1]
+ * (non-zero: an id outside [0,E) -> "invalid router output"). */
+zc_status zc_hip_build_dispatch(zc_hip_ctx* ctx, const int32_t* ids, uint32_t tokens, uint32_t topk,
+                                uint32_t experts, int32_t* offsets, int32_t* slots,
+                                int32_t* selected, int32_t* count, int32_t* status);
+/* dispatch("scatter_experts") (pipeline.cpp:28; qwen.metal:800-803) */
+zc_status zc_hip_scatter_experts(zc_hip_ctx* ctx, const float* x, const int32_t* positions,
+                                 uint32_t n, uint32_t hidden, float* out);
+/* dispatch("moe_sum") (model.cpp:555; qwen.metal:804-816) */
+zc_status zc_hip_moe_sum(zc_hip_ctx* ctx, const float* experts, const float* weights,
+                         const float* shared, const float* gate, uint32_t tokens,
+                         uint32_t hidden, uint32_t topk, float* out);
+/* Metal::grouped_experts (metal.mm:881-912): n<=8 records (host array of device
+ * pointers), distinct positions < topk (host array); scratch holds n*inter floats. */
+zc_status zc_hip_grouped_experts(zc_hip_ctx* ctx, const zc_moe_config* cfg,
+                                 const void* const* host_records, const uint32_t* host_positions,
+                                 uint32_t n, const float* x, float* out, float* scratch);
+
+/* Model::moe (model.cpp:431-557) as one enqueue with routing and dispatch kept on the
+ * device (no CPU readback).  workspace: zc_hip_moe_workspace_bytes() bytes.
+ * trace (optional, host struct of device pointers, any NULL): copies of the
+ * intermediates the reference dumps with --trace-dir (model.cpp:447-448, 549-552). */
+typedef struct {
+    float* logits;     /* [T][E]      router_<layer>  */
+    int32_t* ids;      /* [T][topk]   route_<layer>   */
+    float* weights;    /* [T][topk]   .mlp.weights    */
+    float* expert_out; /* [T][topk][H] .mlp.expert_out */
+    float* shared;     /* [T][H]      .mlp.shared     */
+    float* gate;       /* [T]         .mlp.gate       */
+} zc_moe_trace;
+uint64_t zc_hip_moe_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens);
+zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* layer,
+                             const float* x, uint32_t tokens, float* out, void* workspace,
+                             const zc_moe_trace* trace);
+/* Drains the stream, then reports ZC_RUNTIME_ERROR "invalid router output" if any
+ * zc_hip_moe_forward since the last check saw an id outside [0,E) (model.cpp:459).
+ * Clears the flag. */
+zc_status zc_hip_moe_check(zc_hip_ctx* ctx);
+
+/* Inter-layer glue of the stacked-decode workload (not reference arithmetic):
+ * y = bf(x * 1/sqrt(mean(x^2)+1e-6)) per row. */
+zc_status zc_hip_rms_glue(zc_hip_ctx* ctx, const float* x, uint32_t tokens, uint32_t hidden, float* out);
+
+/* Counter-based synthetic tensors: element i depends only on (seed, i).
+ * kind 0: uint32 words of uniform bits (Q4/Q8 codes), count = words
+ * kind 1: BF16 scale in [lo, lo+span) and BF16 bias = scale*factor, interleaved
+ *         as two arrays scales[count], biases[count]
+ * kind 2: BF16-valued N(0,1)*sigma stored as fp32, count = floats
+ * kind 3: the same stored as BF16 (uint16), count = elements */
+zc_status zc_hip_synth_words(zc_hip_ctx* ctx, uint32_t* dst, uint64_t count, uint64_t seed);
+zc_status zc_hip_synth_scales(zc_hip_ctx* ctx, uint16_t* scales, uint16_t* biases, uint64_t count,
+                              uint64_t seed, float lo, float span, float factor);
+zc_status zc_hip_synth_normal_f32(zc_hip_ctx* ctx, float* dst, uint64_t count, uint64_t seed, float sigma);
+zc_status zc_hip_synth_normal_bf16(zc_hip_ctx* ctx, uint16_t* dst, uint64_t count, uint64_t seed, float sigma);
+/* A whole expert record (or E of them, stride apart) in one launch:
+ * projection p of record r uses seed + r*3 + p. */
+zc_status zc_hip_synth_records(zc_hip_ctx* ctx, const zc_moe_config* cfg, int shared, void* records,
+                               uint64_t stride, uint32_t count, uint64_t seed);
+
+uint64_t zc_hip_projection_bytes(uint32_t input, uint32_t output, uint32_t group, uint32_t bits);
+uint64_t zc_hip_record_bytes(const zc_moe_config* cfg, int shared);
+/* expert_linear (metal.mm:1124-1129) for parameterised shapes. */
+zc_status zc_hip_expert_linear(const zc_moe_config* cfg, int shared, const void* record,
+                               int projection, zc_linear* out);
+#ifdef __cplusplus
+}
+#endif
+#endif

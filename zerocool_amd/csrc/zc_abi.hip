@@ -1,0 +1,450 @@
+// The C ABI: context, memory, validation and the enqueue of each operator.
+// Validation mirrors the reference operator layer (src/engine/metal.mm:261-266,
+// 649-661, 775-827, 845-912) so the same misuse is refused with the same class
+// of error before anything reaches the GPU.
+#include "../../include/zc_hip.h"
+#include "zc_kernels.hpp"
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace {
+thread_local std::string g_error;
+zc_status fail(zc_status code, std::string text) { g_error = std::move(text); return code; }
+
+#define ZC_HIP(call)                                                                         \
+    do {                                                                                     \
+        const hipError_t e_ = (call);                                                        \
+        if (e_ != hipSuccess) return fail(ZC_RUNTIME_ERROR, std::string("HIP execution: ") + hipGetErrorString(e_) + " in " #call); \
+    } while (0)
+#define ZC_REQUIRE(cond, text) do { if (!(cond)) return fail(ZC_INVALID_ARGUMENT, text); } while (0)
+#define ZC_LAUNCHED() ZC_HIP(hipGetLastError())
+
+bool overlaps(const void* a, uint64_t an, const void* b, uint64_t bn) {
+    const auto x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+    return a && b && x < y + bn && y < x + an;
+}
+uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+}  // namespace
+
+struct zc_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    uint64_t budget = 0, allocated = 0, peak = 0;
+    std::unordered_map<void*, uint64_t> blocks;
+    std::vector<hipEvent_t> tickets;   // live tickets: ticket t -> tickets[t - retired - 1]
+    uint64_t retired = 0;              // tickets known complete and destroyed
+    int32_t* moe_status = nullptr;     // device flag: an id outside [0,E) was seen
+    std::mutex mutex;
+};
+
+extern "C" {
+
+const char* zc_hip_last_error(void) { return g_error.c_str(); }
+const char* zc_hip_version(void) { return "zerocool-moe-mi355x 0.1 (gfx950)"; }
+
+zc_status zc_hip_create(int device, uint64_t budget_bytes, zc_hip_ctx** out) {
+    ZC_REQUIRE(out, "null context output");
+    int count = 0;
+    ZC_HIP(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(ZC_RUNTIME_ERROR, "no such HIP device");
+    ZC_HIP(hipSetDevice(device));
+    auto* ctx = new zc_hip_ctx;
+    ctx->device = device; ctx->budget = budget_bytes;
+    if (hipStreamCreate(&ctx->stream) != hipSuccess) { delete ctx; return fail(ZC_RUNTIME_ERROR, "HIP execution: cannot create stream"); }
+    if (hipMalloc(&ctx->moe_status, 256) != hipSuccess || hipMemsetAsync(ctx->moe_status, 0, 256, ctx->stream) != hipSuccess) {
+        hipStreamDestroy(ctx->stream); delete ctx; return fail(ZC_RUNTIME_ERROR, "HIP execution: cannot allocate status word");
+    }
+    *out = ctx;
+    return ZC_OK;
+}
+zc_status zc_hip_destroy(zc_hip_ctx* ctx) {
+    if (!ctx) return ZC_OK;
+    hipSetDevice(ctx->device);
+    hipStreamSynchronize(ctx->stream);
+    for (auto e : ctx->tickets) hipEventDestroy(e);
+    for (auto& b : ctx->blocks) hipFree(b.first);
+    hipFree(ctx->moe_status);
+    hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return ZC_OK;
+}
+zc_status zc_hip_alloc(zc_hip_ctx* ctx, uint64_t bytes, void** out) {
+    ZC_REQUIRE(ctx && out, "null argument");
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    if (ctx->budget && (bytes > ctx->budget || ctx->allocated > ctx->budget - bytes))
+        return fail(ZC_BUDGET_EXCEEDED, "engine memory budget exceeded");
+    void* p = nullptr;
+    ZC_HIP(hipSetDevice(ctx->device));
+    const hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) { (void)hipGetLastError(); return fail(ZC_BUDGET_EXCEEDED, std::string("device allocation failed: ") + hipGetErrorString(e)); }
+    ctx->blocks[p] = bytes; ctx->allocated += bytes;
+    if (ctx->allocated > ctx->peak) ctx->peak = ctx->allocated;
+    *out = p;
+    return ZC_OK;
+}
+zc_status zc_hip_free(zc_hip_ctx* ctx, void* ptr) {
+    ZC_REQUIRE(ctx, "null context");
+    if (!ptr) return ZC_OK;
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    auto it = ctx->blocks.find(ptr);
+    if (it == ctx->blocks.end()) return fail(ZC_LOGIC_ERROR, "free of a pointer this context did not allocate");
+    ZC_HIP(hipStreamSynchronize(ctx->stream));   // no GPU user may outlive its buffer
+    ZC_HIP(hipFree(ptr));
+    ctx->allocated -= it->second; ctx->blocks.erase(it);
+    return ZC_OK;
+}
+zc_status zc_hip_memset(zc_hip_ctx* ctx, void* dst, int byte, uint64_t bytes) {
+    ZC_REQUIRE(ctx && (dst || !bytes), "null argument");
+    if (bytes) ZC_HIP(hipMemsetAsync(dst, byte, bytes, ctx->stream));
+    return ZC_OK;
+}
+zc_status zc_hip_upload(zc_hip_ctx* ctx, void* dst, const void* host_src, uint64_t bytes) {
+    ZC_REQUIRE(ctx && ((dst && host_src) || !bytes), "null argument");
+    if (bytes) { ZC_HIP(hipMemcpyAsync(dst, host_src, bytes, hipMemcpyHostToDevice, ctx->stream)); ZC_HIP(hipStreamSynchronize(ctx->stream)); }
+    return ZC_OK;
+}
+zc_status zc_hip_download(zc_hip_ctx* ctx, void* host_dst, const void* src, uint64_t bytes) {
+    ZC_REQUIRE(ctx && ((host_dst && src) || !bytes), "null argument");
+    if (bytes) { ZC_HIP(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream)); ZC_HIP(hipStreamSynchronize(ctx->stream)); }
+    return ZC_OK;
+}
+zc_status zc_hip_copy(zc_hip_ctx* ctx, void* dst, const void* src, uint64_t bytes) {
+    ZC_REQUIRE(ctx && ((dst && src) || !bytes), "null argument");
+    if (bytes) ZC_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return ZC_OK;
+}
+uint64_t zc_hip_allocated(const zc_hip_ctx* ctx) { return ctx ? ctx->allocated : 0; }
+uint64_t zc_hip_peak(const zc_hip_ctx* ctx) { return ctx ? ctx->peak : 0; }
+void* zc_hip_stream(zc_hip_ctx* ctx) { return ctx ? ctx->stream : nullptr; }
+
+zc_status zc_hip_submit(zc_hip_ctx* ctx, uint64_t* ticket) {
+    ZC_REQUIRE(ctx && ticket, "null argument");
+    hipEvent_t e;
+    ZC_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    ZC_HIP(hipEventRecord(e, ctx->stream));
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->tickets.push_back(e);
+    *ticket = ctx->retired + ctx->tickets.size();
+    return ZC_OK;
+}
+zc_status zc_hip_wait(zc_hip_ctx* ctx, uint64_t ticket) {
+    ZC_REQUIRE(ctx, "null context");
+    hipEvent_t e;
+    {
+        std::lock_guard<std::mutex> lock(ctx->mutex);
+        if (!ticket || ticket > ctx->retired + ctx->tickets.size()) return fail(ZC_LOGIC_ERROR, "wait on a ticket that was never submitted");
+        if (ticket <= ctx->retired) return ZC_OK;
+        e = ctx->tickets[ticket - ctx->retired - 1];
+    }
+    ZC_HIP(hipEventSynchronize(e));
+    return ZC_OK;
+}
+zc_status zc_hip_finish(zc_hip_ctx* ctx) {
+    ZC_REQUIRE(ctx, "null context");
+    ZC_HIP(hipStreamSynchronize(ctx->stream));
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    for (auto e : ctx->tickets) hipEventDestroy(e);
+    ctx->retired += ctx->tickets.size();
+    ctx->tickets.clear();
+    return ZC_OK;
+}
+
+uint64_t zc_hip_projection_bytes(uint32_t K, uint32_t N, uint32_t group, uint32_t bits) {
+    return uint64_t(K) * N * bits / 8 + 2ull * 2 * (K / (group ? group : 64)) * N;
+}
+static void projection_shape(const zc_moe_config* c, int shared, int p, uint32_t* K, uint32_t* N, uint32_t* bits) {
+    *K = p == 2 ? c->inter : c->hidden;
+    *N = p == 2 ? c->hidden : c->inter;
+    *bits = shared ? (p == 2 ? c->shared_bits_down : c->shared_bits_gate_up) : (p == 2 ? c->bits_down : c->bits_gate_up);
+}
+uint64_t zc_hip_record_bytes(const zc_moe_config* c, int shared) {
+    uint64_t total = 0;
+    for (int p = 0; p < 3; ++p) { uint32_t K, N, b; projection_shape(c, shared, p, &K, &N, &b); total += zc_hip_projection_bytes(K, N, c->group, b); }
+    return total;
+}
+static zc_status validate_config(const zc_moe_config* c) {
+    ZC_REQUIRE(c, "null configuration");
+    ZC_REQUIRE(c->hidden && c->inter && c->experts && c->topk, "empty MoE geometry");
+    ZC_REQUIRE(c->group == 32 || c->group == 64, "unsupported affine matrix geometry");
+    ZC_REQUIRE(c->hidden % c->group == 0 && c->inter % c->group == 0, "unsupported affine matrix geometry");
+    ZC_REQUIRE(c->hidden % 16 == 0, "router needs hidden divisible by 16");
+    ZC_REQUIRE(c->experts <= 1024 && c->topk <= 128 && c->topk <= c->experts, "route selection supports at most 1024 experts and top-128");
+    for (uint32_t b : {c->bits_gate_up, c->bits_down, c->shared_bits_gate_up, c->shared_bits_down})
+        ZC_REQUIRE(b == 4 || b == 8, "unsupported affine matrix geometry");
+    return ZC_OK;
+}
+zc_status zc_hip_expert_linear(const zc_moe_config* c, int shared, const void* record, int projection, zc_linear* out) {
+    if (const zc_status s = validate_config(c)) return s;
+    ZC_REQUIRE(record && out && projection >= 0 && projection <= 2, "invalid expert projection");
+    uint64_t offset = 0; uint32_t K, N, bits;
+    for (int p = 0; p < projection; ++p) { projection_shape(c, shared, p, &K, &N, &bits); offset += zc_hip_projection_bytes(K, N, c->group, bits); }
+    projection_shape(c, shared, projection, &K, &N, &bits);
+    const uint64_t wbytes = uint64_t(K) * N * bits / 8, meta = 2ull * (K / c->group) * N;
+    const auto* r = static_cast<const uint8_t*>(record);
+    *out = zc_linear{r + offset, r + offset + wbytes, r + offset + wbytes + meta, K, N, c->group, 0, 1, bits};
+    return ZC_OK;
+}
+
+// metal.mm:649-661 without the binding-coverage test (sizes are the shim's business).
+static zc_status validate_affine(const zc_linear* l) {
+    ZC_REQUIRE(l->input && l->output && (l->bits == 4 || l->bits == 8) && (l->group == 32 || l->group == 64) &&
+               l->input % l->group == 0, "unsupported affine matrix geometry");
+    ZC_REQUIRE(l->weight && l->scales && l->biases, "affine tensor binding is truncated");
+    ZC_REQUIRE(reinterpret_cast<uintptr_t>(l->weight) % 4 == 0 && reinterpret_cast<uintptr_t>(l->scales) % 2 == 0 &&
+               reinterpret_cast<uintptr_t>(l->biases) % 2 == 0, "affine tensor binding is misaligned");
+    return ZC_OK;
+}
+static uint64_t weight_bytes(const zc_linear* l) {
+    return l->quantized ? uint64_t(l->input) * l->output * l->bits / 8 : uint64_t(l->input) * l->output * (l->dtype == 1 ? 4 : 2);
+}
+
+zc_status zc_hip_linear_into(zc_hip_ctx* ctx, const zc_linear* l, const float* x, uint32_t tokens, float* out, int float_output) {
+    ZC_REQUIRE(ctx && l, "null argument");
+    ZC_REQUIRE(tokens && l->input && l->output && x, "linear input shape");
+    ZC_REQUIRE(l->weight, "missing linear weights");
+    if (l->quantized) if (const zc_status s = validate_affine(l)) return s;
+    const uint64_t obytes = uint64_t(tokens) * l->output * 4, xbytes = uint64_t(tokens) * l->input * 4;
+    ZC_REQUIRE(out && reinterpret_cast<uintptr_t>(out) % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+               !overlaps(out, obytes, x, xbytes) && !overlaps(out, obytes, l->weight, weight_bytes(l)),
+               "invalid or overlapping linear output");
+    if (l->quantized) {
+        zc::AffineDesc a; a.gate = *l; a.x = x; a.out = out; a.tokens = tokens; a.float_output = float_output ? 1 : 0;
+        zc::launch_affine(ctx->stream, a);
+    } else {
+        ZC_REQUIRE(l->dtype <= 1, "unsupported plain matrix dtype");
+        zc::launch_plain(ctx->stream, l->weight, l->dtype, x, l->input, l->output, tokens, out, float_output != 0);
+    }
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_router_logits(zc_hip_ctx* ctx, const void* w, const float* x, uint32_t tokens, uint32_t hidden,
+                               uint32_t experts, const float* offsets, float* logits) {
+    ZC_REQUIRE(ctx && w && x && logits && tokens && experts, "linear input shape");
+    ZC_REQUIRE(hidden && hidden % 16 == 0, "router needs hidden divisible by 16");
+    ZC_REQUIRE(reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0, "router operands must be 16-byte aligned");
+    ZC_REQUIRE(!overlaps(logits, uint64_t(tokens) * experts * 4, x, uint64_t(tokens) * hidden * 4) &&
+               !overlaps(logits, uint64_t(tokens) * experts * 4, w, uint64_t(experts) * hidden * 2), "invalid or overlapping linear output");
+    zc::launch_router(ctx->stream, w, x, tokens, hidden, experts, offsets, logits);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_gated_linear(zc_hip_ctx* ctx, const zc_linear* gate, const zc_linear* up, const float* x, uint32_t x_rows,
+                              uint32_t tokens, const int32_t* rows, float* out) {
+    ZC_REQUIRE(ctx && gate && up, "null argument");
+    ZC_REQUIRE(gate->quantized && up->quantized && gate->input == up->input && gate->output == up->output &&
+               gate->group == up->group && gate->bits == up->bits, "fused gate/up requires matching affine matrices");
+    if (const zc_status s = validate_affine(gate)) return s;
+    if (const zc_status s = validate_affine(up)) return s;
+    ZC_REQUIRE(tokens && x && x_rows && (rows || x_rows >= tokens), "fused gate/up input shape");
+    ZC_REQUIRE(out && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+               !overlaps(out, uint64_t(tokens) * gate->output * 4, x, uint64_t(x_rows) * gate->input * 4), "invalid or overlapping linear output");
+    if (rows) {   // metal.mm:852-856: every gathered row must lie inside x
+        std::vector<int32_t> host(tokens);
+        ZC_HIP(hipMemcpyAsync(host.data(), rows, uint64_t(tokens) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        ZC_HIP(hipStreamSynchronize(ctx->stream));
+        for (int32_t r : host) ZC_REQUIRE(r >= 0 && uint32_t(r) < x_rows, "fused gate/up row outside input");
+    }
+    zc::AffineDesc a; a.gate = *gate; a.up = *up; a.gated = true; a.x = x; a.in_rows = rows; a.out = out; a.tokens = tokens;
+    zc::launch_affine(ctx->stream, a);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_route(zc_hip_ctx* ctx, const float* logits, uint32_t tokens, uint32_t experts, uint32_t topk, int32_t* ids, float* weights) {
+    ZC_REQUIRE(ctx && tokens && tokens <= 8192 && logits && ids && weights, "invalid route selection buffers");
+    ZC_REQUIRE(experts && experts <= 1024 && topk && topk <= 128 && topk <= experts, "route selection supports at most 1024 experts and top-128");
+    zc::launch_route(ctx->stream, logits, tokens, experts, topk, ids, weights);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_build_dispatch(zc_hip_ctx* ctx, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t experts,
+                                int32_t* offsets, int32_t* slots, int32_t* selected, int32_t* count, int32_t* status) {
+    ZC_REQUIRE(ctx && ids && offsets && slots && selected && count && status && tokens && topk && experts, "invalid dispatch buffers");
+    ZC_REQUIRE(experts <= 8192, "dispatch supports at most 8192 experts");
+    zc::launch_dispatch(ctx->stream, ids, tokens, topk, experts, offsets, slots, nullptr, selected, count, status);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_scatter_experts(zc_hip_ctx* ctx, const float* x, const int32_t* positions, uint32_t n, uint32_t hidden, float* out) {
+    ZC_REQUIRE(ctx && x && positions && out && hidden, "invalid scatter buffers");
+    if (!n) return ZC_OK;
+    zc::launch_scatter(ctx->stream, x, positions, n, hidden, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_moe_sum(zc_hip_ctx* ctx, const float* experts, const float* weights, const float* shared, const float* gate,
+                         uint32_t tokens, uint32_t hidden, uint32_t topk, float* out) {
+    ZC_REQUIRE(ctx && experts && weights && shared && gate && out && tokens && hidden && topk, "invalid expert reduction buffers");
+    zc::launch_moe_sum(ctx->stream, experts, weights, shared, gate, tokens, hidden, topk, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_grouped_experts(zc_hip_ctx* ctx, const zc_moe_config* cfg, const void* const* records,
+                                 const uint32_t* positions, uint32_t n, const float* x, float* out, float* scratch) {
+    if (const zc_status s = validate_config(cfg)) return s;
+    ZC_REQUIRE(ctx && n && n <= 8 && records && positions && x && out && scratch && x != out && x != scratch && out != scratch,
+               "invalid grouped expert geometry");
+    uint32_t seen = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        ZC_REQUIRE(records[i] && positions[i] < cfg->topk && !(positions[i] < 32 && (seen & (1u << positions[i]))) &&
+                   records[i] != out && records[i] != scratch, "invalid grouped expert record or destination");
+        for (uint32_t k = 0; k < i; ++k) ZC_REQUIRE(positions[k] != positions[i], "invalid grouped expert record or destination");
+        if (positions[i] < 32) seen |= 1u << positions[i];
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        zc_linear g, u, d;
+        zc_hip_expert_linear(cfg, 0, records[i], 0, &g); zc_hip_expert_linear(cfg, 0, records[i], 1, &u); zc_hip_expert_linear(cfg, 0, records[i], 2, &d);
+        zc::AffineDesc a; a.gate = g; a.up = u; a.gated = true; a.x = x; a.out = scratch + uint64_t(i) * cfg->inter; a.tokens = 1;
+        zc::launch_affine(ctx->stream, a);
+        zc::AffineDesc b; b.gate = d; b.x = scratch + uint64_t(i) * cfg->inter; b.out = out + uint64_t(positions[i]) * cfg->hidden; b.tokens = 1;
+        zc::launch_affine(ctx->stream, b);
+    }
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+
+// Workspace of one zc_hip_moe_forward call.
+namespace {
+struct Workspace {
+    float* logits; int32_t* ids; float* weights;
+    int32_t *offsets, *slots, *rows, *selected, *count;
+    float *act, *shared_act, *shared, *gate, *expert_out;
+    uint64_t bytes;
+};
+Workspace carve(const zc_moe_config* c, uint32_t T, void* base) {
+    Workspace w{};
+    uint64_t at = 0;
+    auto take = [&](uint64_t bytes) { void* p = base ? static_cast<uint8_t*>(base) + at : nullptr; at += align_up(bytes, 256); return p; };
+    const uint64_t n = uint64_t(T) * c->topk;
+    w.logits = (float*)take(uint64_t(T) * c->experts * 4);
+    w.ids = (int32_t*)take(n * 4); w.weights = (float*)take(n * 4);
+    w.offsets = (int32_t*)take(uint64_t(c->experts + 1) * 4); w.slots = (int32_t*)take(n * 4); w.rows = (int32_t*)take(n * 4);
+    w.selected = (int32_t*)take(uint64_t(c->experts) * 4); w.count = (int32_t*)take(4);
+    w.act = (float*)take(n * c->inter * 4); w.shared_act = (float*)take(uint64_t(T) * c->inter * 4);
+    w.shared = (float*)take(uint64_t(T) * c->hidden * 4); w.gate = (float*)take(uint64_t(T) * 4);
+    w.expert_out = (float*)take(n * c->hidden * 4);
+    w.bytes = at;
+    return w;
+}
+}  // namespace
+uint64_t zc_hip_moe_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens) {
+    if (validate_config(cfg) != ZC_OK || !tokens) return 0;
+    return carve(cfg, tokens, nullptr).bytes;
+}
+zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
+                             float* out, void* workspace, const zc_moe_trace* trace) {
+    if (const zc_status s = validate_config(c)) return s;
+    ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
+    ZC_REQUIRE(l->router && l->shared_gate && l->shared_record && l->expert_records, "missing MoE layer weights");
+    ZC_REQUIRE(l->record_stride >= zc_hip_record_bytes(c, 0) && l->record_stride % 4 == 0, "expert record stride is too small");
+    ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(workspace) % 256 == 0 &&
+               reinterpret_cast<uintptr_t>(l->router) % 16 == 0 && reinterpret_cast<uintptr_t>(l->expert_records) % 4 == 0 &&
+               reinterpret_cast<uintptr_t>(l->shared_record) % 4 == 0, "MoE layer operands are misaligned");
+    ZC_REQUIRE(x != out, "invalid or overlapping linear output");
+    const Workspace w = carve(c, T, workspace);
+    hipStream_t s = ctx->stream;
+    const uint32_t H = c->hidden, I = c->inter, E = c->experts, k = c->topk;
+    // 1-2. router logits, top-k + softmax (model.cpp:434-436)
+    zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.logits);
+    zc::launch_route(s, w.logits, T, E, k, w.ids, w.weights);
+    // 4. positions / selected, on the device (model.cpp:449-479)
+    zc::launch_dispatch(s, w.ids, T, k, E, w.offsets, w.slots, w.rows, w.selected, w.count, ctx->moe_status);
+    // 5. shared expert and its gate (model.cpp:482-485)
+    zc_linear g, u, d;
+    zc_hip_expert_linear(c, 1, l->shared_record, 0, &g); zc_hip_expert_linear(c, 1, l->shared_record, 1, &u); zc_hip_expert_linear(c, 1, l->shared_record, 2, &d);
+    { zc::AffineDesc a; a.gate = g; a.up = u; a.gated = true; a.x = x; a.out = w.shared_act; a.tokens = T; zc::launch_affine(s, a); }
+    { zc::AffineDesc a; a.gate = d; a.x = w.shared_act; a.out = w.shared; a.tokens = T; zc::launch_affine(s, a); }
+    zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.gate, false);
+    // 6. routed experts (pipeline.cpp:18-29): gate/up on gathered rows, down scattered to its slot
+    zc_linear rg, ru, rd;
+    zc_hip_expert_linear(c, 0, l->expert_records, 0, &rg); zc_hip_expert_linear(c, 0, l->expert_records, 1, &ru); zc_hip_expert_linear(c, 0, l->expert_records, 2, &rd);
+    const auto base = reinterpret_cast<uintptr_t>(l->expert_records);
+    auto off = [&](const void* p) { return uint64_t(reinterpret_cast<uintptr_t>(p) - base); };
+    const uint32_t jobs = uint32_t(std::min<uint64_t>(uint64_t(T) * k, E));
+    {
+        zc::ExpertPhaseDesc p{};
+        p.records = l->expert_records; p.stride = l->record_stride;
+        p.off[0] = off(rg.weight); p.off[1] = off(rg.scales); p.off[2] = off(rg.biases);
+        p.off[3] = off(ru.weight); p.off[4] = off(ru.scales); p.off[5] = off(ru.biases);
+        p.offsets = w.offsets; p.selected = w.selected; p.count = w.count; p.in_rows = w.rows; p.out_rows = nullptr;
+        p.x = x; p.out = w.act; p.K = H; p.N = I; p.group = c->group; p.bits = c->bits_gate_up; p.x_sorted = 0; p.max_jobs = jobs; p.gated = true;
+        zc::launch_expert_phase(s, p);
+    }
+    {
+        zc::ExpertPhaseDesc p{};
+        p.records = l->expert_records; p.stride = l->record_stride;
+        p.off[0] = off(rd.weight); p.off[1] = off(rd.scales); p.off[2] = off(rd.biases);
+        p.offsets = w.offsets; p.selected = w.selected; p.count = w.count; p.in_rows = nullptr; p.out_rows = w.slots;
+        p.x = w.act; p.out = w.expert_out; p.K = I; p.N = H; p.group = c->group; p.bits = c->bits_down; p.x_sorted = 1; p.max_jobs = jobs; p.gated = false;
+        zc::launch_expert_phase(s, p);
+    }
+    // 7. weighted combine (model.cpp:553-556)
+    zc::launch_moe_sum(s, w.expert_out, w.weights, w.shared, w.gate, T, H, k, out);
+    ZC_LAUNCHED();
+    if (trace) {
+        const uint64_t n = uint64_t(T) * k;
+        if (trace->logits) ZC_HIP(hipMemcpyAsync(trace->logits, w.logits, uint64_t(T) * E * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->ids) ZC_HIP(hipMemcpyAsync(trace->ids, w.ids, n * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->weights) ZC_HIP(hipMemcpyAsync(trace->weights, w.weights, n * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->expert_out) ZC_HIP(hipMemcpyAsync(trace->expert_out, w.expert_out, n * H * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->shared) ZC_HIP(hipMemcpyAsync(trace->shared, w.shared, uint64_t(T) * H * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->gate) ZC_HIP(hipMemcpyAsync(trace->gate, w.gate, uint64_t(T) * 4, hipMemcpyDeviceToDevice, s));
+    }
+    return ZC_OK;
+}
+zc_status zc_hip_moe_check(zc_hip_ctx* ctx) {
+    ZC_REQUIRE(ctx, "null context");
+    int32_t flag = 0;
+    ZC_HIP(hipMemcpyAsync(&flag, ctx->moe_status, 4, hipMemcpyDeviceToHost, ctx->stream));
+    ZC_HIP(hipStreamSynchronize(ctx->stream));
+    if (flag) {
+        ZC_HIP(hipMemsetAsync(ctx->moe_status, 0, 4, ctx->stream));
+        return fail(ZC_RUNTIME_ERROR, "invalid router output");
+    }
+    return ZC_OK;
+}
+zc_status zc_hip_rms_glue(zc_hip_ctx* ctx, const float* x, uint32_t tokens, uint32_t hidden, float* out) {
+    ZC_REQUIRE(ctx && x && out && tokens && hidden, "invalid glue buffers");
+    zc::launch_rms_glue(ctx->stream, x, tokens, hidden, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+
+zc_status zc_hip_synth_words(zc_hip_ctx* ctx, uint32_t* dst, uint64_t count, uint64_t seed) {
+    ZC_REQUIRE(ctx && (dst || !count), "null argument");
+    if (count) { zc::launch_synth_words(ctx->stream, dst, count, seed); ZC_LAUNCHED(); }
+    return ZC_OK;
+}
+zc_status zc_hip_synth_scales(zc_hip_ctx* ctx, uint16_t* scales, uint16_t* biases, uint64_t count, uint64_t seed, float lo, float span, float factor) {
+    ZC_REQUIRE(ctx && ((scales && biases) || !count), "null argument");
+    if (count) { zc::launch_synth_scales(ctx->stream, scales, biases, count, seed, lo, span, factor); ZC_LAUNCHED(); }
+    return ZC_OK;
+}
+zc_status zc_hip_synth_normal_f32(zc_hip_ctx* ctx, float* dst, uint64_t count, uint64_t seed, float sigma) {
+    ZC_REQUIRE(ctx && (dst || !count), "null argument");
+    if (count) { zc::launch_synth_normal(ctx->stream, dst, count, seed, sigma, false); ZC_LAUNCHED(); }
+    return ZC_OK;
+}
+zc_status zc_hip_synth_normal_bf16(zc_hip_ctx* ctx, uint16_t* dst, uint64_t count, uint64_t seed, float sigma) {
+    ZC_REQUIRE(ctx && (dst || !count), "null argument");
+    if (count) { zc::launch_synth_normal(ctx->stream, dst, count, seed, sigma, true); ZC_LAUNCHED(); }
+    return ZC_OK;
+}
+zc_status zc_hip_synth_records(zc_hip_ctx* ctx, const zc_moe_config* c, int shared, void* records, uint64_t stride, uint32_t count, uint64_t seed) {
+    if (const zc_status s = validate_config(c)) return s;
+    ZC_REQUIRE(ctx && records && stride >= zc_hip_record_bytes(c, shared) && stride % 4 == 0, "expert record stride is too small");
+    if (!count) return ZC_OK;
+    uint64_t w_off[3], s_off[3], words[3], meta[3]; uint32_t bits[3];
+    for (int p = 0; p < 3; ++p) {
+        zc_linear l; zc_hip_expert_linear(c, shared, records, p, &l);
+        w_off[p] = uint64_t(reinterpret_cast<uintptr_t>(l.weight) - reinterpret_cast<uintptr_t>(records));
+        s_off[p] = uint64_t(reinterpret_cast<uintptr_t>(l.scales) - reinterpret_cast<uintptr_t>(records));
+        words[p] = uint64_t(l.input) * l.output * l.bits / 32; meta[p] = uint64_t(l.input / l.group) * l.output; bits[p] = l.bits;
+    }
+    zc::launch_synth_records(ctx->stream, records, stride, count, w_off, s_off, words, meta, bits, seed);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+}  // extern "C"

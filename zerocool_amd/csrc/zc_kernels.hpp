@@ -1,0 +1,48 @@
+// Host-side launchers of the MoE-path kernels.  Each only enqueues on `s`.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/zc_hip.h"
+
+namespace zc {
+
+struct AffineDesc {
+    zc_linear gate, up;          // up used only when gated
+    bool gated = false;
+    const float* x = nullptr;
+    const int32_t* in_rows = nullptr;
+    const int32_t* out_rows = nullptr;
+    float* out = nullptr;
+    uint32_t tokens = 0;
+    uint32_t float_output = 0;
+};
+void launch_affine(hipStream_t s, const AffineDesc& a);
+
+struct ExpertPhaseDesc {
+    const void* records; uint64_t stride;
+    uint64_t off[6];             // w,s,b of the first matrix, then of the second (gate/up phase)
+    const int32_t *offsets, *selected, *count, *in_rows, *out_rows;
+    const float* x; float* out;
+    uint32_t K, N, group, bits, x_sorted, max_jobs;
+    bool gated;
+};
+void launch_expert_phase(hipStream_t s, const ExpertPhaseDesc& d);
+
+void launch_plain(hipStream_t s, const void* w, uint32_t dtype, const float* x, uint32_t K, uint32_t N,
+                  uint32_t tokens, float* out, bool float_output);
+void launch_router(hipStream_t s, const void* w, const float* x, uint32_t T, uint32_t K, uint32_t E,
+                   const float* offsets, float* out);
+void launch_route(hipStream_t s, const float* logits, uint32_t T, uint32_t E, uint32_t topk, int32_t* ids, float* weights);
+void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets,
+                     int32_t* slots, int32_t* rows, int32_t* selected, int32_t* count, int32_t* status);
+void launch_scatter(hipStream_t s, const float* x, const int32_t* positions, uint32_t n, uint32_t H, float* out);
+void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, const float* shared, const float* gate,
+                    uint32_t T, uint32_t H, uint32_t topk, float* out);
+void launch_rms_glue(hipStream_t s, const float* x, uint32_t T, uint32_t H, float* out);
+void launch_synth_words(hipStream_t s, uint32_t* dst, uint64_t count, uint64_t seed);
+void launch_synth_scales(hipStream_t s, uint16_t* sc, uint16_t* bi, uint64_t count, uint64_t seed, float lo, float span, float factor);
+void launch_synth_normal(hipStream_t s, void* dst, uint64_t count, uint64_t seed, float sigma, bool half);
+void launch_synth_records(hipStream_t s, void* records, uint64_t stride, uint32_t count, const uint64_t* w_off,
+                          const uint64_t* s_off, const uint64_t* words, const uint64_t* meta, const uint32_t* bits, uint64_t seed);
+
+}  // namespace zc

@@ -1,0 +1,232 @@
+"""ctypes face of the C ABI in include/zc_hip.h.  Device memory is owned by the
+context (`Context.alloc`), addressed by plain integers wrapped in `DevBuf`."""
+import ctypes as C
+import os
+import numpy as np
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libzc_hip.so")
+_lib = None
+
+
+class ZcError(RuntimeError):
+    """Raised for any non-zero zc_status; `.status` keeps the code (1 invalid argument,
+    2 runtime error, 3 logic error, 4 out of range, 5 budget exceeded)."""
+
+    def __init__(self, status, text):
+        super().__init__(text)
+        self.status = status
+
+
+class Linear(C.Structure):
+    _fields_ = [("weight", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p),
+                ("input", C.c_uint32), ("output", C.c_uint32), ("group", C.c_uint32), ("dtype", C.c_uint32),
+                ("quantized", C.c_uint32), ("bits", C.c_uint32)]
+
+
+class Config(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("hidden", "experts", "topk", "inter", "group", "bits_gate_up",
+                                          "bits_down", "shared_bits_gate_up", "shared_bits_down")]
+
+
+class Layer(C.Structure):
+    _fields_ = [("router", C.c_void_p), ("router_offsets", C.c_void_p), ("shared_gate", C.c_void_p),
+                ("shared_record", C.c_void_p), ("expert_records", C.c_void_p), ("record_stride", C.c_uint64)]
+
+
+class Trace(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("logits", "ids", "weights", "expert_out", "shared", "gate")]
+
+
+def load_library():
+    """Loads libzc_hip.so; there is no fallback path."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`")
+    lib = C.CDLL(LIB_PATH)
+    lib.zc_hip_last_error.restype = C.c_char_p
+    lib.zc_hip_version.restype = C.c_char_p
+    for name in ("zc_hip_allocated", "zc_hip_peak", "zc_hip_moe_workspace_bytes", "zc_hip_projection_bytes",
+                 "zc_hip_record_bytes"):
+        getattr(lib, name).restype = C.c_uint64
+    lib.zc_hip_stream.restype = C.c_void_p
+    lib.zc_hip_projection_bytes.argtypes = [C.c_uint32] * 4
+    _lib = lib
+    return lib
+
+
+class DevBuf:
+    """A device allocation (or a view into one)."""
+
+    def __init__(self, ctx, ptr, nbytes, owner=None):
+        self.ctx, self.ptr, self.nbytes, self.owner = ctx, ptr, nbytes, owner
+
+    def view(self, offset, nbytes=None):
+        nbytes = self.nbytes - offset if nbytes is None else nbytes
+        assert 0 <= offset and offset + nbytes <= self.nbytes
+        return DevBuf(self.ctx, self.ptr + offset, nbytes, self.owner or self)
+
+    def numpy(self, dtype, count=None):
+        dtype = np.dtype(dtype)
+        count = self.nbytes // dtype.itemsize if count is None else count
+        out = np.empty(count, dtype)
+        self.ctx._call("zc_hip_download", out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr), C.c_uint64(out.nbytes))
+        return out
+
+
+def _ptr(b):
+    if b is None:
+        return C.c_void_p(None)
+    return C.c_void_p(b.ptr if isinstance(b, DevBuf) else int(b))
+
+
+class Context:
+    def __init__(self, device=0, budget=0):
+        self.lib = load_library()
+        self.handle = C.c_void_p()
+        self._check(self.lib.zc_hip_create(C.c_int(device), C.c_uint64(budget), C.byref(self.handle)))
+
+    def close(self):
+        if self.handle:
+            self.lib.zc_hip_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, status):
+        if status:
+            raise ZcError(status, self.lib.zc_hip_last_error().decode())
+
+    def _call(self, name, *args):
+        self._check(getattr(self.lib, name)(self.handle, *args))
+
+    # memory --------------------------------------------------------------
+    def alloc(self, nbytes):
+        p = C.c_void_p()
+        self._call("zc_hip_alloc", C.c_uint64(nbytes), C.byref(p))
+        return DevBuf(self, p.value, nbytes)
+
+    def free(self, buf):
+        self._call("zc_hip_free", C.c_void_p(buf.ptr))
+
+    def zeros(self, nbytes):
+        b = self.alloc(nbytes)
+        self._call("zc_hip_memset", _ptr(b), C.c_int(0), C.c_uint64(nbytes))
+        return b
+
+    def fill(self, buf, byte):
+        self._call("zc_hip_memset", _ptr(buf), C.c_int(byte), C.c_uint64(buf.nbytes))
+
+    def upload(self, array, into=None):
+        a = np.ascontiguousarray(array)
+        b = into or self.alloc(max(a.nbytes, 4))
+        self._call("zc_hip_upload", _ptr(b), a.ctypes.data_as(C.c_void_p), C.c_uint64(a.nbytes))
+        return b
+
+    def finish(self):
+        self._call("zc_hip_finish")
+
+    def submit(self):
+        t = C.c_uint64()
+        self._call("zc_hip_submit", C.byref(t))
+        return t.value
+
+    def wait(self, ticket):
+        self._call("zc_hip_wait", C.c_uint64(ticket))
+
+    @property
+    def allocated(self):
+        return self.lib.zc_hip_allocated(self.handle)
+
+    @property
+    def stream(self):
+        return self.lib.zc_hip_stream(self.handle)
+
+    # operators -----------------------------------------------------------
+    def linear(self, l, x, tokens, float_output=False, out=None):
+        out = out or self.alloc(tokens * l.output * 4)
+        self._call("zc_hip_linear_into", C.byref(l), _ptr(x), C.c_uint32(tokens), _ptr(out), C.c_int(int(float_output)))
+        return out
+
+    def router_logits(self, w, x, tokens, hidden, experts, offsets=None, out=None):
+        out = out or self.alloc(tokens * experts * 4)
+        self._call("zc_hip_router_logits", _ptr(w), _ptr(x), C.c_uint32(tokens), C.c_uint32(hidden), C.c_uint32(experts),
+                   _ptr(offsets), _ptr(out))
+        return out
+
+    def gated_linear(self, gate, up, x, x_rows, tokens, rows=None, out=None):
+        out = out or self.alloc(tokens * gate.output * 4)
+        self._call("zc_hip_gated_linear", C.byref(gate), C.byref(up), _ptr(x), C.c_uint32(x_rows), C.c_uint32(tokens),
+                   _ptr(rows), _ptr(out))
+        return out
+
+    def route(self, logits, tokens, experts, topk=10):
+        ids, w = self.alloc(tokens * topk * 4), self.alloc(tokens * topk * 4)
+        self._call("zc_hip_route", _ptr(logits), C.c_uint32(tokens), C.c_uint32(experts), C.c_uint32(topk), _ptr(ids), _ptr(w))
+        return ids, w
+
+    def build_dispatch(self, ids, tokens, topk, experts):
+        off, slots = self.alloc((experts + 1) * 4), self.zeros(tokens * topk * 4)
+        sel, count, status = self.zeros(experts * 4), self.zeros(4), self.zeros(4)
+        self._call("zc_hip_build_dispatch", _ptr(ids), C.c_uint32(tokens), C.c_uint32(topk), C.c_uint32(experts),
+                   _ptr(off), _ptr(slots), _ptr(sel), _ptr(count), _ptr(status))
+        return off, slots, sel, count, status
+
+    def scatter_experts(self, x, positions, n, hidden, out):
+        self._call("zc_hip_scatter_experts", _ptr(x), _ptr(positions), C.c_uint32(n), C.c_uint32(hidden), _ptr(out))
+
+    def moe_sum(self, experts, weights, shared, gate, tokens, hidden, topk=10, out=None):
+        out = out or self.alloc(tokens * hidden * 4)
+        self._call("zc_hip_moe_sum", _ptr(experts), _ptr(weights), _ptr(shared), _ptr(gate), C.c_uint32(tokens),
+                   C.c_uint32(hidden), C.c_uint32(topk), _ptr(out))
+        return out
+
+    def grouped_experts(self, cfg, records, positions, x, out, scratch):
+        n = len(records)
+        recs = (C.c_void_p * max(n, 1))(*[r.ptr for r in records])
+        pos = (C.c_uint32 * max(len(positions), 1))(*positions)
+        self._call("zc_hip_grouped_experts", C.byref(cfg), recs, pos, C.c_uint32(n), _ptr(x), _ptr(out), _ptr(scratch))
+
+    def expert_linear(self, cfg, record, projection, shared=False):
+        l = Linear()
+        self._check(self.lib.zc_hip_expert_linear(C.byref(cfg), C.c_int(int(shared)), _ptr(record), C.c_int(projection), C.byref(l)))
+        return l
+
+    def record_bytes(self, cfg, shared=False):
+        return self.lib.zc_hip_record_bytes(C.byref(cfg), C.c_int(int(shared)))
+
+    def moe_workspace_bytes(self, cfg, tokens):
+        return self.lib.zc_hip_moe_workspace_bytes(C.byref(cfg), C.c_uint32(tokens))
+
+    def moe_forward(self, cfg, layer, x, tokens, out, workspace, trace=None):
+        self._call("zc_hip_moe_forward", C.byref(cfg), C.byref(layer), _ptr(x), C.c_uint32(tokens), _ptr(out),
+                   _ptr(workspace), C.byref(trace) if trace is not None else None)
+
+    def moe_check(self):
+        self._call("zc_hip_moe_check")
+
+    def rms_glue(self, x, tokens, hidden, out):
+        self._call("zc_hip_rms_glue", _ptr(x), C.c_uint32(tokens), C.c_uint32(hidden), _ptr(out))
+
+    # synthetic tensors ---------------------------------------------------
+    def synth_words(self, dst, count, seed):
+        self._call("zc_hip_synth_words", _ptr(dst), C.c_uint64(count), C.c_uint64(seed))
+
+    def synth_scales(self, scales, biases, count, seed, lo, span, factor):
+        self._call("zc_hip_synth_scales", _ptr(scales), _ptr(biases), C.c_uint64(count), C.c_uint64(seed),
+                   C.c_float(lo), C.c_float(span), C.c_float(factor))
+
+    def synth_normal_f32(self, dst, count, seed, sigma=1.0):
+        self._call("zc_hip_synth_normal_f32", _ptr(dst), C.c_uint64(count), C.c_uint64(seed), C.c_float(sigma))
+
+    def synth_normal_bf16(self, dst, count, seed, sigma=1.0):
+        self._call("zc_hip_synth_normal_bf16", _ptr(dst), C.c_uint64(count), C.c_uint64(seed), C.c_float(sigma))
+
+    def synth_records(self, cfg, records, stride, count, seed, shared=False):
+        self._call("zc_hip_synth_records", C.byref(cfg), C.c_int(int(shared)), _ptr(records), C.c_uint64(stride),
+                   C.c_uint32(count), C.c_uint64(seed))

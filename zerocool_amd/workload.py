@@ -1,0 +1,80 @@
+"""Synthetic MoE layers of the benchmark configurations, generated on the device.
+
+Shapes: S = one layer (hidden 2048, 512 experts, top-10, intermediate 512, group 64);
+F = one layer of the 48-layer stand-in stack (hidden 3072, intermediate 1024).
+Routed records are affine Q4 (codes uniform 0..15, BF16 scale ~U(0.002,0.02), bias -8*scale);
+the mixed artifact keeps gate/up Q4 and makes down + the shared expert affine Q8
+(scale ~U(0.0002,0.002), bias -128*scale)."""
+import ctypes as C
+import math
+import numpy as np
+from . import synth
+from .hip import Config, Layer
+
+BASE_SEED = 0x5EED
+
+
+def config(name):
+    if name == "S":
+        return Config(2048, 512, 10, 512, 64, 4, 4, 4, 4)
+    if name == "S-mixed":
+        return Config(2048, 512, 10, 512, 64, 4, 8, 8, 8)
+    if name == "F":
+        return Config(3072, 512, 10, 1024, 64, 4, 4, 4, 4)
+    if name == "ref":   # the reference's own shape (storage.hpp:26-27)
+        return Config(2560, 512, 10, 640, 64, 4, 4, 4, 4)
+    raise KeyError(name)
+
+
+def tiny_config(hidden=512, experts=32, topk=4, inter=128, group=64, bits=(4, 4, 4, 4)):
+    return Config(hidden, experts, topk, inter, group, *bits)
+
+
+def record_stride(ctx, cfg):
+    return (ctx.record_bytes(cfg) + 255) // 256 * 256
+
+
+class LayerWeights:
+    """Device buffers of one layer plus the zc_moe_layer that points at them."""
+
+    def __init__(self, ctx, cfg, seed, skew=None, records=None):
+        H, E = cfg.hidden, cfg.experts
+        self.ctx, self.cfg, self.seed = ctx, cfg, seed
+        self.stride = record_stride(ctx, cfg)
+        self.router = ctx.alloc(E * H * 2)
+        self.shared_gate = ctx.alloc(H * 2)
+        self.shared_record = ctx.alloc(ctx.record_bytes(cfg, shared=True))
+        self.records = records if records is not None else ctx.alloc(E * self.stride)
+        sigma = 1.0 / math.sqrt(H)
+        ctx.synth_normal_bf16(self.router, E * H, seed * 16 + 1, sigma)
+        ctx.synth_normal_bf16(self.shared_gate, H, seed * 16 + 2, sigma)
+        ctx.synth_records(cfg, self.shared_record, self.shared_record.nbytes, 1, seed * 16 + 3, shared=True)
+        ctx.synth_records(cfg, self.records, self.stride, E, (seed * 16 + 4) * 4096)
+        self.offsets_host = None
+        if skew is not None:
+            kind, value = skew
+            self.offsets_host = (synth.normal_offsets(E, seed * 16 + 5, value) if kind == "normal"
+                                 else synth.zipf_offsets(E, seed * 16 + 5, value))
+        self.offsets = ctx.upload(self.offsets_host) if self.offsets_host is not None else None
+        self.layer = Layer(self.router.ptr, self.offsets.ptr if self.offsets else None, self.shared_gate.ptr,
+                           self.shared_record.ptr, self.records.ptr, self.stride)
+
+    def host(self):
+        """Host copies for the CPU checker: router, shared_gate (uint16), records (uint8)."""
+        return dict(router=self.router.numpy(np.uint16), shared_gate=self.shared_gate.numpy(np.uint16),
+                    shared_record=self.shared_record.numpy(np.uint8), records=self.records.numpy(np.uint8),
+                    offsets=self.offsets_host, stride=self.stride)
+
+
+def hidden_rows(ctx, tokens, hidden, seed):
+    x = ctx.alloc(tokens * hidden * 4)
+    ctx.synth_normal_f32(x, tokens * hidden, seed, 1.0)
+    return x
+
+
+def layer_bytes(cfg, unique_experts, tokens, ctx):
+    """Algorithmic bytes of one layer step: router + shared gate + U routed records +
+    shared record + activations in/out + route ids/weights."""
+    H, E, k = cfg.hidden, cfg.experts, cfg.topk
+    return (2 * H * E + 2 * H + unique_experts * ctx.record_bytes(cfg) + ctx.record_bytes(cfg, shared=True)
+            + tokens * 4 * H + tokens * k * 8)

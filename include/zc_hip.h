@@ -81,6 +81,12 @@ uint64_t zc_hip_peak(const zc_hip_ctx* ctx);
 zc_status zc_hip_submit(zc_hip_ctx* ctx, uint64_t* ticket);
 zc_status zc_hip_wait(zc_hip_ctx* ctx, uint64_t ticket);
 zc_status zc_hip_finish(zc_hip_ctx* ctx);
+/* Metal::configure (metal.hpp:87; KernelConfig::policy, metal.hpp:17-26): which kernels
+ * serve the affine products.  0 = the literal lane kernels for every shape (the
+ * reference's "reference" policy); 1 = the exact-integer matrix-core kernels wherever
+ * the shape allows (wide Q4, group 64), literal otherwise.  Default 1.  Both policies
+ * produce identical bytes; only speed differs. */
+zc_status zc_hip_configure(zc_hip_ctx* ctx, uint32_t affine_policy);
 /* The raw hipStream_t the context enqueues on (for event timing by the caller). */
 void* zc_hip_stream(zc_hip_ctx* ctx);
 

@@ -37,6 +37,7 @@ struct zc_hip_ctx {
     std::vector<hipEvent_t> tickets;   // live tickets: ticket t -> tickets[t - retired - 1]
     uint64_t retired = 0;              // tickets known complete and destroyed
     int32_t* moe_status = nullptr;     // device flag: an id outside [0,E) was seen
+    uint32_t affine_policy = 1;        // 0 literal lane kernels, 1 exact-integer matrix-core kernels where possible
     std::mutex mutex;
 };
 
@@ -114,6 +115,12 @@ zc_status zc_hip_download(zc_hip_ctx* ctx, void* host_dst, const void* src, uint
 zc_status zc_hip_copy(zc_hip_ctx* ctx, void* dst, const void* src, uint64_t bytes) {
     ZC_REQUIRE(ctx && ((dst && src) || !bytes), "null argument");
     if (bytes) ZC_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return ZC_OK;
+}
+zc_status zc_hip_configure(zc_hip_ctx* ctx, uint32_t affine_policy) {
+    ZC_REQUIRE(ctx, "null context");
+    ZC_REQUIRE(affine_policy <= 1, "unknown kernel policy");
+    ctx->affine_policy = affine_policy;
     return ZC_OK;
 }
 uint64_t zc_hip_allocated(const zc_hip_ctx* ctx) { return ctx ? ctx->allocated : 0; }
@@ -212,7 +219,8 @@ zc_status zc_hip_linear_into(zc_hip_ctx* ctx, const zc_linear* l, const float* x
                "invalid or overlapping linear output");
     if (l->quantized) {
         zc::AffineDesc a; a.gate = *l; a.x = x; a.out = out; a.tokens = tokens; a.float_output = float_output ? 1 : 0;
-        zc::launch_affine(ctx->stream, a);
+        if (ctx->affine_policy == 1 && zc::xint_supported(*l)) zc::launch_affine_xint(ctx->stream, a);
+        else zc::launch_affine(ctx->stream, a);
     } else {
         ZC_REQUIRE(l->dtype <= 1, "unsupported plain matrix dtype");
         zc::launch_plain(ctx->stream, l->weight, l->dtype, x, l->input, l->output, tokens, out, float_output != 0);
@@ -248,7 +256,8 @@ zc_status zc_hip_gated_linear(zc_hip_ctx* ctx, const zc_linear* gate, const zc_l
         for (int32_t r : host) ZC_REQUIRE(r >= 0 && uint32_t(r) < x_rows, "fused gate/up row outside input");
     }
     zc::AffineDesc a; a.gate = *gate; a.up = *up; a.gated = true; a.x = x; a.in_rows = rows; a.out = out; a.tokens = tokens;
-    zc::launch_affine(ctx->stream, a);
+    if (ctx->affine_policy == 1 && zc::xint_supported(*gate) && zc::xint_supported(*up)) zc::launch_affine_xint(ctx->stream, a);
+    else zc::launch_affine(ctx->stream, a);
     ZC_LAUNCHED();
     return ZC_OK;
 }

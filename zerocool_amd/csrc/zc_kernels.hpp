@@ -16,7 +16,9 @@ struct AffineDesc {
     uint32_t tokens = 0;
     uint32_t float_output = 0;
 };
-void launch_affine(hipStream_t s, const AffineDesc& a);
+void launch_affine(hipStream_t s, const AffineDesc& a);          // literal lane arithmetic, any shape
+bool xint_supported(const zc_linear& l);                          // wide affine Q4, group 64, 16-byte aligned
+void launch_affine_xint(hipStream_t s, const AffineDesc& a);     // exact-integer matrix-core form
 
 struct ExpertPhaseDesc {
     const void* records; uint64_t stride;

@@ -128,6 +128,10 @@ class Context:
         self._call("zc_hip_upload", _ptr(b), a.ctypes.data_as(C.c_void_p), C.c_uint64(a.nbytes))
         return b
 
+    def configure(self, affine_policy):
+        """0: literal lane kernels everywhere; 1 (default): exact-integer matrix-core kernels where the shape allows."""
+        self._call("zc_hip_configure", C.c_uint32(affine_policy))
+
     def finish(self):
         self._call("zc_hip_finish")
 

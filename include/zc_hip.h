@@ -146,9 +146,29 @@ zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc
  * Clears the flag. */
 zc_status zc_hip_moe_check(zc_hip_ctx* ctx);
 
-/* Inter-layer glue of the stacked-decode workload (not reference arithmetic):
- * y = bf(x * 1/sqrt(mean(x^2)+1e-6)) per row. */
-zc_status zc_hip_rms_glue(zc_hip_ctx* ctx, const float* x, uint32_t tokens, uint32_t hidden, float* out);
+/* Stacked decode: n_layers MoE layers (Model::moe, model.cpp:431-557, called once per
+ * layer by Model::forward_impl, model.cpp:637-672) chained for a few tokens.  The trunk
+ * between the reference's MoE layers (attention / GDN / hyper-connections) is outside
+ * this path; the stack stands in for it with a glue that keeps activations bounded and
+ * BF16-valued: x_next = bf(y * (1 / max|y|)) per token (zc_hip_stack_glue).
+ * Up to 8 tokens run as ONE persistent kernel launch for the whole stack (routing,
+ * dispatch and combine stay on the device, no host synchronisation between layers);
+ * larger batches run layer by layer through zc_hip_moe_forward.  Both give identical bytes.
+ * out: [tokens][hidden], the last layer's output.  flags bit 0: force the layer-by-layer path. */
+typedef struct zc_hip_stack zc_hip_stack;
+typedef struct {       /* optional device buffers, any may be NULL */
+    int32_t* ids;      /* [n_layers][tokens][topk] */
+    float* weights;    /* [n_layers][tokens][topk] */
+    float* outputs;    /* [n_layers][tokens][hidden] layer outputs before the glue */
+} zc_stack_trace;
+zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
+                              uint32_t n_layers, uint32_t max_tokens, zc_hip_stack** out);
+zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* stack);
+zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* stack, const float* x, uint32_t tokens,
+                              float* out, const zc_stack_trace* trace, uint32_t flags);
+/* 1 if zc_hip_stack_decode would take the persistent single-launch path for `tokens`. */
+int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* stack, uint32_t tokens);
+zc_status zc_hip_stack_glue(zc_hip_ctx* ctx, const float* y, uint32_t tokens, uint32_t hidden, float* x_next);
 
 /* Counter-based synthetic tensors: element i depends only on (seed, i).
  * kind 0: uint32 words of uniform bits (Q4/Q8 codes), count = words

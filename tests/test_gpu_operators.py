@@ -260,9 +260,12 @@ def test_scatter_rows(ctx):  # qwen.metal:800-803
     assert same_bytes(got, want)
 
 
-def test_rms_glue_is_deterministic_and_normalised(ctx):
-    x = synth.normal(3 * 3072, 9, 5.0)
-    out = ctx.alloc(x.nbytes); ctx.rms_glue(ctx.upload(x), 3, 3072, out)
+def test_stack_glue_is_max_normalised(ctx):
+    y = synth.normal(3 * 3072, 9, 5.0).reshape(3, 3072)
+    y[1, 7] = np.nan
+    out = ctx.alloc(y.nbytes); ctx.stack_glue(ctx.upload(y), 3, 3072, out)
     got = out.numpy(f32).reshape(3, 3072)
-    assert np.allclose(np.sqrt((got.astype(np.float64) ** 2).mean(1)), 1, atol=5e-3)
-    assert ((got.view(np.uint32) & 0xffff) == 0).all()
+    m = np.nanmax(np.abs(y), axis=1, keepdims=True).astype(f32)
+    want = oracle.bf(y * (f32(1) / m))
+    assert got.tobytes() == want.tobytes()
+    assert np.nanmax(np.abs(got)) == 1.0

@@ -1,0 +1,108 @@
+"""Stacked decode (BASELINE config 5 at reduced size): the persistent single-launch kernel,
+the layer-by-layer path and the CPU oracle chained through the same glue must agree byte
+for byte on routing ids, softmax weights and every layer's output."""
+import numpy as np
+import pytest
+import oracle
+import zerocool_amd as z
+from zerocool_amd import workload
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = z.Context(0)
+    yield c
+    c.close()
+
+
+def oracle_cfg(cfg):
+    return oracle.Config(*[getattr(cfg, n) for n, _ in z.Config._fields_])
+
+
+def glue(y):
+    """The stack's stand-in glue: x_next = bf(y * (1 / max|y|)) per token."""
+    m = np.nanmax(np.abs(y), axis=1, keepdims=True).astype(f32)
+    inv = np.where((m > 0) & np.isfinite(m), f32(1) / m, f32(1)).astype(f32)
+    return oracle.bf(y * inv)
+
+
+def oracle_stack(cfg, layers, x, T):
+    ocfg = oracle_cfg(cfg)
+    ids, weights, outs = [], [], []
+    cur = x.reshape(T, cfg.hidden)
+    for h in layers:
+        y, tr = oracle.moe_layer(ocfg, h["router"], h["shared_gate"], h["shared_record"], h["records"], h["stride"], cur, T,
+                                 router_offsets=h["offsets"], threads=8, trace=True)
+        ids.append(tr["ids"]); weights.append(tr["weights"]); outs.append(y)
+        cur = glue(y)
+    return np.stack(ids), np.stack(weights), np.stack(outs)
+
+
+def run_stack(ctx, cfg, stack, x_dev, T, L, layered):
+    n = T * cfg.topk
+    ids, w, outs = ctx.alloc(L * n * 4), ctx.alloc(L * n * 4), ctx.alloc(L * T * cfg.hidden * 4)
+    out = ctx.alloc(T * cfg.hidden * 4)
+    ctx.stack_decode(stack, x_dev, T, out, z.StackTrace(ids.ptr, w.ptr, outs.ptr), layered=layered)
+    ctx.moe_check()
+    r = (ids.numpy(np.int32).reshape(L, T, cfg.topk), w.numpy(f32).reshape(L, T, cfg.topk),
+         outs.numpy(f32).reshape(L, T, cfg.hidden), out.numpy(f32).reshape(T, cfg.hidden))
+    for b in (ids, w, outs, out):
+        ctx.free(b)
+    return r
+
+
+def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1)):
+    layers = [workload.LayerWeights(ctx, cfg, seed + l, skew) for l in range(L)]
+    hosts = [l.host() for l in layers]
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], max(tokens))
+    for T in tokens:
+        x_dev = workload.hidden_rows(ctx, T, cfg.hidden, seed * 131 + T)
+        x = x_dev.numpy(f32)
+        want = oracle_stack(cfg, hosts, x, T)
+        assert ctx.stack_is_persistent(stack, T) == (T <= 8)
+        for layered in (True, False):
+            got = run_stack(ctx, cfg, stack, x_dev, T, L, layered)
+            name = "layered" if layered else "persistent"
+            assert got[0].tobytes() == want[0].tobytes(), f"{name}: routing ids differ (T={T})"
+            assert got[1].tobytes() == want[1].tobytes(), f"{name}: softmax weights differ (T={T})"
+            assert got[2].tobytes() == want[2].tobytes(), f"{name}: layer outputs differ (T={T})"
+            assert got[3].tobytes() == want[2][-1].tobytes()
+            rel = float(np.max(np.abs(got[3] - want[2][-1])) / np.max(np.abs(want[2][-1])))
+            assert rel <= 2e-3
+        ctx.free(x_dev)
+    ctx.stack_destroy(stack)
+    for l in layers:
+        for b in (l.router, l.shared_gate, l.shared_record, l.records):
+            ctx.free(b)
+
+
+def test_tiny_stack(ctx):
+    check_stack(ctx, workload.tiny_config(hidden=512, experts=32, topk=4, inter=512), 3, [1, 2, 3, 5, 8, 11])
+
+
+def test_small_stack_many_experts(ctx):
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=128, topk=10, inter=512), 4, [1, 8])
+
+
+def test_stand_in_stack_shape(ctx):  # hidden 3072 / intermediate 1024, two layers of the 48
+    check_stack(ctx, workload.config("F"), 2, [1, 8])
+
+
+def test_stack_reports_invalid_router_output(ctx):
+    cfg = workload.tiny_config(hidden=512, experts=32, topk=4, inter=512)
+    layers = [workload.LayerWeights(ctx, cfg, 77 + l, None) for l in range(2)]
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], 2)
+    bad = ctx.upload(np.full(2 * cfg.hidden, np.nan, f32)); out = ctx.alloc(2 * cfg.hidden * 4)
+    ctx.stack_decode(stack, bad, 2, out)
+    with pytest.raises(z.ZcError) as err:
+        ctx.moe_check()
+    assert "invalid router output" in str(err.value)
+    notbf = ctx.upload(np.full(2 * cfg.hidden, 1.0000001, f32))
+    ctx.stack_decode(stack, notbf, 2, out)
+    with pytest.raises(z.ZcError) as err:
+        ctx.moe_check()
+    assert "BF16" in str(err.value)
+    ctx.stack_destroy(stack)

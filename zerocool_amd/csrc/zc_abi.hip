@@ -410,13 +410,168 @@ zc_status zc_hip_moe_check(zc_hip_ctx* ctx) {
     ZC_HIP(hipStreamSynchronize(ctx->stream));
     if (flag) {
         ZC_HIP(hipMemsetAsync(ctx->moe_status, 0, 4, ctx->stream));
+        if (flag & 2) return fail(ZC_RUNTIME_ERROR, "HIP execution: the persistent decode kernel could not synchronise its workgroups");
+        if (flag & 4) return fail(ZC_INVALID_ARGUMENT, "stacked decode input is not BF16-valued");
         return fail(ZC_RUNTIME_ERROR, "invalid router output");
     }
     return ZC_OK;
 }
-zc_status zc_hip_rms_glue(zc_hip_ctx* ctx, const float* x, uint32_t tokens, uint32_t hidden, float* out) {
-    ZC_REQUIRE(ctx && x && out && tokens && hidden, "invalid glue buffers");
-    zc::launch_rms_glue(ctx->stream, x, tokens, hidden, out);
+zc_status zc_hip_stack_glue(zc_hip_ctx* ctx, const float* y, uint32_t tokens, uint32_t hidden, float* x_next) {
+    ZC_REQUIRE(ctx && y && x_next && tokens && hidden, "invalid glue buffers");
+    zc::launch_stack_glue(ctx->stream, y, tokens, hidden, x_next);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+}  // extern "C"
+
+struct zc_hip_stack {
+    zc_moe_config cfg{};
+    std::vector<zc_moe_layer> layers;
+    uint32_t max_tokens = 0;
+    // persistent path
+    zc::DecodeLayer* dev_layers = nullptr;
+    uint8_t* arena = nullptr; uint64_t arena_bytes = 0;
+    float *logits = nullptr, *gate = nullptr, *shared_act = nullptr, *act = nullptr, *layer_out = nullptr;
+    uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
+    uint32_t epoch = 1u << 12;
+    int cus = 0; uint32_t lds_limit = 0;
+    bool persistent_ok = false;
+    // layered path
+    void* workspace = nullptr; float *xa = nullptr, *xb = nullptr;
+};
+
+namespace {
+bool persistent_shape(const zc_moe_config& c) {
+    return c.bits_gate_up == 4 && c.bits_down == 4 && c.shared_bits_gate_up == 4 && c.shared_bits_down == 4 && c.group == 64 &&
+           c.hidden % 512 == 0 && c.inter % 512 == 0 && c.experts <= 1024 && c.topk <= 64;
+}
+uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : tokens <= 2 ? 2 : tokens <= 4 ? 4 : 8; }
+}  // namespace
+
+extern "C" {
+zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* host_layers, uint32_t n_layers,
+                              uint32_t max_tokens, zc_hip_stack** out) {
+    if (const zc_status s = validate_config(c)) return s;
+    ZC_REQUIRE(ctx && host_layers && n_layers && max_tokens && max_tokens <= 8192 && out, "invalid stack geometry");
+    for (uint32_t l = 0; l < n_layers; ++l) {
+        const zc_moe_layer& y = host_layers[l];
+        ZC_REQUIRE(y.router && y.shared_gate && y.shared_record && y.expert_records, "missing MoE layer weights");
+        ZC_REQUIRE(y.record_stride >= zc_hip_record_bytes(c, 0) && y.record_stride % 16 == 0, "expert record stride is too small");
+        ZC_REQUIRE(reinterpret_cast<uintptr_t>(y.router) % 16 == 0 && reinterpret_cast<uintptr_t>(y.expert_records) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(y.shared_record) % 16 == 0, "MoE layer operands are misaligned");
+    }
+    auto* st = new zc_hip_stack;
+    st->cfg = *c; st->layers.assign(host_layers, host_layers + n_layers); st->max_tokens = max_tokens;
+    auto cleanup = [&](zc_status code) { zc_hip_stack_destroy(ctx, st); return code; };
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, ctx->device) != hipSuccess) return cleanup(fail(ZC_RUNTIME_ERROR, "HIP execution: cannot query device"));
+    st->cus = prop.multiProcessorCount;
+    st->lds_limit = uint32_t(prop.sharedMemPerBlock) - 1024;
+    const uint32_t T = max_tokens, H = c->hidden, E = c->experts, k = c->topk, I = c->inter;
+    // layered path buffers
+    void* p = nullptr;
+    if (zc_hip_alloc(ctx, zc_hip_moe_workspace_bytes(c, T), &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+    st->workspace = p;
+    if (zc_hip_alloc(ctx, uint64_t(T) * H * 4, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+    st->xa = static_cast<float*>(p);
+    if (zc_hip_alloc(ctx, uint64_t(T) * H * 4, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+    st->xb = static_cast<float*>(p);
+    // persistent path arena
+    st->persistent_ok = persistent_shape(*c);
+    if (st->persistent_ok) {
+        const uint32_t Tp = T < 8 ? T : 8;
+        uint64_t at = 0;
+        auto take = [&](uint64_t bytes) { const uint64_t o = at; at += align_up(bytes, 256); return o; };
+        const uint64_t o_layers = take(sizeof(zc::DecodeLayer) * n_layers), o_logits = take(uint64_t(Tp) * E * 4), o_gate = take(Tp * 4),
+                       o_sact = take(uint64_t(Tp) * I * 4), o_act = take(uint64_t(Tp) * k * I * 4), o_lout = take(uint64_t(Tp) * H * 4),
+                       o_max = take(uint64_t(n_layers) * Tp * 4), o_sync = take(zc::kDecodeSyncBytes);
+        if (zc_hip_alloc(ctx, at, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+        st->arena = static_cast<uint8_t*>(p); st->arena_bytes = at;
+        st->dev_layers = reinterpret_cast<zc::DecodeLayer*>(st->arena + o_layers);
+        st->logits = reinterpret_cast<float*>(st->arena + o_logits); st->gate = reinterpret_cast<float*>(st->arena + o_gate);
+        st->shared_act = reinterpret_cast<float*>(st->arena + o_sact); st->act = reinterpret_cast<float*>(st->arena + o_act);
+        st->layer_out = reinterpret_cast<float*>(st->arena + o_lout); st->maxabs = reinterpret_cast<uint32_t*>(st->arena + o_max);
+        st->sync = reinterpret_cast<uint32_t*>(st->arena + o_sync);
+        std::vector<zc::DecodeLayer> host(n_layers);
+        for (uint32_t l = 0; l < n_layers; ++l) {
+            const zc_moe_layer& y = host_layers[l];
+            host[l] = zc::DecodeLayer{static_cast<const uint16_t*>(y.router), y.router_offsets, static_cast<const uint16_t*>(y.shared_gate),
+                                      static_cast<const uint8_t*>(y.shared_record), static_cast<const uint8_t*>(y.expert_records), y.record_stride};
+        }
+        if (hipMemsetAsync(st->arena, 0, at, ctx->stream) != hipSuccess ||
+            hipMemcpyAsync(st->dev_layers, host.data(), sizeof(zc::DecodeLayer) * n_layers, hipMemcpyHostToDevice, ctx->stream) != hipSuccess ||
+            hipStreamSynchronize(ctx->stream) != hipSuccess)
+            return cleanup(fail(ZC_RUNTIME_ERROR, "HIP execution: cannot initialise the decode stack"));
+    }
+    *out = st;
+    return ZC_OK;
+}
+zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* st) {
+    if (!st) return ZC_OK;
+    ZC_REQUIRE(ctx, "null context");
+    for (void* p : {static_cast<void*>(st->workspace), static_cast<void*>(st->xa), static_cast<void*>(st->xb), static_cast<void*>(st->arena)})
+        if (p) zc_hip_free(ctx, p);
+    delete st;
+    return ZC_OK;
+}
+static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, zc::DecodeLdsPlan* plan, uint32_t* nt) {
+    if (!st->persistent_ok || tokens > 8 || tokens > st->max_tokens) return false;
+    const zc_moe_config& c = st->cfg;
+    *nt = token_tile(tokens);
+    if (tokens * c.topk > 512) return false;
+    *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, *nt, st->lds_limit);
+    if (plan->total > st->lds_limit || plan->slots_per_batch == 0) return false;
+    int per_cu = 0;
+    if (zc::decode_stack_occupancy(*nt, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+    (void)ctx;
+    return per_cu >= 1;
+}
+int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
+    if (!ctx || !st) return 0;
+    zc::DecodeLdsPlan plan; uint32_t nt;
+    return persistent_plan(ctx, st, tokens, &plan, &nt) ? 1 : 0;
+}
+zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
+                              const zc_stack_trace* trace, uint32_t flags) {
+    ZC_REQUIRE(ctx && st && x && out && tokens && tokens <= st->max_tokens, "invalid stack decode buffers");
+    ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && x != out, "invalid or overlapping linear output");
+    const zc_moe_config& c = st->cfg;
+    const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
+    zc::DecodeLdsPlan plan; uint32_t nt = 0;
+    if (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &nt)) {
+        zc::DecodeParams p{};
+        p.H = H; p.E = c.experts; p.topk = k; p.I = c.inter; p.T = tokens; p.L = L;
+        for (int shared = 0; shared < 2; ++shared)
+            for (int pr = 0; pr < 3; ++pr) {
+                zc_linear l; zc_hip_expert_linear(&c, shared, reinterpret_cast<const void*>(uintptr_t(4096)), pr, &l);
+                uint64_t* o = shared ? p.so : p.ro;
+                o[pr * 3 + 0] = reinterpret_cast<uintptr_t>(l.weight) - 4096; o[pr * 3 + 1] = reinterpret_cast<uintptr_t>(l.scales) - 4096;
+                o[pr * 3 + 2] = reinterpret_cast<uintptr_t>(l.biases) - 4096;
+            }
+        p.layers = st->dev_layers; p.x_in = x; p.out = out;
+        p.logits = st->logits; p.gate = st->gate; p.shared_act = st->shared_act; p.act = st->act; p.layer_out = st->layer_out;
+        p.maxabs = st->maxabs;
+        p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
+        if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
+        p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = 1u << 22;
+        st->epoch += 3 * L + 16;   // wraps modulo 2^32; the barrier compares epochs as signed differences
+        const uint32_t workgroups = uint32_t(st->cus);
+        ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
+        return ZC_OK;
+    }
+    // layer by layer: y = moe(x); x_next = glue(y)
+    const float* cur = x;
+    for (uint32_t l = 0; l < L; ++l) {
+        float* y = l + 1 == L ? out : st->xa;
+        zc_moe_trace tr{};
+        if (trace) {
+            tr.ids = trace->ids ? trace->ids + uint64_t(l) * tokens * k : nullptr;
+            tr.weights = trace->weights ? trace->weights + uint64_t(l) * tokens * k : nullptr;
+        }
+        if (const zc_status s = zc_hip_moe_forward(ctx, &c, &st->layers[l], cur, tokens, y, st->workspace, trace ? &tr : nullptr)) return s;
+        if (trace && trace->outputs) ZC_HIP(hipMemcpyAsync(trace->outputs + uint64_t(l) * tokens * H, y, uint64_t(tokens) * H * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        if (l + 1 < L) { zc::launch_stack_glue(ctx->stream, y, tokens, H, st->xb); cur = st->xb; }
+    }
     ZC_LAUNCHED();
     return ZC_OK;
 }

@@ -1,0 +1,438 @@
+// Persistent decode kernel: a whole stack of MoE layers for a few tokens in ONE launch.
+//
+// One workgroup per compute unit stays resident for all layers.  A layer is three
+// phases separated by grid barriers:
+//   R  router logits (16-split chains), shared expert gate/up, shared-expert gate dot
+//   G  every workgroup routes (top-k + softmax) for itself, then the routed gate/up tiles
+//   D  routed + shared down tiles; a workgroup owns 16 output rows for ALL experts, so
+//      the weighted combine (moe_sum) runs inside it without another exchange
+// Arithmetic is the exact-integer matrix-core form (zc_xint.hpp) and the literal router /
+// route / combine expressions, so every value equals the operator kernels bit for bit.
+//
+// Cross-workgroup data (logits, activations, layer outputs) is written and read ONLY with
+// agent-scope relaxed atomics, which write through to / read from device-coherent
+// memory; barriers then need no cache write-back or invalidate, only wait counters.
+// Weights are read with ordinary cached loads: nothing writes them.
+//
+// Between layers the stacked-decode workload applies a stand-in glue (not reference
+// arithmetic): x_next = bf(y * (1 / max|y|)) per token, order independent.
+#include "zc_kernels.hpp"
+#include "zc_xint.hpp"
+
+namespace zc {
+
+#define ZC_LD(p) __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define ZC_ST(p, v) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+__device__ __forceinline__ void st_f32(float* p, float v) { ZC_ST(reinterpret_cast<uint32_t*>(p), __float_as_uint(v)); }
+__device__ __forceinline__ void st_i32(int32_t* p, int32_t v) { ZC_ST(reinterpret_cast<uint32_t*>(p), uint32_t(v)); }
+
+constexpr uint32_t kDecodeThreads = 512, kDecodeWaves = 8;
+constexpr uint32_t kFlagStride = 32, kReleaseBase = 32 * 1024, kReleaseStride = 64, kAbortWord = kReleaseBase + 8 * kReleaseStride;
+
+struct Barrier {
+    uint32_t* mem; uint32_t epoch, spin_limit; int32_t* status; uint32_t token;   // token: this launch's first epoch
+    // Flags + collector: every workgroup stores its epoch; workgroup 0 polls all flags
+    // (one per thread) and then stores eight release words.  No fences: the data that
+    // crosses is written with write-through atomics and each wave has drained its own
+    // stores (workgroup-scope release) before the flag is stored.
+    __device__ __forceinline__ void wait() {
+        ++epoch;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (blockIdx.x == 0) {
+            for (uint32_t w = threadIdx.x; w < gridDim.x; w += blockDim.x)
+                if (w) spin(mem + kFlagStride * w);
+            __syncthreads();
+            if (threadIdx.x < 8) ZC_ST(mem + kReleaseBase + kReleaseStride * threadIdx.x, epoch);
+        } else if (threadIdx.x == 0) {
+            ZC_ST(mem + kFlagStride * blockIdx.x, epoch);
+            spin(mem + kReleaseBase + kReleaseStride * (blockIdx.x & 7u));
+        }
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+    // Bounded: a grid that is not fully resident must not hang the GPU.  Epochs only grow,
+    // so "reached" is a signed comparison that survives wrap-around.
+    __device__ __forceinline__ void spin(uint32_t* word) {
+        for (uint32_t i = 0; int32_t(ZC_LD(word) - epoch) < 0; ++i) {
+            if ((i & 255u) == 255u && ZC_LD(mem + kAbortWord) == token) return;   // someone gave up in this launch
+            if (i >= spin_limit) { ZC_ST(mem + kAbortWord, token); atomicOr(status, 2); return; }
+        }
+    }
+};
+
+template <int NT>
+__device__ __forceinline__ void route_token(const float* logits, uint32_t E, uint32_t topk, uint32_t lane,
+                                            int32_t* ids, float* weights) {
+    constexpr int PER = 16;
+    const float ninf = __uint_as_float(0xff800000u);
+    float cand[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const uint32_t e = lane + 64u * i;
+        const float c = e < E ? load_shared_f32(logits + e) : ninf;
+        cand[i] = c > ninf ? c : ninf;
+    }
+    float score = ninf, top = ninf;   // lane j keeps score j
+    for (uint32_t j = 0; j < topk; ++j) {
+        float best = ninf; uint32_t index = 0x7fffffffu;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) if (cand[i] > best) { best = cand[i]; index = lane + 64u * i; }
+        float m = best;
+#pragma unroll
+        for (int o = 32; o; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+        uint32_t winner = (best == m && best > ninf) ? index : 0x7fffffffu;
+#pragma unroll
+        for (int o = 32; o; o >>= 1) winner = min(winner, uint32_t(__shfl_xor(int(winner), o)));
+        const bool found = winner < E;
+        // the owner's candidate keeps the original bits (signed zero included)
+        float value = ninf;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) if (lane + 64u * i == winner) { value = cand[i]; cand[i] = ninf; }
+        value = __shfl(value, found ? (winner & 63u) : 0);
+        if (!found) value = ninf;
+        if (lane == j) score = value;
+        if (j == 0) top = value;
+        if (lane == 0) ids[j] = found ? int32_t(winner) : -1;
+    }
+    // softmax over the selected: reference lane l sums values 4l..4l+3 (qwen.metal:758-764)
+    const float v = lane < topk ? exp32(score - top) : 0.0f;
+    float s4 = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float other = __shfl(v, (4 * lane + i) & 63u);
+        s4 += (4 * lane + i < 64) ? other : 0.0f;
+    }
+    const float inverse = 1.0f / __shfl(lane_sum32(s4), 0);
+    if (lane < topk) weights[lane] = v * inverse;
+}
+
+template <int NT>
+__global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wg = blockIdx.x, nwg = gridDim.x;
+    const uint32_t H = p.H, E = p.E, I = p.I, k = p.topk, T = p.T, n = T * k;
+    const uint32_t col = lane & 15u, G = lane >> 4;
+    int32_t* ids = reinterpret_cast<int32_t*>(lds + lp.ids);
+    float* weights = reinterpret_cast<float*>(lds + lp.weights);
+    float* gatev = reinterpret_cast<float*>(lds + lp.gatev);
+    int32_t* head = reinterpret_cast<int32_t*>(lds + lp.head);
+    int32_t* next = reinterpret_cast<int32_t*>(lds + lp.next);
+    int32_t* experts = reinterpret_cast<int32_t*>(lds + lp.experts);
+    int32_t* misc = reinterpret_cast<int32_t*>(lds + lp.misc);   // [0] U, [1..8] wave counts
+    const XintLayout LH{H}, LI{I};
+    Barrier bar{p.sync, p.epoch, p.spin_limit, p.status, p.epoch};
+
+    if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
+
+    for (uint32_t layer = 0; layer < p.L; ++layer) {
+        const DecodeLayer L = p.layers[layer];
+        // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
+        __syncthreads();
+        for (uint32_t t = 0; t < T; ++t) {
+            uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh) + t * H;
+            float inv = 1.0f;
+            if (layer) {
+                const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + t));
+                if (m > 0.0f && m < __uint_as_float(0x7f800000u)) inv = 1.0f / m;
+            }
+            int bad = 0;
+            for (uint32_t i = tid; i < H; i += blockDim.x) {
+                float v = load_shared_f32((layer ? p.layer_out : p.x_in) + uint64_t(t) * H + i);
+                if (layer) v = bf(v * inv);
+                const uint32_t u = __float_as_uint(v);
+                bad |= (u & 0xffffu) != 0;
+                xh[i] = uint16_t(u >> 16);
+            }
+            if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
+        }
+        __syncthreads();
+        for (uint32_t t = 0; t < T; ++t)
+            xint_prepare(LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.xh) + t * H}, LH, lds + lp.img_rg + t * LH.bytes());
+        __syncthreads();
+        {
+            const uint32_t router_units = (E + 3) / 4, shared_units = I / 8, gate_units = (T + 1) / 2;
+            const uint32_t units = router_units + shared_units + gate_units;
+            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
+                if (u < router_units) {
+                    // four experts x sixteen K partitions; k-ascending fused chain per partition
+                    const uint32_t e = u * 4 + lane / 16, split = lane % 16, P = H / 16;
+                    float c[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) c[t] = 0;
+                    if (e < E) {
+                        const uint16_t* wr = L.router + uint64_t(e) * H + split * P;
+                        for (uint32_t i = 0; i < P; i += 8) {
+                            const uint4 wv = *reinterpret_cast<const uint4*>(wr + i);
+                            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+                            for (int t = 0; t < NT; ++t) {
+                                if (t >= int(T)) break;
+                                const uint4 xv = *reinterpret_cast<const uint4*>(lds + lp.xh + (uint64_t(t) * H + split * P + i) * 2);
+                                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) {
+                                    c[t] = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c[t]);
+                                    c[t] = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c[t]);
+                                }
+                            }
+                        }
+                    }
+                    const uint32_t base = lane & ~15u;
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        if (t >= int(T)) break;
+                        float sum = 0;
+                        for (uint32_t sidx = 0; sidx < 16; ++sidx) sum += __shfl(c[t], base + sidx);
+                        if (split == 0 && e < E) st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + L.offsets[e] : sum);
+                    }
+                } else if (u < router_units + shared_units) {
+                    const uint32_t tile = u - router_units, row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                    const uint8_t* rec = L.shared_record;
+                    const uint4* codes = reinterpret_cast<const uint4*>(rec + p.so[pr] + uint64_t(row) * (H / 2)) + G;
+                    const uint16_t* sr = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64) + (G >> 1);
+                    const uint16_t* br = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64) + (G >> 1);
+                    const uint8_t* img[NT]; LdsBf16 src[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const uint32_t tt = t < int(T) ? t : 0;
+                        img[t] = lds + lp.img_rg + tt * LH.bytes();
+                        src[t] = LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.xh) + tt * H};
+                    }
+                    XintTile<NT> tile_state; tile_state.clear();
+#pragma unroll 4
+                    for (uint32_t dg = 0; dg < H / 128; ++dg)
+                        tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), img, LH, src, lane, int(T));
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        if (t >= int(T)) break;
+                        const float v = tile_state.finish(t);
+                        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                        if (G == 0 && col < 8) st_f32(p.shared_act + uint64_t(t) * I + row, swiglu_bf(v, up));
+                    }
+                } else {
+                    // shared_expert_gate: reference lane chain k = lane + 32 j (qwen.metal:499-506); two tokens per wave
+                    const uint32_t t = (u - router_units - shared_units) * 2 + (lane >> 5), l32 = lane & 31u;
+                    float sum = 0;
+                    if (t < T) {
+                        const uint16_t* xh = reinterpret_cast<const uint16_t*>(lds + lp.xh) + t * H;
+                        for (uint32_t kk = l32; kk < H; kk += 32) sum += b16(xh[kk]) * b16(L.shared_gate[kk]);
+                    }
+                    sum = lane_sum32(sum);
+                    if (t < T && l32 == 0) st_f32(p.gate + t, bf(sum));
+                }
+            }
+        }
+        bar.wait();
+        // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
+        for (uint32_t t = wave; t < T; t += kDecodeWaves)
+            route_token<NT>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k);
+        if (tid < T) gatev[tid] = load_shared_f32(p.gate + tid);
+        for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
+        __syncthreads();
+        if (tid < n) {
+            const int32_t e = ids[tid];
+            if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); next[tid] = -1; }
+            else next[tid] = atomicExch(&head[e], int32_t(tid));
+            if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * n + tid, e); st_f32(p.weights_trace + uint64_t(layer) * n + tid, weights[tid]); }
+        }
+        __syncthreads();
+        {   // compact the experts that own at least one slot (any order: slots are independent)
+            uint32_t base = 0;
+            for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+                const uint32_t e = e0 + tid;
+                const bool used = e < E && head[e] >= 0;
+                const uint64_t m = __ballot(used);
+                if (lane == 0) misc[1 + wave] = __popcll(m);
+                __syncthreads();
+                uint32_t before = base;
+                for (uint32_t w = 0; w < wave; ++w) before += misc[1 + w];
+                if (used) experts[before + __popcll(m & ((1ull << lane) - 1))] = int32_t(e);
+                for (uint32_t w = 0; w < kDecodeWaves; ++w) base += misc[1 + w];
+                __syncthreads();
+            }
+            if (tid == 0) misc[0] = int32_t(base);
+        }
+        __syncthreads();
+        const uint32_t U = uint32_t(misc[0]);
+        {
+            const uint32_t tiles = I / 8, units = U * tiles;
+            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
+                const uint32_t e = uint32_t(experts[u / tiles]), tile = u % tiles;
+                const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                const uint8_t* rec = L.records + uint64_t(e) * L.stride;
+                const uint4* codes = reinterpret_cast<const uint4*>(rec + p.ro[pr] + uint64_t(row) * (H / 2)) + G;
+                const uint16_t* sr = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64) + (G >> 1);
+                const uint16_t* br = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64) + (G >> 1);
+                const uint8_t* img[NT]; LdsBf16 src[NT]; int32_t slot[NT]; int nt = 0;
+                {
+                    int32_t s = head[e];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) { slot[t] = s; if (s >= 0) { nt = t + 1; s = next[s]; } }
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint32_t tt = t < nt ? uint32_t(slot[t]) / k : 0;
+                    img[t] = lds + lp.img_rg + tt * LH.bytes();
+                    src[t] = LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.xh) + tt * H};
+                }
+                XintTile<NT> tile_state; tile_state.clear();
+#pragma unroll 4
+                for (uint32_t dg = 0; dg < H / 128; ++dg)
+                    tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), img, LH, src, lane, nt);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (t >= nt) break;
+                    const float v = tile_state.finish(t);
+                    const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                    if (G == 0 && col < 8) st_f32(p.act + uint64_t(slot[t]) * I + row, swiglu_bf(v, up));
+                }
+            }
+        }
+        bar.wait();
+        // ---------------- phase D: down tiles per 16 output rows, combine ----------------
+        float* otile = reinterpret_cast<float*>(lds + lp.otile);
+        const uint32_t slots_total = n + T, SB = lp.slots_per_batch;
+        for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
+            for (uint32_t s0 = 0; s0 < slots_total; s0 += SB) {
+                const uint32_t sn = min(SB, slots_total - s0);
+                __syncthreads();
+                for (uint32_t q = 0; q < sn; ++q) {
+                    const uint32_t s = s0 + q;
+                    const float* a = s < n ? p.act + uint64_t(s) * I : p.shared_act + uint64_t(s - n) * I;
+                    uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah) + q * I;
+                    for (uint32_t i = tid; i < I; i += blockDim.x) ah[i] = uint16_t(__float_as_uint(load_shared_f32(a + i)) >> 16);
+                }
+                __syncthreads();
+                for (uint32_t q = 0; q < sn; ++q)
+                    xint_prepare(LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.ah) + q * I}, LI, lds + lp.img_d + q * LI.bytes());
+                __syncthreads();
+                for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
+                    // the unit's slots that lie in this batch, packed to the front
+                    int32_t slot[NT]; int nt = 0;
+                    const uint8_t* rec; const uint64_t* off;
+                    int32_t s = -1;
+                    if (u < U) { const uint32_t e = uint32_t(experts[u]); s = head[e]; rec = L.records + uint64_t(e) * L.stride; off = p.ro; }
+                    else { s = int32_t(n); rec = L.shared_record; off = p.so; }
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) slot[t] = 0;
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const bool have = u < U ? s >= 0 : uint32_t(s) < n + T;
+                        if (have) {
+                            if (uint32_t(s) >= s0 && uint32_t(s) < s0 + sn) {
+#pragma unroll
+                                for (int q = 0; q < NT; ++q) if (q == nt) slot[q] = s;
+                                ++nt;
+                            }
+                            s = u < U ? next[s] : s + 1;
+                        }
+                    }
+                    if (!nt) continue;
+                    const uint32_t row = rt * 16 + col;
+                    const uint4* codes = reinterpret_cast<const uint4*>(rec + off[6] + uint64_t(row) * (I / 2)) + G;
+                    const uint16_t* sr = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64) + (G >> 1);
+                    const uint16_t* br = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64) + (G >> 1);
+                    const uint8_t* img[NT]; LdsBf16 src[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const uint32_t q = t < nt ? uint32_t(slot[t]) - s0 : 0;
+                        img[t] = lds + lp.img_d + q * LI.bytes();
+                        src[t] = LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.ah) + q * I};
+                    }
+                    XintTile<NT> tile_state; tile_state.clear();
+#pragma unroll 4
+                    for (uint32_t dg = 0; dg < I / 128; ++dg)
+                        tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), img, LI, src, lane, nt);
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        if (t >= nt) break;
+                        const float v = bf(tile_state.finish(t));
+                        if (G == 0) otile[uint32_t(slot[t]) * 16 + col] = v;
+                    }
+                }
+            }
+            __syncthreads();
+            // weighted combine of the tile (reference: qwen.metal:804-816)
+            if (tid < T * 16) {
+                const uint32_t t = tid / 16, c = tid % 16;
+                float partial[8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) partial[q] = 0;
+                for (uint32_t kk = 0; kk < k; ++kk) {
+                    const int32_t e = ids[t * k + kk];
+                    const float value = (e >= 0 && e < int32_t(E)) ? otile[(t * k + kk) * 16 + c] : 0.0f;
+                    const float product = value * weights[t * k + kk];
+                    if (kk < 8) partial[kk] = product; else partial[kk % 8] = partial[kk % 8] + product;
+                }
+                float sum = partial[0];
+                for (uint32_t kk = 1; kk < 8 && kk < k; ++kk) sum += partial[kk];
+                const float g = bf(sigmoid_bf(gatev[t]));
+                const float y = bf(bf(sum) + bf(g * otile[(n + t) * 16 + c]));
+                const uint64_t at = uint64_t(t) * H + rt * 16 + c;
+                st_f32(p.layer_out + at, y);
+                if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * T * H + at, y);
+                if (layer + 1 == p.L) st_f32(p.out + at, y);
+                uint32_t m = __float_as_uint(y) & 0x7fffffffu;
+                if (m > 0x7f800000u) m = 0;   // NaN does not take part in the maximum
+#pragma unroll
+                for (int o = 8; o; o >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), o)));
+                if (c == 0) __hip_atomic_fetch_max(p.maxabs + layer * T + t, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        bar.wait();
+    }
+}
+
+static uint32_t align16(uint32_t v) { return (v + 15u) / 16u * 16u; }
+
+DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t NT, uint32_t lds_limit) {
+    DecodeLdsPlan lp{};
+    const XintLayout LH{H}, LI{I};
+    uint32_t at = 0;
+    auto take = [&](uint32_t bytes) { const uint32_t o = at; at += align16(bytes); return o; };
+    lp.ids = take(NT * topk * 4); lp.weights = take(NT * topk * 4); lp.gatev = take(NT * 4);
+    lp.head = take(E * 4); lp.next = take(NT * topk * 4); lp.experts = take(E * 4); lp.misc = take(64);
+    lp.region = at;
+    lp.img_rg = lp.region; lp.xh = lp.img_rg + NT * LH.bytes();
+    const uint32_t rg_end = lp.xh + align16(NT * H * 2);
+    lp.otile = lp.region;
+    const uint32_t slots = NT * (topk + 1);
+    lp.img_d = lp.otile + align16(slots * 16 * 4);
+    const uint32_t per_slot = LI.bytes() + align16(I * 2);
+    uint32_t sb = lp.img_d < lds_limit ? (lds_limit - lp.img_d) / per_slot : 0;
+    if (sb > slots) sb = slots;
+    lp.slots_per_batch = sb;
+    lp.ah = lp.img_d + sb * LI.bytes();
+    const uint32_t d_end = lp.ah + sb * align16(I * 2);
+    lp.total = rg_end > d_end ? rg_end : d_end;
+    return lp;
+}
+
+hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp) {
+#define ZC_DECODE(NT)                                                                                              \
+    do {                                                                                                           \
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<NT>),                  \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));             \
+        if (e != hipSuccess) return e;                                                                             \
+        hipLaunchKernelGGL((decode_stack_kernel<NT>), dim3(workgroups), dim3(kDecodeThreads), lp.total, s, p, lp);  \
+    } while (0)
+    if (nt == 1) ZC_DECODE(1); else if (nt == 2) ZC_DECODE(2); else if (nt == 4) ZC_DECODE(4); else ZC_DECODE(8);
+#undef ZC_DECODE
+    return hipGetLastError();
+}
+hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu) {
+    const void* f = nt == 1 ? reinterpret_cast<const void*>(decode_stack_kernel<1>)
+                  : nt == 2 ? reinterpret_cast<const void*>(decode_stack_kernel<2>)
+                  : nt == 4 ? reinterpret_cast<const void*>(decode_stack_kernel<4>)
+                            : reinterpret_cast<const void*>(decode_stack_kernel<8>);
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (e != hipSuccess) return e;
+    if (nt == 1) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<1>, kDecodeThreads, lds_bytes);
+    if (nt == 2) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<2>, kDecodeThreads, lds_bytes);
+    if (nt == 4) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<4>, kDecodeThreads, lds_bytes);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<8>, kDecodeThreads, lds_bytes);
+}
+
+}  // namespace zc

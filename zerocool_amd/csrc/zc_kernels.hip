@@ -404,20 +404,26 @@ void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, c
                     uint32_t T, uint32_t H, uint32_t topk, float* out) {
     hipLaunchKernelGGL(moe_sum_kernel, dim3((H + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
 }
-__global__ __launch_bounds__(256) void rms_glue_kernel(const float* x, uint32_t H, float* out) {
-    __shared__ float inv;
-    const float* row = x + uint64_t(blockIdx.x) * H;
-    if (threadIdx.x < 64) {
-        float acc = 0;
-        if (threadIdx.x < 32) for (uint32_t k = threadIdx.x; k < H; k += 32) acc = __builtin_fmaf(row[k], row[k], acc);
-        acc = lane_sum32(acc);
-        if (threadIdx.x == 0) inv = 1.0f / __builtin_sqrtf(acc / float(H) + 1e-6f);
+// Stand-in glue between stacked layers: x_next = bf(y * (1 / max|y|)) per token.
+__global__ __launch_bounds__(256) void stack_glue_kernel(const float* y, uint32_t H, float* out) {
+    __shared__ uint32_t wave_max[4];
+    const float* row = y + uint64_t(blockIdx.x) * H;
+    uint32_t m = 0;
+    for (uint32_t k = threadIdx.x; k < H; k += blockDim.x) {
+        const uint32_t a = __float_as_uint(row[k]) & 0x7fffffffu;
+        if (a <= 0x7f800000u) m = max(m, a);   // NaN does not take part
     }
+#pragma unroll
+    for (int o = 32; o; o >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), o)));
+    if ((threadIdx.x & 63u) == 0) wave_max[threadIdx.x >> 6] = m;
     __syncthreads();
+    m = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+    const float top = __uint_as_float(m);
+    const float inv = (top > 0.0f && top < __uint_as_float(0x7f800000u)) ? 1.0f / top : 1.0f;
     for (uint32_t k = threadIdx.x; k < H; k += blockDim.x) out[uint64_t(blockIdx.x) * H + k] = bf(row[k] * inv);
 }
-void launch_rms_glue(hipStream_t s, const float* x, uint32_t T, uint32_t H, float* out) {
-    hipLaunchKernelGGL(rms_glue_kernel, dim3(T), dim3(256), 0, s, x, H, out);
+void launch_stack_glue(hipStream_t s, const float* y, uint32_t T, uint32_t H, float* out) {
+    hipLaunchKernelGGL(stack_glue_kernel, dim3(T), dim3(256), 0, s, y, H, out);
 }
 
 // ---------------------------------------------------------------------------

@@ -40,11 +40,36 @@ void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_
 void launch_scatter(hipStream_t s, const float* x, const int32_t* positions, uint32_t n, uint32_t H, float* out);
 void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, const float* shared, const float* gate,
                     uint32_t T, uint32_t H, uint32_t topk, float* out);
-void launch_rms_glue(hipStream_t s, const float* x, uint32_t T, uint32_t H, float* out);
+void launch_stack_glue(hipStream_t s, const float* y, uint32_t T, uint32_t H, float* out);
 void launch_synth_words(hipStream_t s, uint32_t* dst, uint64_t count, uint64_t seed);
 void launch_synth_scales(hipStream_t s, uint16_t* sc, uint16_t* bi, uint64_t count, uint64_t seed, float lo, float span, float factor);
 void launch_synth_normal(hipStream_t s, void* dst, uint64_t count, uint64_t seed, float sigma, bool half);
 void launch_synth_records(hipStream_t s, void* records, uint64_t stride, uint32_t count, const uint64_t* w_off,
                           const uint64_t* s_off, const uint64_t* words, const uint64_t* meta, const uint32_t* bits, uint64_t seed);
+
+
+// Persistent stacked decode (zc_decode.hip)
+struct DecodeLayer {
+    const uint16_t* router; const float* offsets; const uint16_t* shared_gate;
+    const uint8_t* shared_record; const uint8_t* records; uint64_t stride;
+};
+struct DecodeParams {
+    uint32_t H, E, topk, I, T, L;
+    uint64_t ro[9], so[9];           // byte offsets [projection*3 + {codes, scales, biases}] in a routed / shared record
+    const DecodeLayer* layers;       // device array [L]
+    const float* x_in; float* out;   // [T][H]
+    float *logits, *gate, *shared_act, *act, *layer_out;   // exchange buffers
+    uint32_t* maxabs;                // [L][T] bit patterns of max |layer output|
+    int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][T][topk], [L][T][topk], [L][T][H]
+    uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
+};
+struct DecodeLdsPlan {
+    uint32_t ids, weights, gatev, head, next, experts, misc, region, total;
+    uint32_t img_rg, xh, img_d, ah, otile, slots_per_batch;
+};
+DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t NT, uint32_t lds_limit);
+hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp);
+hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu);
+constexpr uint32_t kDecodeSyncBytes = (32 * 1024 + 16 * 64) * 4;
 
 }  // namespace zc

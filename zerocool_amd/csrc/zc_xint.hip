@@ -20,11 +20,11 @@ template <int NT, bool GATED>
 __device__ __forceinline__ void xint_rows(const XintJob& j, uint32_t tile, uint32_t t0, uint8_t* lds_base) {
     const XintLayout L{j.K};
     const uint32_t lane = threadIdx.x & 63u, col = lane & 15u, G = lane >> 4;
-    const uint8_t* lds[NT]; const float* xr[NT];
+    const uint8_t* lds[NT]; GlobalF32 xr[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const uint32_t tt = min(t0 + t, j.tokens - 1);
-        xr[t] = j.x + uint64_t(j.in_rows ? uint32_t(j.in_rows[tt]) : tt) * j.K;
+        xr[t] = GlobalF32{j.x + uint64_t(j.in_rows ? uint32_t(j.in_rows[tt]) : tt) * j.K};
         lds[t] = lds_base + t * L.bytes();
         xint_prepare(xr[t], L, lds_base + t * L.bytes());
     }

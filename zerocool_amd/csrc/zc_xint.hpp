@@ -47,9 +47,22 @@ __device__ __forceinline__ float load_shared_f32(const float* p) {
     return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
 
-// Builds the LDS image of x[0..K) cooperatively (all threads of the workgroup call it,
-// then __syncthreads()).  One thread per block.
-__device__ __forceinline__ void xint_prepare(const float* x, const XintLayout L, uint8_t* lds) {
+// Input sources.  bits(k) returns the fp32 bit pattern of element k.
+struct GlobalF32 {   // a row in global memory, possibly written by another workgroup
+    const float* x;
+    __device__ __forceinline__ uint32_t bits(uint32_t k) const { return __float_as_uint(load_shared_f32(x + k)); }
+    __device__ __forceinline__ float at(uint32_t k) const { return load_shared_f32(x + k); }
+};
+struct LdsBf16 {     // a BF16 copy of the row in LDS
+    const uint16_t* x;
+    __device__ __forceinline__ uint32_t bits(uint32_t k) const { return uint32_t(x[k]) << 16; }
+    __device__ __forceinline__ float at(uint32_t k) const { return b16(x[k]); }
+};
+
+// Builds the LDS image of a K-element row cooperatively (all threads of the workgroup
+// call it, then __syncthreads()).  One thread per block.
+template <class Source>
+__device__ __forceinline__ void xint_prepare(const Source x, const XintLayout L, uint8_t* lds) {
     uint8_t* planes = lds;
     float2* info = reinterpret_cast<float2*>(lds + L.planes_bytes());
     uint32_t* mask = reinterpret_cast<uint32_t*>(lds + L.planes_bytes() + L.info_bytes());
@@ -59,7 +72,7 @@ __device__ __forceinline__ void xint_prepare(const float* x, const XintLayout L,
     for (uint32_t b = threadIdx.x; b < L.blocks(); b += blockDim.x) {
         uint32_t bits[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) bits[i] = __float_as_uint(load_shared_f32(x + b * 16 + i));
+        for (int i = 0; i < 16; ++i) bits[i] = x.bits(b * 16 + i);
         // bias sum: BF16 rounding after each addition of four inputs (reference: qwen.metal:55)
         float sum = 0;
 #pragma unroll
@@ -111,13 +124,14 @@ __device__ __forceinline__ void xint_prepare(const float* x, const XintLayout L,
 
 // The literal fp32 chain of one block (reference: qwen.metal:52-57) for a lane that
 // holds the block's two code words.
-__device__ __forceinline__ float xint_literal_dot(uint32_t w0, uint32_t w1, const float* xb) {
+template <class Source>
+__device__ __forceinline__ float xint_literal_dot(uint32_t w0, uint32_t w1, const Source x, uint32_t k0) {
     float dot = 0;
 #pragma unroll
     for (int i = 0; i < 16; i += 4) {
         const uint32_t packed = ((i < 8 ? w0 : w1) >> (4 * (i % 8))) & 0xffffu;
-        dot += load_shared_f32(xb + i) * float(packed & 15u) + load_shared_f32(xb + i + 1) * float((packed >> 4) & 15u) +
-               load_shared_f32(xb + i + 2) * float((packed >> 8) & 15u) + load_shared_f32(xb + i + 3) * float((packed >> 12) & 15u);
+        dot += x.at(k0 + i) * float(packed & 15u) + x.at(k0 + i + 1) * float((packed >> 4) & 15u) +
+               x.at(k0 + i + 2) * float((packed >> 8) & 15u) + x.at(k0 + i + 3) * float((packed >> 12) & 15u);
     }
     return dot;
 }
@@ -136,8 +150,10 @@ struct XintTile {
     }
     // One 128-element span `dg` of the row: codes = the lane's 16 bytes (blocks 2G, 2G+1),
     // scale/bias = the row's group values for group 2*dg + G/2.
+    // nt <= NT tokens are live (wave-uniform); lds[t] / x[t] are token t's image and source.
+    template <class Source>
     __device__ __forceinline__ void step(uint32_t dg, const uint4 codes, float scale, float bias, const uint8_t* const* lds,
-                                         const XintLayout L, const float* const* x, uint32_t lane) {
+                                         const XintLayout L, const Source* x, uint32_t lane, int nt = NT) {
         const uint32_t G = lane >> 4, i = lane & 15u, c = i >> 2, p = i & 3u;
         const uint32_t M = 0x0f0f0f0fu;
         v4i b0 = {int(codes.x & M), int((codes.x >> 4) & M), int(codes.y & M), int((codes.y >> 4) & M)};
@@ -148,6 +164,7 @@ struct XintTile {
         const uint32_t zero_slot = L.blocks() * 48;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
+            if (t >= nt) break;
             const uint8_t* planes = lds[t];
             const float2* info = reinterpret_cast<const float2*>(planes + L.planes_bytes());
             const uint32_t* mask = reinterpret_cast<const uint32_t*>(planes + L.planes_bytes() + L.info_bytes());
@@ -162,7 +179,7 @@ struct XintTile {
                 const v4i d = h ? d1 : d0;
                 const float2 fi = info[blk + h];
                 float dot = float(d[0] + (d[1] << 7) + (d[2] << 14)) * fi.x;
-                if (unsafe & (1u << h)) dot = xint_literal_dot(h ? codes.z : codes.x, h ? codes.w : codes.y, x[t] + (blk + h) * 16);
+                if (unsafe & (1u << h)) dot = xint_literal_dot(h ? codes.z : codes.x, h ? codes.w : codes.y, x[t], (blk + h) * 16);
                 acc[t][dg & 3u][h] += scale * dot + fi.y * bias;
             }
         }

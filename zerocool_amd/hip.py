@@ -33,6 +33,10 @@ class Layer(C.Structure):
                 ("shared_record", C.c_void_p), ("expert_records", C.c_void_p), ("record_stride", C.c_uint64)]
 
 
+class StackTrace(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("ids", "weights", "outputs")]
+
+
 class Trace(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("logits", "ids", "weights", "expert_out", "shared", "gate")]
 
@@ -214,8 +218,24 @@ class Context:
     def moe_check(self):
         self._call("zc_hip_moe_check")
 
-    def rms_glue(self, x, tokens, hidden, out):
-        self._call("zc_hip_rms_glue", _ptr(x), C.c_uint32(tokens), C.c_uint32(hidden), _ptr(out))
+    def stack_glue(self, y, tokens, hidden, out):
+        self._call("zc_hip_stack_glue", _ptr(y), C.c_uint32(tokens), C.c_uint32(hidden), _ptr(out))
+
+    def stack_create(self, cfg, layers, max_tokens):
+        arr = (Layer * len(layers))(*layers)
+        h = C.c_void_p()
+        self._call("zc_hip_stack_create", C.byref(cfg), arr, C.c_uint32(len(layers)), C.c_uint32(max_tokens), C.byref(h))
+        return h
+
+    def stack_destroy(self, stack):
+        self._call("zc_hip_stack_destroy", stack)
+
+    def stack_decode(self, stack, x, tokens, out, trace=None, layered=False):
+        self._call("zc_hip_stack_decode", stack, _ptr(x), C.c_uint32(tokens), _ptr(out),
+                   C.byref(trace) if trace is not None else None, C.c_uint32(1 if layered else 0))
+
+    def stack_is_persistent(self, stack, tokens):
+        return bool(self.lib.zc_hip_stack_is_persistent(self.handle, stack, C.c_uint32(tokens)))
 
     # synthetic tensors ---------------------------------------------------
     def synth_words(self, dst, count, seed):

@@ -87,6 +87,10 @@ zc_status zc_hip_finish(zc_hip_ctx* ctx);
  * the shape allows (wide Q4, group 64), literal otherwise.  Default 1.  Both policies
  * produce identical bytes; only speed differs. */
 zc_status zc_hip_configure(zc_hip_ctx* ctx, uint32_t affine_policy);
+/* HIP-event stopwatch on the context's stream: start enqueues an event, stop enqueues a
+ * second one, waits for it and returns the milliseconds between them. */
+zc_status zc_hip_timer_start(zc_hip_ctx* ctx);
+zc_status zc_hip_timer_stop(zc_hip_ctx* ctx, float* milliseconds);
 /* The raw hipStream_t the context enqueues on (for event timing by the caller). */
 void* zc_hip_stream(zc_hip_ctx* ctx);
 
@@ -160,6 +164,9 @@ typedef struct {       /* optional device buffers, any may be NULL */
     int32_t* ids;      /* [n_layers][tokens][topk] */
     float* weights;    /* [n_layers][tokens][topk] */
     float* outputs;    /* [n_layers][tokens][hidden] layer outputs before the glue */
+    uint64_t* clocks;  /* [n_layers][10] timestamps (100 MHz) of the persistent kernel's workgroup 0 at
+                          layer start, images built, phase R done, barrier 1, routed, phase G done,
+                          barrier 2, phase D done, barrier 3 (tuning aid; persistent path only) */
 } zc_stack_trace;
 zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
                               uint32_t n_layers, uint32_t max_tokens, zc_hip_stack** out);

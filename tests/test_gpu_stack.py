@@ -45,7 +45,7 @@ def run_stack(ctx, cfg, stack, x_dev, T, L, layered):
     n = T * cfg.topk
     ids, w, outs = ctx.alloc(L * n * 4), ctx.alloc(L * n * 4), ctx.alloc(L * T * cfg.hidden * 4)
     out = ctx.alloc(T * cfg.hidden * 4)
-    ctx.stack_decode(stack, x_dev, T, out, z.StackTrace(ids.ptr, w.ptr, outs.ptr), layered=layered)
+    ctx.stack_decode(stack, x_dev, T, out, z.StackTrace(ids.ptr, w.ptr, outs.ptr, None), layered=layered)
     ctx.moe_check()
     r = (ids.numpy(np.int32).reshape(L, T, cfg.topk), w.numpy(f32).reshape(L, T, cfg.topk),
          outs.numpy(f32).reshape(L, T, cfg.hidden), out.numpy(f32).reshape(T, cfg.hidden))

@@ -37,6 +37,7 @@ struct zc_hip_ctx {
     std::vector<hipEvent_t> tickets;   // live tickets: ticket t -> tickets[t - retired - 1]
     uint64_t retired = 0;              // tickets known complete and destroyed
     int32_t* moe_status = nullptr;     // device flag: an id outside [0,E) was seen
+    hipEvent_t timer[2] = {nullptr, nullptr};
     uint32_t affine_policy = 1;        // 0 literal lane kernels, 1 exact-integer matrix-core kernels where possible
     std::mutex mutex;
 };
@@ -66,6 +67,7 @@ zc_status zc_hip_destroy(zc_hip_ctx* ctx) {
     hipSetDevice(ctx->device);
     hipStreamSynchronize(ctx->stream);
     for (auto e : ctx->tickets) hipEventDestroy(e);
+    for (auto e : ctx->timer) if (e) hipEventDestroy(e);
     for (auto& b : ctx->blocks) hipFree(b.first);
     hipFree(ctx->moe_status);
     hipStreamDestroy(ctx->stream);
@@ -121,6 +123,19 @@ zc_status zc_hip_configure(zc_hip_ctx* ctx, uint32_t affine_policy) {
     ZC_REQUIRE(ctx, "null context");
     ZC_REQUIRE(affine_policy <= 1, "unknown kernel policy");
     ctx->affine_policy = affine_policy;
+    return ZC_OK;
+}
+zc_status zc_hip_timer_start(zc_hip_ctx* ctx) {
+    ZC_REQUIRE(ctx, "null context");
+    for (auto& e : ctx->timer) if (!e) ZC_HIP(hipEventCreate(&e));
+    ZC_HIP(hipEventRecord(ctx->timer[0], ctx->stream));
+    return ZC_OK;
+}
+zc_status zc_hip_timer_stop(zc_hip_ctx* ctx, float* milliseconds) {
+    ZC_REQUIRE(ctx && milliseconds && ctx->timer[0], "timer was not started");
+    ZC_HIP(hipEventRecord(ctx->timer[1], ctx->stream));
+    ZC_HIP(hipEventSynchronize(ctx->timer[1]));
+    ZC_HIP(hipEventElapsedTime(milliseconds, ctx->timer[0], ctx->timer[1]));
     return ZC_OK;
 }
 uint64_t zc_hip_allocated(const zc_hip_ctx* ctx) { return ctx ? ctx->allocated : 0; }
@@ -443,9 +458,9 @@ struct zc_hip_stack {
 namespace {
 bool persistent_shape(const zc_moe_config& c) {
     return c.bits_gate_up == 4 && c.bits_down == 4 && c.shared_bits_gate_up == 4 && c.shared_bits_down == 4 && c.group == 64 &&
-           c.hidden % 512 == 0 && c.inter % 512 == 0 && c.experts <= 1024 && c.topk <= 64;
+           c.hidden % 512 == 0 && c.inter % 512 == 0 && c.hidden <= 3072 && c.inter <= 1024 && c.experts <= 1024 && c.topk <= 64;
 }
-uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : tokens <= 2 ? 2 : tokens <= 4 ? 4 : 8; }
+uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : 8; }   // kernel variant; LDS is sized by the real token count
 }  // namespace
 
 extern "C" {
@@ -518,8 +533,8 @@ static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, 
     if (!st->persistent_ok || tokens > 8 || tokens > st->max_tokens) return false;
     const zc_moe_config& c = st->cfg;
     *nt = token_tile(tokens);
-    if (tokens * c.topk > 512) return false;
-    *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, *nt, st->lds_limit);
+    if (tokens * c.topk > 256) return false;
+    *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
     if (plan->total > st->lds_limit || plan->slots_per_batch == 0) return false;
     int per_cu = 0;
     if (zc::decode_stack_occupancy(*nt, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
@@ -553,6 +568,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.maxabs = st->maxabs;
         p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
         if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
+        p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = 1u << 22;
         st->epoch += 3 * L + 16;   // wraps modulo 2^32; the barrier compares epochs as signed differences
         const uint32_t workgroups = uint32_t(st->cus);

@@ -27,7 +27,7 @@ namespace zc {
 __device__ __forceinline__ void st_f32(float* p, float v) { ZC_ST(reinterpret_cast<uint32_t*>(p), __float_as_uint(v)); }
 __device__ __forceinline__ void st_i32(int32_t* p, int32_t v) { ZC_ST(reinterpret_cast<uint32_t*>(p), uint32_t(v)); }
 
-constexpr uint32_t kDecodeThreads = 512, kDecodeWaves = 8;
+constexpr uint32_t kDecodeThreads = 256, kDecodeWaves = 4;
 constexpr uint32_t kFlagStride = 32, kReleaseBase = 32 * 1024, kReleaseStride = 64, kAbortWord = kReleaseBase + 8 * kReleaseStride;
 
 struct Barrier {
@@ -62,40 +62,48 @@ struct Barrier {
     }
 };
 
-template <int NT>
+// Top-k of one token by one wavefront.  Lane l holds experts l*per .. l*per+per-1, so the
+// lowest lane holding the maximum, then the lowest slot inside it, is the lowest expert id:
+// one DPP maximum, one ballot and two scalar-lane reads per pick.
+template <int PER, class Clock>
 __device__ __forceinline__ void route_token(const float* logits, uint32_t E, uint32_t topk, uint32_t lane,
-                                            int32_t* ids, float* weights) {
-    constexpr int PER = 16;
+                                            int32_t* ids, float* weights, Clock clock) {
+    const uint32_t per = PER == 16 ? (E + 63) / 64 : uint32_t(PER);
     const float ninf = __uint_as_float(0xff800000u);
     float cand[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        const uint32_t e = lane + 64u * i;
-        const float c = e < E ? load_shared_f32(logits + e) : ninf;
-        cand[i] = c > ninf ? c : ninf;
+        const uint32_t e = lane * per + i;
+        const float c = (uint32_t(i) < per && e < E) ? load_shared_f32(logits + e) : ninf;
+        cand[i] = c > ninf ? c : ninf;   // NaN and -inf never win
     }
     float score = ninf, top = ninf;   // lane j keeps score j
+    if (__ballot(cand[0] == 12345.678f) == ~0ull) return;   // (forces the loads to complete before the stamp)
+    clock();
     for (uint32_t j = 0; j < topk; ++j) {
-        float best = ninf; uint32_t index = 0x7fffffffu;
+        float best = cand[0];
 #pragma unroll
-        for (int i = 0; i < PER; ++i) if (cand[i] > best) { best = cand[i]; index = lane + 64u * i; }
-        float m = best;
+        for (int i = 1; i < PER; ++i) if (uint32_t(i) < per) best = fmaxf(best, cand[i]);
+        const float m = wave_max_f32(best);
+        const uint64_t holders = __ballot(best == m && m > ninf);
+        const bool found = holders != 0;
+        const uint32_t owner = found ? uint32_t(__ffsll((long long)holders) - 1) : 0u;
+        int first = PER;
 #pragma unroll
-        for (int o = 32; o; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-        uint32_t winner = (best == m && best > ninf) ? index : 0x7fffffffu;
+        for (int i = PER - 1; i >= 0; --i) if (uint32_t(i) < per && cand[i] == m) first = i;
+        float value = ninf;   // the winner's original bits (signed zero included)
 #pragma unroll
-        for (int o = 32; o; o >>= 1) winner = min(winner, uint32_t(__shfl_xor(int(winner), o)));
-        const bool found = winner < E;
-        // the owner's candidate keeps the original bits (signed zero included)
-        float value = ninf;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) if (lane + 64u * i == winner) { value = cand[i]; cand[i] = ninf; }
-        value = __shfl(value, found ? (winner & 63u) : 0);
+        for (int i = 0; i < PER; ++i) if (i == first) value = cand[i];
+        const uint32_t winner = uint32_t(__builtin_amdgcn_readlane(int(lane * per + uint32_t(first)), int(owner)));
+        value = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, value), int(owner)));
         if (!found) value = ninf;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) if (found && lane == owner && i == first) cand[i] = ninf;
         if (lane == j) score = value;
         if (j == 0) top = value;
         if (lane == 0) ids[j] = found ? int32_t(winner) : -1;
     }
+    clock();
     // softmax over the selected: reference lane l sums values 4l..4l+3 (qwen.metal:758-764)
     const float v = lane < topk ? exp32(score - top) : 0.0f;
     float s4 = 0;
@@ -108,8 +116,14 @@ __device__ __forceinline__ void route_token(const float* logits, uint32_t E, uin
     if (lane < topk) weights[lane] = v * inverse;
 }
 
+constexpr int kRing = 8;         // 128-element spans of a tile in flight per lane (four when the span count is odd in eights)
+#define ZC_RUN_TILE(SPANS, ...) do { if ((SPANS) % 8 == 0) xint_run_tile<PT, 8>(__VA_ARGS__); else xint_run_tile<PT, 4>(__VA_ARGS__); } while (0)
+constexpr int kMaxTokens = 8;
+
+// NT = 1: single-token decode.  NT = 8: up to eight tokens, tiles take four at a time.
 template <int NT>
 __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
+    constexpr int PT = NT < 4 ? NT : 4;   // tokens per tile pass
     extern __shared__ __align__(16) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wg = blockIdx.x, nwg = gridDim.x;
     const uint32_t H = p.H, E = p.E, I = p.I, k = p.topk, T = p.T, n = T * k;
@@ -121,26 +135,36 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
     int32_t* next = reinterpret_cast<int32_t*>(lds + lp.next);
     int32_t* experts = reinterpret_cast<int32_t*>(lds + lp.experts);
     int32_t* misc = reinterpret_cast<int32_t*>(lds + lp.misc);   // [0] U, [1..8] wave counts
+    const uint16_t* xh_all = reinterpret_cast<const uint16_t*>(lds + lp.xh);
     const XintLayout LH{H}, LI{I};
     Barrier bar{p.sync, p.epoch, p.spin_limit, p.status, p.epoch};
+    uint32_t stamp = 0;
+    auto clock = [&]() { if (p.clocks && wg == 0 && tid == 0) p.clocks[stamp] = wall_clock64(); ++stamp; };
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
 
     for (uint32_t layer = 0; layer < p.L; ++layer) {
         const DecodeLayer L = p.layers[layer];
+        clock();
+        if (p.clocks) {   // calibration: 1024 dependent fused multiply-adds
+            float v = __uint_as_float(p.epoch);
+            for (int i = 0; i < 1024; ++i) v = __builtin_fmaf(v, 1.0000001f, 0.5f);
+            if (v == 12345.0f) atomicOr(p.status, 8);
+        }
+        clock();
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
-        for (uint32_t t = 0; t < T; ++t) {
-            uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh) + t * H;
-            float inv = 1.0f;
-            if (layer) {
-                const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + t));
-                if (m > 0.0f && m < __uint_as_float(0x7f800000u)) inv = 1.0f / m;
+        {
+            uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
+            if (layer && tid < T) {   // the glue's scale per token, kept where the gate values go later
+                const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
+                gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
             }
+            __syncthreads();
             int bad = 0;
-            for (uint32_t i = tid; i < H; i += blockDim.x) {
-                float v = load_shared_f32((layer ? p.layer_out : p.x_in) + uint64_t(t) * H + i);
-                if (layer) v = bf(v * inv);
+            for (uint32_t i = tid; i < T * H; i += blockDim.x) {
+                float v = load_shared_f32((layer ? p.layer_out : p.x_in) + i);
+                if (layer) v = bf(v * gatev[i / H]);
                 const uint32_t u = __float_as_uint(v);
                 bad |= (u & 0xffffu) != 0;
                 xh[i] = uint16_t(u >> 16);
@@ -148,9 +172,8 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
             if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
         }
         __syncthreads();
-        for (uint32_t t = 0; t < T; ++t)
-            xint_prepare(LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.xh) + t * H}, LH, lds + lp.img_rg + t * LH.bytes());
-        __syncthreads();
+        xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
+        clock();
         {
             const uint32_t router_units = (E + 3) / 4, shared_units = I / 8, gate_units = (T + 1) / 2;
             const uint32_t units = router_units + shared_units + gate_units;
@@ -158,79 +181,89 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 if (u < router_units) {
                     // four experts x sixteen K partitions; k-ascending fused chain per partition
                     const uint32_t e = u * 4 + lane / 16, split = lane % 16, P = H / 16;
+                    const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
+                    const uint32_t pieces = P / 8;   // sixteen-byte pieces of the partition, kRing in flight
+                    uint4 wv[kRing];
+#pragma unroll
+                    for (int i = 0; i < kRing; ++i) if (uint32_t(i) < pieces) wv[i] = ldg_u4(wr, i);
                     float c[NT];
 #pragma unroll
                     for (int t = 0; t < NT; ++t) c[t] = 0;
-                    if (e < E) {
-                        const uint16_t* wr = L.router + uint64_t(e) * H + split * P;
-                        for (uint32_t i = 0; i < P; i += 8) {
-                            const uint4 wv = *reinterpret_cast<const uint4*>(wr + i);
-                            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+                    for (uint32_t i0 = 0; i0 < pieces; i0 += kRing) {
 #pragma unroll
-                            for (int t = 0; t < NT; ++t) {
-                                if (t >= int(T)) break;
-                                const uint4 xv = *reinterpret_cast<const uint4*>(lds + lp.xh + (uint64_t(t) * H + split * P + i) * 2);
-                                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+                        for (int j = 0; j < kRing; ++j) {
+                            const uint32_t i = i0 + j;
+                            if (i < pieces) {
+                                const uint32_t ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+                                if (i + kRing < pieces) wv[j] = ldg_u4(wr, i + kRing);
 #pragma unroll
-                                for (int q = 0; q < 4; ++q) {
-                                    c[t] = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c[t]);
-                                    c[t] = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c[t]);
+                                for (int t = 0; t < NT; ++t) {
+                                    if (t >= int(T)) break;
+                                    const uint4 xv = *reinterpret_cast<const uint4*>(xh_all + uint64_t(t) * H + split * P + i * 8);
+                                    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q) {
+                                        c[t] = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c[t]);
+                                        c[t] = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c[t]);
+                                    }
                                 }
                             }
                         }
                     }
-                    const uint32_t base = lane & ~15u;
+                    // partials added 0..15: after step s the lane of partition i <= s holds ((c0 + c1) + ..) + ci
+                    const float offset = (L.offsets && e < E) ? ldg_f32(L.offsets, e) : 0.0f;
 #pragma unroll
                     for (int t = 0; t < NT; ++t) {
                         if (t >= int(T)) break;
-                        float sum = 0;
-                        for (uint32_t sidx = 0; sidx < 16; ++sidx) sum += __shfl(c[t], base + sidx);
-                        if (split == 0 && e < E) st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + L.offsets[e] : sum);
+                        float sum = 0.0f + c[t];
+#pragma unroll
+                        for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c[t];
+                        if (split == 15 && e < E) st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + offset : sum);
                     }
                 } else if (u < router_units + shared_units) {
                     const uint32_t tile = u - router_units, row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                     const uint8_t* rec = L.shared_record;
-                    const uint4* codes = reinterpret_cast<const uint4*>(rec + p.so[pr] + uint64_t(row) * (H / 2)) + G;
-                    const uint16_t* sr = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64) + (G >> 1);
-                    const uint16_t* br = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64) + (G >> 1);
-                    const uint8_t* img[NT]; LdsBf16 src[NT];
+                    const uint8_t* w_row = rec + p.so[pr] + uint64_t(row) * (H / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64);
+                    for (uint32_t t0 = 0; t0 < T; t0 += PT) {
+                        const uint8_t* img[PT]; LdsBf16 src[PT];
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        const uint32_t tt = t < int(T) ? t : 0;
-                        img[t] = lds + lp.img_rg + tt * LH.bytes();
-                        src[t] = LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.xh) + tt * H};
-                    }
-                    XintTile<NT> tile_state; tile_state.clear();
-#pragma unroll 4
-                    for (uint32_t dg = 0; dg < H / 128; ++dg)
-                        tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), img, LH, src, lane, int(T));
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        if (t >= int(T)) break;
-                        const float v = tile_state.finish(t);
-                        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
-                        if (G == 0 && col < 8) st_f32(p.shared_act + uint64_t(t) * I + row, swiglu_bf(v, up));
+                        for (int t = 0; t < PT; ++t) {
+                            const uint32_t tt = t0 + t < T ? t0 + t : 0;
+                            img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
+                        }
+                        auto emit = [&](int t, float v) {
+                            const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                            if (G == 0 && col < 8) st_f32(p.shared_act + uint64_t(t0 + t) * I + row, swiglu_bf(v, up));
+                        };
+                        ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, int(min(uint32_t(PT), T - t0)), emit);
                     }
                 } else {
                     // shared_expert_gate: reference lane chain k = lane + 32 j (qwen.metal:499-506); two tokens per wave
                     const uint32_t t = (u - router_units - shared_units) * 2 + (lane >> 5), l32 = lane & 31u;
                     float sum = 0;
-                    if (t < T) {
-                        const uint16_t* xh = reinterpret_cast<const uint16_t*>(lds + lp.xh) + t * H;
-                        for (uint32_t kk = l32; kk < H; kk += 32) sum += b16(xh[kk]) * b16(L.shared_gate[kk]);
-                    }
+                    if (t < T)
+                        for (uint32_t kk = l32; kk < H; kk += 32) sum += b16(xh_all[t * H + kk]) * b16(ldg_u16(L.shared_gate, kk));
                     sum = lane_sum32(sum);
                     if (t < T && l32 == 0) st_f32(p.gate + t, bf(sum));
                 }
             }
         }
+        clock();
         bar.wait();
+        clock();
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
         for (uint32_t t = wave; t < T; t += kDecodeWaves)
-            route_token<NT>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k);
+        {
+            auto stamp = [&]() { if (t == 0) clock(); };
+            if (E == 512) route_token<8>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
+            else route_token<16>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
+        }
         if (tid < T) gatev[tid] = load_shared_f32(p.gate + tid);
         for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
         __syncthreads();
+        clock();
         if (tid < n) {
             const int32_t e = ids[tid];
             if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); next[tid] = -1; }
@@ -256,104 +289,88 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
         }
         __syncthreads();
         const uint32_t U = uint32_t(misc[0]);
+        clock();
         {
             const uint32_t tiles = I / 8, units = U * tiles;
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
                 const uint32_t e = uint32_t(experts[u / tiles]), tile = u % tiles;
                 const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                 const uint8_t* rec = L.records + uint64_t(e) * L.stride;
-                const uint4* codes = reinterpret_cast<const uint4*>(rec + p.ro[pr] + uint64_t(row) * (H / 2)) + G;
-                const uint16_t* sr = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64) + (G >> 1);
-                const uint16_t* br = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64) + (G >> 1);
-                const uint8_t* img[NT]; LdsBf16 src[NT]; int32_t slot[NT]; int nt = 0;
-                {
-                    int32_t s = head[e];
+                const uint8_t* w_row = rec + p.ro[pr] + uint64_t(row) * (H / 2);
+                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64);
+                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64);
+                int32_t s = head[e];
+                while (s >= 0) {   // the expert's slots, PT at a time
+                    const uint8_t* img[PT]; LdsBf16 src[PT]; int32_t slot[PT]; int nt = 0;
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) { slot[t] = s; if (s >= 0) { nt = t + 1; s = next[s]; } }
-                }
+                    for (int t = 0; t < PT; ++t) { slot[t] = s; if (s >= 0) { nt = t + 1; s = next[s]; } }
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const uint32_t tt = t < nt ? uint32_t(slot[t]) / k : 0;
-                    img[t] = lds + lp.img_rg + tt * LH.bytes();
-                    src[t] = LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.xh) + tt * H};
-                }
-                XintTile<NT> tile_state; tile_state.clear();
-#pragma unroll 4
-                for (uint32_t dg = 0; dg < H / 128; ++dg)
-                    tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), img, LH, src, lane, nt);
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    if (t >= nt) break;
-                    const float v = tile_state.finish(t);
-                    const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
-                    if (G == 0 && col < 8) st_f32(p.act + uint64_t(slot[t]) * I + row, swiglu_bf(v, up));
+                    for (int t = 0; t < PT; ++t) {
+                        const uint32_t tt = t < nt ? uint32_t(slot[t]) / k : 0;
+                        img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
+                    }
+                    auto emit = [&](int t, float v) {
+                        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                        if (G == 0 && col < 8) st_f32(p.act + uint64_t(slot[t]) * I + row, swiglu_bf(v, up));
+                    };
+                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, nt, emit);
                 }
             }
         }
+        clock();
         bar.wait();
+        clock();
         // ---------------- phase D: down tiles per 16 output rows, combine ----------------
         float* otile = reinterpret_cast<float*>(lds + lp.otile);
         const uint32_t slots_total = n + T, SB = lp.slots_per_batch;
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
+            const uint32_t row = rt * 16 + col;
             for (uint32_t s0 = 0; s0 < slots_total; s0 += SB) {
                 const uint32_t sn = min(SB, slots_total - s0);
                 __syncthreads();
-                for (uint32_t q = 0; q < sn; ++q) {
-                    const uint32_t s = s0 + q;
-                    const float* a = s < n ? p.act + uint64_t(s) * I : p.shared_act + uint64_t(s - n) * I;
-                    uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah) + q * I;
-                    for (uint32_t i = tid; i < I; i += blockDim.x) ah[i] = uint16_t(__float_as_uint(load_shared_f32(a + i)) >> 16);
+                uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
+                for (uint32_t i = tid; i < sn * I / 2; i += blockDim.x) {   // two activations per coherent 8-byte read
+                    const uint32_t sl = s0 + (2 * i) / I, kk = (2 * i) % I;
+                    const float* a = sl < n ? p.act + uint64_t(sl) * I : p.shared_act + uint64_t(sl - n) * I;
+                    const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(a + kk), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    reinterpret_cast<uint32_t*>(ah)[i] = (uint32_t(v) >> 16) | (uint32_t(v >> 32) & 0xffff0000u);
                 }
                 __syncthreads();
-                for (uint32_t q = 0; q < sn; ++q)
-                    xint_prepare(LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.ah) + q * I}, LI, lds + lp.img_d + q * LI.bytes());
-                __syncthreads();
+                auto source_of = [&](uint32_t q) { return LdsBf16{ah + q * I}; };
+                if (s0 == 0) clock();
+                xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
+                if (s0 == 0) clock();
                 for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
-                    // the unit's slots that lie in this batch, packed to the front
-                    int32_t slot[NT]; int nt = 0;
-                    const uint8_t* rec; const uint64_t* off;
-                    int32_t s = -1;
+                    const uint8_t* rec; const uint64_t* off; int32_t s;
                     if (u < U) { const uint32_t e = uint32_t(experts[u]); s = head[e]; rec = L.records + uint64_t(e) * L.stride; off = p.ro; }
                     else { s = int32_t(n); rec = L.shared_record; off = p.so; }
+                    const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
+                    while (u < U ? s >= 0 : uint32_t(s) < n + T) {
+                        // next PT slots of this unit that lie in the batch
+                        int32_t slot[PT]; int nt = 0;
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) slot[t] = 0;
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        const bool have = u < U ? s >= 0 : uint32_t(s) < n + T;
-                        if (have) {
+                        for (int t = 0; t < PT; ++t) slot[t] = int32_t(s0);
+                        while (nt < PT && (u < U ? s >= 0 : uint32_t(s) < n + T)) {
                             if (uint32_t(s) >= s0 && uint32_t(s) < s0 + sn) {
 #pragma unroll
-                                for (int q = 0; q < NT; ++q) if (q == nt) slot[q] = s;
+                                for (int q = 0; q < PT; ++q) if (q == nt) slot[q] = s;
                                 ++nt;
                             }
                             s = u < U ? next[s] : s + 1;
                         }
-                    }
-                    if (!nt) continue;
-                    const uint32_t row = rt * 16 + col;
-                    const uint4* codes = reinterpret_cast<const uint4*>(rec + off[6] + uint64_t(row) * (I / 2)) + G;
-                    const uint16_t* sr = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64) + (G >> 1);
-                    const uint16_t* br = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64) + (G >> 1);
-                    const uint8_t* img[NT]; LdsBf16 src[NT];
+                        if (!nt) break;
+                        const uint8_t* img[PT]; LdsBf16 src[PT];
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        const uint32_t q = t < nt ? uint32_t(slot[t]) - s0 : 0;
-                        img[t] = lds + lp.img_d + q * LI.bytes();
-                        src[t] = LdsBf16{reinterpret_cast<const uint16_t*>(lds + lp.ah) + q * I};
-                    }
-                    XintTile<NT> tile_state; tile_state.clear();
-#pragma unroll 4
-                    for (uint32_t dg = 0; dg < I / 128; ++dg)
-                        tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), img, LI, src, lane, nt);
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        if (t >= nt) break;
-                        const float v = bf(tile_state.finish(t));
-                        if (G == 0) otile[uint32_t(slot[t]) * 16 + col] = v;
+                        for (int t = 0; t < PT; ++t) { img[t] = lds + lp.img_d + (uint32_t(slot[t]) - s0) * LI.bytes(); src[t] = source_of(uint32_t(slot[t]) - s0); }
+                        auto emit = [&](int t, float v) { if (G == 0) otile[uint32_t(slot[t]) * 16 + col] = bf(v); };
+                        ZC_RUN_TILE(I / 128, w_row, s_row, b_row, I / 128, img, src, LI, lane, nt, emit);
                     }
                 }
             }
             __syncthreads();
+            clock();
             // weighted combine of the tile (reference: qwen.metal:804-816)
             if (tid < T * 16) {
                 const uint32_t t = tid / 16, c = tid % 16;
@@ -381,7 +398,9 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 if (c == 0) __hip_atomic_fetch_max(p.maxabs + layer * T + t, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+        clock();
         bar.wait();
+        clock();
     }
 }
 
@@ -418,20 +437,15 @@ hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt
         if (e != hipSuccess) return e;                                                                             \
         hipLaunchKernelGGL((decode_stack_kernel<NT>), dim3(workgroups), dim3(kDecodeThreads), lp.total, s, p, lp);  \
     } while (0)
-    if (nt == 1) ZC_DECODE(1); else if (nt == 2) ZC_DECODE(2); else if (nt == 4) ZC_DECODE(4); else ZC_DECODE(8);
+    if (nt == 1) ZC_DECODE(1); else ZC_DECODE(8);
 #undef ZC_DECODE
     return hipGetLastError();
 }
 hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu) {
-    const void* f = nt == 1 ? reinterpret_cast<const void*>(decode_stack_kernel<1>)
-                  : nt == 2 ? reinterpret_cast<const void*>(decode_stack_kernel<2>)
-                  : nt == 4 ? reinterpret_cast<const void*>(decode_stack_kernel<4>)
-                            : reinterpret_cast<const void*>(decode_stack_kernel<8>);
+    const void* f = nt == 1 ? reinterpret_cast<const void*>(decode_stack_kernel<1>) : reinterpret_cast<const void*>(decode_stack_kernel<8>);
     hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
     if (nt == 1) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<1>, kDecodeThreads, lds_bytes);
-    if (nt == 2) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<2>, kDecodeThreads, lds_bytes);
-    if (nt == 4) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<4>, kDecodeThreads, lds_bytes);
     return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<8>, kDecodeThreads, lds_bytes);
 }
 

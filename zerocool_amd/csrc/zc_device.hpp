@@ -59,6 +59,41 @@ __device__ __forceinline__ float lane_sum32(float v) {
     return v;
 }
 
+// Read-only data in device memory, addressed in the GLOBAL address space.  A pointer that
+// was itself loaded from memory is generic to the compiler; generic loads share the LDS
+// wait counter, so waiting for an LDS read would also wait for every weight prefetch.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <class T> using gptr = const T __attribute__((address_space(1)))*;
+template <class T> __device__ __forceinline__ gptr<T> as_global(const void* p) { return (gptr<T>)(uintptr_t)p; }
+__device__ __forceinline__ uint4 ldg_u4(const void* p, uint32_t index = 0) {
+    const u32x4 v = as_global<u32x4>(p)[index];
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint16_t ldg_u16(const void* p, uint32_t index = 0) { return as_global<uint16_t>(p)[index]; }
+__device__ __forceinline__ float ldg_f32(const void* p, uint32_t index = 0) { return as_global<float>(p)[index]; }
+
+// DPP moves inside rows of 16 lanes.  row_shr:1 hands lane i the value of lane i-1
+// (0 for the first lane of a row); the xor patterns are permutations.
+__device__ __forceinline__ float dpp_row_shr1(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));
+}
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// Maximum over the 64 lanes, returned in every lane: four DPP steps inside each row
+// (quad swaps, half mirror, mirror), then the four row values through scalar lanes.
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, dpp_f32<0xb1>(v));    // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_f32<0x4e>(v));    // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_f32<0x141>(v));   // row_half_mirror
+    v = fmaxf(v, dpp_f32<0x140>(v));   // row_mirror
+    const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
 // splitmix64 finaliser: the counter-based generator behind every synthetic tensor.
 __host__ __device__ inline uint64_t mix64(uint64_t z) {
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;

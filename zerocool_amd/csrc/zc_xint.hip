@@ -20,15 +20,19 @@ template <int NT, bool GATED>
 __device__ __forceinline__ void xint_rows(const XintJob& j, uint32_t tile, uint32_t t0, uint8_t* lds_base) {
     const XintLayout L{j.K};
     const uint32_t lane = threadIdx.x & 63u, col = lane & 15u, G = lane >> 4;
-    const uint8_t* lds[NT]; GlobalF32 xr[NT];
+    const uint8_t* lds[NT]; LdsF32 xr[NT];
+    float* xf = reinterpret_cast<float*>(lds_base + NT * L.bytes());   // fp32 copies of the rows
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const uint32_t tt = min(t0 + t, j.tokens - 1);
-        xr[t] = GlobalF32{j.x + uint64_t(j.in_rows ? uint32_t(j.in_rows[tt]) : tt) * j.K};
+        const float* row = j.x + uint64_t(j.in_rows ? uint32_t(j.in_rows[tt]) : tt) * j.K;
+        for (uint32_t i = threadIdx.x; i < j.K / 4; i += blockDim.x)
+            reinterpret_cast<float4*>(xf + t * j.K)[i] = reinterpret_cast<const float4*>(row)[i];
+        xr[t] = LdsF32{xf + t * j.K};
         lds[t] = lds_base + t * L.bytes();
-        xint_prepare(xr[t], L, lds_base + t * L.bytes());
     }
     __syncthreads();
+    xint_prepare_batch([&](uint32_t q) { return LdsF32{xf + q * j.K}; }, NT, L, lds_base);
     uint32_t row; const uint8_t* w; const uint16_t *s, *b;
     if (GATED) {
         row = tile * 8 + (col & 7u);
@@ -38,24 +42,17 @@ __device__ __forceinline__ void xint_rows(const XintJob& j, uint32_t tile, uint3
     }
     const bool valid = row < j.N;
     const uint32_t r = valid ? row : j.N - 1;
-    const uint4* codes = reinterpret_cast<const uint4*>(w + uint64_t(r) * (j.K / 2)) + G;
-    const uint16_t* sr = s + uint64_t(r) * (j.K / 64) + (G >> 1);
-    const uint16_t* br = b + uint64_t(r) * (j.K / 64) + (G >> 1);
-    XintTile<NT> tile_state; tile_state.clear();
-    const uint32_t spans = j.K / 128;
-#pragma unroll 4
-    for (uint32_t dg = 0; dg < spans; ++dg)
-        tile_state.step(dg, codes[dg * 4], b16(sr[2 * dg]), b16(br[2 * dg]), lds, L, xr, lane);
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        float v = tile_state.finish(t);
+    auto emit = [&](int t, float v) {
         if (GATED) {
             const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
             v = swiglu_bf(v, up);
         } else if (!j.float_output) v = bf(v);
         const bool writer = G == 0 && valid && (!GATED || col < 8) && t0 + t < j.tokens;
         if (writer) j.out[uint64_t(j.out_rows ? uint32_t(j.out_rows[t0 + t]) : t0 + t) * j.N + row] = v;
-    }
+    };
+    const uint8_t* w_row = w + uint64_t(r) * (j.K / 2);
+    if ((j.K / 128) % 8 == 0) xint_run_tile<NT, 8>(w_row, s + uint64_t(r) * (j.K / 64), b + uint64_t(r) * (j.K / 64), j.K / 128, lds, xr, L, lane, NT, emit);
+    else xint_run_tile<NT, 4>(w_row, s + uint64_t(r) * (j.K / 64), b + uint64_t(r) * (j.K / 64), j.K / 128, lds, xr, L, lane, NT, emit);
 }
 
 template <int NT, bool GATED>
@@ -81,7 +78,7 @@ void launch_affine_xint(hipStream_t s, const AffineDesc& a) {
     const uint32_t tiles = a.gated ? j.N / 8 : (j.N + 15) / 16;
     const uint32_t nt = a.tokens >= 4 ? 4 : a.tokens >= 2 ? 2 : 1;
     const dim3 grid((tiles + kXintWaves - 1) / kXintWaves, (a.tokens + nt - 1) / nt), block(64 * kXintWaves);
-    const size_t lds = size_t(L.bytes()) * nt;
+    const size_t lds = (size_t(L.bytes()) + size_t(j.K) * 4) * nt;
 #define ZC_GO(NT, GATED) hipLaunchKernelGGL((xint_op_kernel<NT, GATED>), grid, block, lds, s, j)
     if (a.gated) { if (nt == 4) ZC_GO(4, true); else if (nt == 2) ZC_GO(2, true); else ZC_GO(1, true); }
     else { if (nt == 4) ZC_GO(4, false); else if (nt == 2) ZC_GO(2, false); else ZC_GO(1, false); }

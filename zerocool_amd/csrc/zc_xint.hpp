@@ -41,162 +41,257 @@ __device__ __forceinline__ uint32_t xint_element_of_byte(uint32_t t) {
     return (t & 8u) + ((t & 3u) << 1) + ((t >> 2) & 1u);
 }
 
-// Loads with agent scope: inputs may have been written by another workgroup of a
-// persistent kernel, so they must not come from a stale cache line.
+// Loads with agent scope: data written by another workgroup of a persistent kernel must
+// not come from a stale cache line.
 __device__ __forceinline__ float load_shared_f32(const float* p) {
     return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
 
-// Input sources.  bits(k) returns the fp32 bit pattern of element k.
-struct GlobalF32 {   // a row in global memory, possibly written by another workgroup
-    const float* x;
-    __device__ __forceinline__ uint32_t bits(uint32_t k) const { return __float_as_uint(load_shared_f32(x + k)); }
-    __device__ __forceinline__ float at(uint32_t k) const { return load_shared_f32(x + k); }
-};
-struct LdsBf16 {     // a BF16 copy of the row in LDS
+// Input sources: a row staged in LDS.  block(b, out) gives the fp32 bit patterns of the
+// sixteen elements of block b.  kExactProducts: every element is BF16-valued, so x*q is
+// exact and a fused multiply-add equals the reference's separate multiply and add.
+struct LdsBf16 {     // BF16 copy of a BF16-valued row
+    static constexpr bool kExactProducts = true;
     const uint16_t* x;
-    __device__ __forceinline__ uint32_t bits(uint32_t k) const { return uint32_t(x[k]) << 16; }
-    __device__ __forceinline__ float at(uint32_t k) const { return b16(x[k]); }
+    __device__ __forceinline__ void block(uint32_t b, uint32_t* out) const {
+        const uint4 lo = *reinterpret_cast<const uint4*>(x + b * 16), hi = *reinterpret_cast<const uint4*>(x + b * 16 + 8);
+        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { out[2 * i] = w[i] << 16; out[2 * i + 1] = w[i] & 0xffff0000u; }
+    }
+};
+struct LdsF32 {      // fp32 copy of an arbitrary row
+    static constexpr bool kExactProducts = false;
+    const float* x;
+    __device__ __forceinline__ void block(uint32_t b, uint32_t* out) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(x + b * 16 + 4 * i);
+            out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+        }
+    }
 };
 
-// Builds the LDS image of a K-element row cooperatively (all threads of the workgroup
-// call it, then __syncthreads()).  One thread per block.
+// Builds one 16-block `b` of an image: digit planes, {2^e, bias sum}, unsafe bit.
+// The image's mask words must have been zeroed (xint_prepare_begin) before.
 template <class Source>
-__device__ __forceinline__ void xint_prepare(const Source x, const XintLayout L, uint8_t* lds) {
+__device__ __forceinline__ void xint_prepare_block(const Source x, const XintLayout L, uint8_t* lds, uint32_t b) {
     uint8_t* planes = lds;
     float2* info = reinterpret_cast<float2*>(lds + L.planes_bytes());
     uint32_t* mask = reinterpret_cast<uint32_t*>(lds + L.planes_bytes() + L.info_bytes());
-    for (uint32_t i = threadIdx.x; i < L.mask_bytes() / 4; i += blockDim.x) mask[i] = 0;
-    if (threadIdx.x < 4) reinterpret_cast<uint32_t*>(planes + L.blocks() * 48)[threadIdx.x] = 0;
-    __syncthreads();
-    for (uint32_t b = threadIdx.x; b < L.blocks(); b += blockDim.x) {
-        uint32_t bits[16];
+    uint32_t bits[16];
+    x.block(b, bits);
+    // bias sum: BF16 rounding after each addition of four inputs (reference: qwen.metal:55)
+    float sum = 0;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) bits[i] = x.bits(b * 16 + i);
-        // bias sum: BF16 rounding after each addition of four inputs (reference: qwen.metal:55)
-        float sum = 0;
+    for (int i = 0; i < 16; i += 4)
+        sum += bf(bf(bf(__uint_as_float(bits[i]) + __uint_as_float(bits[i + 1])) + __uint_as_float(bits[i + 2])) + __uint_as_float(bits[i + 3]));
+    uint32_t emin = 255, lowbits = 0, special = 0;
 #pragma unroll
-        for (int i = 0; i < 16; i += 4)
-            sum += bf(bf(bf(__uint_as_float(bits[i]) + __uint_as_float(bits[i + 1])) + __uint_as_float(bits[i + 2])) + __uint_as_float(bits[i + 3]));
-        uint32_t emin = 255, lowbits = 0, special = 0;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t e = (bits[i] >> 23) & 255u, m = bits[i] & 0x7fffffu;
-            lowbits |= bits[i] & 0xffffu;
-            special |= (e == 255u);
-            if (e | m) emin = min(emin, max(e, 1u));
-        }
-        if (emin == 255) emin = 1;   // all zero
-        uint32_t sumabs = 0, over = 0;
-        uint32_t mag[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t e = (bits[i] >> 23) & 255u;
-            const uint32_t sig = ((e ? 128u : 0u) | ((bits[i] >> 16) & 127u));
-            const uint32_t shift = max(e, 1u) - emin;
-            over |= (shift > 13u);
-            mag[i] = sig << min(shift, 13u);
-            sumabs += mag[i];
-        }
-        const bool safe = !lowbits && !special && !over && 15u * sumabs < (1u << 24);
-        uint32_t words[3][4] = {};
-#pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            const uint32_t i = xint_element_of_byte(t);
-            const uint32_t neg = bits[i] >> 31;
-#pragma unroll
-            for (int p = 0; p < 3; ++p) {
-                const uint32_t d = (mag[i] >> (7 * p)) & 127u;
-                const uint32_t byte = (neg ? (0u - d) : d) & 255u;
-                words[p][t / 4] |= byte << (8 * (t % 4));
-            }
-        }
-        if (!safe) { for (int p = 0; p < 3; ++p) for (int q = 0; q < 4; ++q) words[p][q] = 0; atomicOr(mask + b / 32, 1u << (b % 32)); }
-#pragma unroll
-        for (int p = 0; p < 3; ++p)
-            *reinterpret_cast<uint4*>(planes + b * 48 + p * 16) = make_uint4(words[p][0], words[p][1], words[p][2], words[p][3]);
-        // 2^(emin-134): x = sig * 2^(e-127-7)
-        const int ex = int(emin) - 134;
-        const float scale = ex >= -126 ? __uint_as_float(uint32_t(ex + 127) << 23) : __uint_as_float(1u << (ex + 149));
-        info[b] = make_float2(scale, sum);
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t e = (bits[i] >> 23) & 255u, m = bits[i] & 0x7fffffu;
+        lowbits |= bits[i] & 0xffffu;
+        special |= (e == 255u);
+        if (e | m) emin = min(emin, max(e, 1u));
     }
+    if (emin == 255) emin = 1;   // all zero
+    uint32_t sumabs = 0, over = 0;
+    uint32_t mag[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t e = (bits[i] >> 23) & 255u;
+        const uint32_t sig = ((e ? 128u : 0u) | ((bits[i] >> 16) & 127u));
+        const uint32_t shift = sig ? max(e, 1u) - emin : 0u;   // zeros put no demand on the range
+        over |= (shift > 13u);
+        mag[i] = sig << min(shift, 13u);
+        sumabs += mag[i];
+    }
+    const bool safe = !lowbits && !special && !over && 15u * sumabs < (1u << 24);
+    uint32_t words[3][4] = {};
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        const uint32_t i = xint_element_of_byte(t);
+        const uint32_t neg = bits[i] >> 31;
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            const uint32_t d = (mag[i] >> (7 * p)) & 127u;
+            const uint32_t byte = (neg ? (0u - d) : d) & 255u;
+            words[p][t / 4] |= byte << (8 * (t % 4));
+        }
+    }
+    if (!safe) { for (int p = 0; p < 3; ++p) for (int q = 0; q < 4; ++q) words[p][q] = 0; atomicOr(mask + b / 32, 1u << (b % 32)); }
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+        *reinterpret_cast<uint4*>(planes + b * 48 + p * 16) = make_uint4(words[p][0], words[p][1], words[p][2], words[p][3]);
+    // 2^(emin-134): x = sig * 2^(e-127-7)
+    const int ex = int(emin) - 134;
+    const float scale = ex >= -126 ? __uint_as_float(uint32_t(ex + 127) << 23) : __uint_as_float(1u << (ex + 149));
+    info[b] = make_float2(scale, sum);
+}
+// Clears the unsafe masks and zero slots of `count` consecutive images (stride L.bytes()).
+__device__ __forceinline__ void xint_prepare_begin(const XintLayout L, uint8_t* lds, uint32_t count) {
+    const uint32_t words = L.mask_bytes() / 4;
+    for (uint32_t i = threadIdx.x; i < count * words; i += blockDim.x)
+        reinterpret_cast<uint32_t*>(lds + (i / words) * L.bytes() + L.planes_bytes() + L.info_bytes())[i % words] = 0;
+    for (uint32_t i = threadIdx.x; i < count * 4; i += blockDim.x)
+        reinterpret_cast<uint32_t*>(lds + (i / 4) * L.bytes() + L.blocks() * 48)[i % 4] = 0;
+}
+// Builds `count` images cooperatively: all threads call it; source_of(q) gives image q's
+// input row.  Work is the flat list of (image, block) pairs.  Ends with a barrier.
+template <class SourceOf>
+__device__ __forceinline__ void xint_prepare_batch(const SourceOf source_of, uint32_t count, const XintLayout L, uint8_t* lds) {
+    xint_prepare_begin(L, lds, count);
+    __syncthreads();
+    const uint32_t blocks = L.blocks();
+    for (uint32_t i = threadIdx.x; i < count * blocks; i += blockDim.x) {
+        const uint32_t q = i / blocks;
+        xint_prepare_block(source_of(q), L, lds + q * L.bytes(), i % blocks);
+    }
+    __syncthreads();
 }
 
-// The literal fp32 chain of one block (reference: qwen.metal:52-57) for a lane that
-// holds the block's two code words.
+// The literal fp32 chain of one block (reference: qwen.metal:52-57) from the block's
+// expanded code bytes (MFMA byte order: element of byte t is xint_element_of_byte(t)).
 template <class Source>
-__device__ __forceinline__ float xint_literal_dot(uint32_t w0, uint32_t w1, const Source x, uint32_t k0) {
+__device__ __forceinline__ float xint_literal_dot(const v4i codes, const Source x, uint32_t block) {
+    uint32_t xb[16];
+    x.block(block, xb);
+    float q[16];   // q[element]
+#pragma unroll
+    for (int t = 0; t < 16; ++t) q[(t & 8) + ((t & 3) << 1) + ((t >> 2) & 1)] = float((uint32_t(codes[t / 4]) >> (8 * (t % 4))) & 255u);
     float dot = 0;
 #pragma unroll
     for (int i = 0; i < 16; i += 4) {
-        const uint32_t packed = ((i < 8 ? w0 : w1) >> (4 * (i % 8))) & 0xffffu;
-        dot += x.at(k0 + i) * float(packed & 15u) + x.at(k0 + i + 1) * float((packed >> 4) & 15u) +
-               x.at(k0 + i + 2) * float((packed >> 8) & 15u) + x.at(k0 + i + 3) * float((packed >> 12) & 15u);
+        const float a = __uint_as_float(xb[i]), c = __uint_as_float(xb[i + 1]), d = __uint_as_float(xb[i + 2]), e = __uint_as_float(xb[i + 3]);
+        if constexpr (Source::kExactProducts)
+            dot += __builtin_fmaf(e, q[i + 3], __builtin_fmaf(d, q[i + 2], __builtin_fmaf(c, q[i + 1], a * q[i])));
+        else
+            dot += a * q[i] + c * q[i + 1] + d * q[i + 2] + e * q[i + 3];
     }
     return dot;
 }
 
-// Per-lane state of one 16-row tile: lane = (j = row in tile, G = lane / 16).
-// Processes NT tokens at once; acc[t][m][h] is the running sum of reference lane
-// 8*m + 2*G + h of row j.
-template <int NT>
-struct XintTile {
-    float acc[NT][4][2];
-    __device__ __forceinline__ void clear() {
+// Runs a whole 16-column tile for nt <= PT tokens and hands each finished row sum to
+// emit(t, sum).  lane = (j = column, G = lane / 16); acc[t][m][h] is the running sum of
+// reference lane 8*m + 2*G + h of the column's row.
+//
+// Weights stream through a ring of R spans (128 elements each) per lane: R sixteen-byte
+// code loads plus the matching scale / bias dwords (dword d of a row's vector holds
+// groups 2d, 2d+1) are in flight while earlier spans are multiplied.  Each ring body is
+// three straight-line passes so the scheduler can overlap LDS reads, MFMAs and VALU work:
+//   1. every span: A operands from LDS, two MFMAs, digit sums -> fp32 block dots
+//   2. only if some block of the body is unsafe: those dots again by the literal chain
+//   3. every span: acc += scale*dot + sum*bias, in span order
+template <int PT, int R, class Source, class Emit>
+__device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                              const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,
+                                              int nt, Emit emit) {
+    static_assert(R == 8 || R == 4, "bodies of eight or four spans; spans must be a multiple of R");
+    const uint32_t G = lane >> 4, row_a = lane & 15u, c_a = row_a >> 2, p_a = row_a & 3u;
+    const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
+    uint4 ring[R], sring[R / 4], bring[R / 4];
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
 #pragma unroll
-            for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
-    }
-    // One 128-element span `dg` of the row: codes = the lane's 16 bytes (blocks 2G, 2G+1),
-    // scale/bias = the row's group values for group 2*dg + G/2.
-    // nt <= NT tokens are live (wave-uniform); lds[t] / x[t] are token t's image and source.
-    template <class Source>
-    __device__ __forceinline__ void step(uint32_t dg, const uint4 codes, float scale, float bias, const uint8_t* const* lds,
-                                         const XintLayout L, const Source* x, uint32_t lane, int nt = NT) {
-        const uint32_t G = lane >> 4, i = lane & 15u, c = i >> 2, p = i & 3u;
-        const uint32_t M = 0x0f0f0f0fu;
-        v4i b0 = {int(codes.x & M), int((codes.x >> 4) & M), int(codes.y & M), int((codes.y >> 4) & M)};
-        v4i b1 = {int(codes.z & M), int((codes.z >> 4) & M), int(codes.w & M), int((codes.w >> 4) & M)};
-        const uint32_t blk = 8 * dg + 2 * G;                 // this lane's result blocks: blk, blk+1
-        const uint32_t ablk = 8 * dg + 2 * (c == G ? G : 0); // A rows: plane p of block 2c(+h) in lane group c
-        const bool live = (c == G) && p < 3;
-        const uint32_t zero_slot = L.blocks() * 48;
+    for (int q = 0; q < R / 4; ++q) { sring[q] = ldg_u4(s_row, q); bring[q] = ldg_u4(b_row, q); }
+    float acc[PT][4][2];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
+    for (int t = 0; t < PT; ++t)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
+    const uint32_t shamt = (lane & 32u) ? 0u : 16u;   // group 2d + (G >> 1): low half for G < 2
+    // A operand: row (c,p) of lane group G holds digit plane p of block 2c (+1) when c == G, zeros otherwise
+    const bool live = (c_a == G) && p_a < 3;
+    const uint32_t a_first = live ? 2 * G * 48 + p_a * 16 : L.blocks() * 48, a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
+    const uint32_t M = 0x0f0f0f0fu;
+    const v4i zero = {0, 0, 0, 0};
+    auto expand = [&](uint32_t lo, uint32_t hi) { const v4i r = {int(lo & M), int((lo >> 4) & M), int(hi & M), int((hi >> 4) & M)}; return r; };
+    for (uint32_t d0 = 0; d0 < spans; d0 += R) {
+        uint4 codes[R]; uint32_t sd[R], bd[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            codes[j] = ring[j];
+            const uint4 sq = sring[j / 4], bq = bring[j / 4];
+            sd[j] = (j % 4 == 0) ? sq.x : (j % 4 == 1) ? sq.y : (j % 4 == 2) ? sq.z : sq.w;
+            bd[j] = (j % 4 == 0) ? bq.x : (j % 4 == 1) ? bq.y : (j % 4 == 2) ? bq.z : bq.w;
+        }
+        if (d0 + R < spans) {
+#pragma unroll
+            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
+#pragma unroll
+            for (int q = 0; q < R / 4; ++q) { sring[q] = ldg_u4(s_row, (d0 + R) / 4 + q); bring[q] = ldg_u4(b_row, (d0 + R) / 4 + q); }
+        }
+#pragma unroll
+        for (int t = 0; t < PT; ++t) {
             if (t >= nt) break;
-            const uint8_t* planes = lds[t];
+            const uint8_t* planes = img[t];
             const float2* info = reinterpret_cast<const float2*>(planes + L.planes_bytes());
             const uint32_t* mask = reinterpret_cast<const uint32_t*>(planes + L.planes_bytes() + L.info_bytes());
-            const v4i a0 = *reinterpret_cast<const v4i*>(planes + (live ? ablk * 48 + p * 16 : zero_slot));
-            const v4i a1 = *reinterpret_cast<const v4i*>(planes + (live ? (ablk + 1) * 48 + p * 16 : zero_slot));
-            const v4i z = {0, 0, 0, 0};
-            const v4i d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, z, 0, 0, 0);
-            const v4i d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, z, 0, 0, 0);
-            const uint32_t unsafe = (mask[blk / 32] >> (blk % 32)) & 3u;
+            float dot[R][2], bsum[R][2];
+            // pass 1
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const v4i d = h ? d1 : d0;
-                const float2 fi = info[blk + h];
-                float dot = float(d[0] + (d[1] << 7) + (d[2] << 14)) * fi.x;
-                if (unsafe & (1u << h)) dot = xint_literal_dot(h ? codes.z : codes.x, h ? codes.w : codes.y, x[t], (blk + h) * 16);
-                acc[t][dg & 3u][h] += scale * dot + fi.y * bias;
+            for (int j = 0; j < R; ++j) {
+                const uint32_t d = d0 + j;
+                {
+                    const v4i b0 = expand(codes[j].x, codes[j].y), b1 = expand(codes[j].z, codes[j].w);
+                    const uint8_t* a_at = planes + a_first + d * a_span;
+                    const v4i a0 = *reinterpret_cast<const v4i*>(a_at), a1 = *reinterpret_cast<const v4i*>(a_at + a_next);
+#ifdef ZC_PROBE_NO_MFMA
+                    const v4i r0 = a0 + b0 + zero, r1 = a1 + b1;
+#else
+                    const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
+                    const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, zero, 0, 0, 0);
+#endif
+                    const float4 fi = *reinterpret_cast<const float4*>(info + 8 * d + 2 * G);   // {2^e, sum} of blocks 2G, 2G+1
+                    dot[j][0] = float(r0[0] + (r0[1] << 7) + (r0[2] << 14)) * fi.x; bsum[j][0] = fi.y;
+                    dot[j][1] = float(r1[0] + (r1[1] << 7) + (r1[2] << 14)) * fi.z; bsum[j][1] = fi.w;
+                }
+            }
+            // pass 2: blocks 8d + 2G + h of spans d0 .. d0+7 sit in mask words d0/4, d0/4 + 1
+            const uint32_t mine = 0x03030303u << (2 * G);
+            const uint32_t u0 = mask[d0 / 4] & mine, u1 = R == 8 ? mask[d0 / 4 + 1] & mine : 0u;
+#ifdef ZC_PROBE_NO_FALLBACK
+            if (false) {
+#else
+            if (__builtin_expect(__ballot((u0 | u1) != 0) != 0, 0)) {
+#endif
+#pragma unroll
+                for (int j = 0; j < R; ++j) {
+                    const uint32_t d = d0 + j;
+                    {
+                        const uint32_t bits = ((j < 4 ? u0 : u1) >> (8 * (j % 4) + 2 * G)) & 3u;
+                        if (bits & 1u) dot[j][0] = xint_literal_dot(expand(codes[j].x, codes[j].y), src[t], 8 * d + 2 * G);
+                        if (bits & 2u) dot[j][1] = xint_literal_dot(expand(codes[j].z, codes[j].w), src[t], 8 * d + 2 * G + 1);
+                    }
+                }
+            }
+            // pass 3
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                {
+                    const float scale = __uint_as_float((sd[j] << shamt) & 0xffff0000u), bias = __uint_as_float((bd[j] << shamt) & 0xffff0000u);
+                    acc[t][j & 3][0] += scale * dot[j][0] + bsum[j][0] * bias;
+                    acc[t][j & 3][1] += scale * dot[j][1] + bsum[j][1] * bias;
+                }
             }
         }
     }
-    // Reference lane sum (xor butterfly 16, 8, 4, 2, 1) of token t; every lane of row j returns it.
-    __device__ __forceinline__ float finish(int t) const {
+    // Reference lane sum (xor butterfly 16, 8, 4, 2, 1): strides 16 and 8 pair accumulators,
+    // 4 and 2 pair lane groups, 1 pairs the two blocks of a lane.
+#pragma unroll
+    for (int t = 0; t < PT; ++t) {
+        if (t >= nt) break;
         float v[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const float a0 = acc[t][0][h] + acc[t][2][h], a1 = acc[t][1][h] + acc[t][3][h];   // stride 16
-            float s = a0 + a1;                                                                    // stride 8
-            s = s + __shfl_xor(s, 32);                                                            // stride 4
-            s = s + __shfl_xor(s, 16);                                                            // stride 2
-            v[h] = s;
+            const float a0 = acc[t][0][h] + acc[t][2][h], a1 = acc[t][1][h] + acc[t][3][h];
+            float sum = a0 + a1;
+            sum = sum + __shfl_xor(sum, 32);
+            sum = sum + __shfl_xor(sum, 16);
+            v[h] = sum;
         }
-        return v[0] + v[1];                                                                       // stride 1
+        emit(t, v[0] + v[1]);
     }
-};
+}
 
 }  // namespace zc

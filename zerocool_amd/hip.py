@@ -34,7 +34,7 @@ class Layer(C.Structure):
 
 
 class StackTrace(C.Structure):
-    _fields_ = [(n, C.c_void_p) for n in ("ids", "weights", "outputs")]
+    _fields_ = [(n, C.c_void_p) for n in ("ids", "weights", "outputs", "clocks")]
 
 
 class Trace(C.Structure):
@@ -131,6 +131,14 @@ class Context:
         b = into or self.alloc(max(a.nbytes, 4))
         self._call("zc_hip_upload", _ptr(b), a.ctypes.data_as(C.c_void_p), C.c_uint64(a.nbytes))
         return b
+
+    def timer_start(self):
+        self._call("zc_hip_timer_start")
+
+    def timer_stop(self):
+        ms = C.c_float()
+        self._call("zc_hip_timer_stop", C.byref(ms))
+        return ms.value
 
     def configure(self, affine_policy):
         """0: literal lane kernels everywhere; 1 (default): exact-integer matrix-core kernels where the shape allows."""

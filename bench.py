@@ -1,0 +1,125 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the MoE-layer path on one MI355X.
+
+Workload (BASELINE.json configs[4]): decode through a 48-layer MoE stack at the stand-in
+scale -- hidden 3072, 512 experts, top-10, expert intermediate 1024, affine Q4 group 64,
+about 130 GB of expert records resident in HBM -- at decode batch 1.  Every layer's router
+has its own seed and Zipf(1.1)-skewed expert offsets.  A step is one token batch through
+all 48 layers: ONE launch of the persistent decode kernel.  Inputs are resident in HBM
+before the timed region; timing uses HIP events on the stream the kernel runs on.
+
+Prints one JSON line.  `roofline.achieved` = algorithmic bytes of one launch (router +
+shared gate + distinct routed records + shared record + activations, summed over the 48
+layers) / average launch duration.  `cpu_baseline` = the CPU oracle (a restatement of the
+reference arithmetic; the reference has no CPU path of its own) on a bounded sample of the
+same workload, on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=48)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--extra", action="store_true", help="also time decode batch 8 and the single-layer configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
+              "(DESIGN.md describes how it would shard by expert)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import zerocool_amd as z
+    from zerocool_amd import workload
+
+    ctx = z.Context(0)
+    cfg = workload.config("F")
+    L, T = args.layers, args.batch
+    layers = [workload.LayerWeights(ctx, cfg, workload.BASE_SEED + 4 * 1000 + l, ("zipf", 1.1)) for l in range(L)]
+    ctx.finish()
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], max(T, 8))
+
+    def run(tokens, steps, warmup):
+        x = workload.hidden_rows(ctx, tokens, cfg.hidden, workload.BASE_SEED + 4 * 7 + tokens)
+        out = ctx.alloc(tokens * cfg.hidden * 4)
+        n = tokens * cfg.topk
+        ids, w = ctx.alloc(L * n * 4), ctx.alloc(L * n * 4)
+        ctx.stack_decode(stack, x, tokens, out, z.StackTrace(ids.ptr, w.ptr, None, None))
+        ctx.moe_check()
+        unique = [len(np.unique(r)) for r in ids.numpy(np.int32).reshape(L, n)]
+        nbytes = sum(workload.layer_bytes(cfg, u, tokens, ctx) for u in unique)
+        for _ in range(warmup):
+            ctx.stack_decode(stack, x, tokens, out)
+        ctx.finish()
+        ctx.timer_start()
+        for _ in range(steps):
+            ctx.stack_decode(stack, x, tokens, out)
+        ms = ctx.timer_stop() / steps
+        ctx.moe_check()
+        for b in (x, out, ids, w):
+            ctx.free(b)
+        return ms, nbytes, unique
+
+    ms, nbytes, unique = run(T, args.steps, args.warmup)
+    persistent = ctx.stack_is_persistent(stack, T)
+    achieved = nbytes / (ms * 1e-3) / 1e9
+    result = {
+        "metric": "moe_decode_tokens_per_s", "value": T / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u4 codes x bf16 inputs, fp32 accumulation",
+        "data": "synthetic (counter-based generator, seeded; random-init weights of the named shape)",
+        "config": {"workload": "BASELINE configs[4]: 48-layer MoE stack decode, hidden 3072, 512 experts, top-10, "
+                               "intermediate 1024, affine Q4 group 64, ~130 GB of expert records resident in HBM, "
+                               "Zipf(1.1) router offsets, one seed per layer",
+                   "layers": L, "decode_batch": T, "hbm_resident_bytes": int(ctx.allocated),
+                   "distinct_experts_per_layer": float(np.mean(unique)),
+                   "path": "persistent single-launch kernel" if persistent else "layer by layer"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s", "frac": achieved / 8000.0,
+                     "traffic": None, "kernel": "zc::decode_stack_kernel (one launch = one step)",
+                     "algorithmic_bytes_per_launch": int(nbytes), "launch_us": ms * 1e3},
+    }
+
+    if args.extra:
+        extra = {}
+        ms8, b8, u8 = run(8, max(5, args.steps // 4), 2)
+        extra["stack_batch8"] = {"tokens_per_s": 8 / (ms8 * 1e-3), "ms_per_step": ms8, "GBps": b8 / (ms8 * 1e-3) / 1e9,
+                                 "distinct_experts_per_layer": float(np.mean(u8))}
+        result["extra"] = extra
+
+    if not args.no_cpu:
+        import oracle
+        sample_layers = 2
+        threads = min(os.cpu_count() or 1, 16)
+        ocfg = oracle.Config(*[getattr(cfg, n) for n, _ in z.Config._fields_])
+        x = workload.hidden_rows(ctx, T, cfg.hidden, workload.BASE_SEED + 4 * 7 + T).numpy(np.float32)
+        hosts = [layers[l].host() for l in range(sample_layers)]
+        def cpu_pass():
+            cur = x.reshape(T, cfg.hidden)
+            for h in hosts:
+                cur = oracle.moe_layer(ocfg, h["router"], h["shared_gate"], h["shared_record"], h["records"], h["stride"],
+                                       cur, T, router_offsets=h["offsets"], threads=threads)
+        cpu_pass()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 10 and reps < 200):
+            cpu_pass(); reps += 1
+        per_layer = (time.perf_counter() - t0) / reps / sample_layers
+        result["cpu_baseline"] = {"value": T / (per_layer * L), "unit": "tokens/s", "cores": threads, "kind": "port",
+                                  "sample": f"{sample_layers} of {L} layers x {reps} repetitions at batch {T}, per-layer mean "
+                                            f"extrapolated to {L} layers (the CPU oracle, OpenMP over output rows)",
+                                  "ms_per_layer": per_layer * 1e3}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

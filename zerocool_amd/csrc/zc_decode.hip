@@ -62,6 +62,34 @@ struct Barrier {
     }
 };
 
+// Copies `pairs` pairs of fp32 values written by other workgroups into LDS as BF16 (high
+// halves), eight coherent 8-byte loads in flight per thread; returns whether any value
+// had low mantissa bits.  transform(pair index, a, b) may rescale the two values first.
+template <class Transform>
+__device__ __forceinline__ int stage_bf16(const float* src, uint32_t pairs, uint32_t* dst, Transform transform) {
+    int inexact = 0;
+    for (uint32_t base = 0; base < pairs; base += blockDim.x * 8) {
+        uint64_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint32_t i = base + u * blockDim.x + threadIdx.x;
+            v[u] = i < pairs ? __hip_atomic_load(reinterpret_cast<const uint64_t*>(src) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint32_t i = base + u * blockDim.x + threadIdx.x;
+            if (i < pairs) {
+                float a = __uint_as_float(uint32_t(v[u])), b = __uint_as_float(uint32_t(v[u] >> 32));
+                transform(i, a, b);
+                const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+                inexact |= ((ua | ub) & 0xffffu) != 0;
+                dst[i] = (ua >> 16) | (ub & 0xffff0000u);
+            }
+        }
+    }
+    return inexact;
+}
+
 // Top-k of one token by one wavefront.  Lane l holds experts l*per .. l*per+per-1, so the
 // lowest lane holding the maximum, then the lowest slot inside it, is the lowest expert id:
 // one DPP maximum, one ballot and two scalar-lane reads per pick.
@@ -161,14 +189,10 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
             }
             __syncthreads();
-            int bad = 0;
-            for (uint32_t i = tid; i < T * H; i += blockDim.x) {
-                float v = load_shared_f32((layer ? p.layer_out : p.x_in) + i);
-                if (layer) v = bf(v * gatev[i / H]);
-                const uint32_t u = __float_as_uint(v);
-                bad |= (u & 0xffffu) != 0;
-                xh[i] = uint16_t(u >> 16);
-            }
+            const bool glue = layer != 0;
+            const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), [&](uint32_t i, float& a, float& b) {
+                if (glue) { const float inv = gatev[(2 * i) / H]; a = bf(a * inv); b = bf(b * inv); }
+            });
             if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
         }
         __syncthreads();
@@ -329,11 +353,11 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 const uint32_t sn = min(SB, slots_total - s0);
                 __syncthreads();
                 uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
-                for (uint32_t i = tid; i < sn * I / 2; i += blockDim.x) {   // two activations per coherent 8-byte read
-                    const uint32_t sl = s0 + (2 * i) / I, kk = (2 * i) % I;
-                    const float* a = sl < n ? p.act + uint64_t(sl) * I : p.shared_act + uint64_t(sl - n) * I;
-                    const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(a + kk), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    reinterpret_cast<uint32_t*>(ah)[i] = (uint32_t(v) >> 16) | (uint32_t(v >> 32) & 0xffff0000u);
+                {   // rows s0 .. s0+sn-1 of [act ; shared_act]: contiguous except across the seam between the two buffers
+                    const uint32_t routed = s0 < n ? min(sn, n - s0) : 0;
+                    if (routed) stage_bf16(p.act + uint64_t(s0) * I, routed * I / 2, reinterpret_cast<uint32_t*>(ah), [](uint32_t, float&, float&) {});
+                    if (sn > routed) stage_bf16(p.shared_act + uint64_t(s0 + routed - n) * I, (sn - routed) * I / 2,
+                                                reinterpret_cast<uint32_t*>(ah + routed * I), [](uint32_t, float&, float&) {});
                 }
                 __syncthreads();
                 auto source_of = [&](uint32_t q) { return LdsBf16{ah + q * I}; };

@@ -6,7 +6,7 @@
 // partial sums of a block fit 24 bits the whole chain is exact: `dot` then equals the
 // true sum, whatever the order.  Such a block is computed here in integers:
 //   x_k = X_k * 2^e   (e = smallest exponent in the block, X_k integer, |X_k| < 2^21)
-//   X_k = d0 + 2^7 d1 + 2^14 d2  (signed 7-bit digits, sign of x_k)
+//   X_k = d0 + 2^7 d1 + 2^14 d2  (two's-complement digits: d0, d1 in [0,127], d2 signed)
 //   dot = float(sum_k X_k q_k) * 2^e,  sum_k X_k q_k from three int8 MFMA rows.
 // A block is "safe" when 15 * sum_k |X_k| < 2^24 and every x_k is BF16-valued; any
 // other block takes the literal fp32 chain.  Per-block terms are then combined in the
@@ -107,17 +107,16 @@ __device__ __forceinline__ void xint_prepare_block(const Source x, const XintLay
         sumabs += mag[i];
     }
     const bool safe = !lowbits && !special && !over && 15u * sumabs < (1u << 24);
+    // digits of the signed integer Xs in two's complement: Xs = d0 + 2^7 d1 + 2^14 d2 with
+    // d0, d1 in [0,127] and d2 = Xs >> 14 in [-128,127] (|Xs| < 2^21)
     uint32_t words[3][4] = {};
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
         const uint32_t i = xint_element_of_byte(t);
-        const uint32_t neg = bits[i] >> 31;
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-            const uint32_t d = (mag[i] >> (7 * p)) & 127u;
-            const uint32_t byte = (neg ? (0u - d) : d) & 255u;
-            words[p][t / 4] |= byte << (8 * (t % 4));
-        }
+        const int32_t xs = (bits[i] >> 31) ? -int32_t(mag[i]) : int32_t(mag[i]);
+        words[0][t / 4] |= (uint32_t(xs) & 127u) << (8 * (t % 4));
+        words[1][t / 4] |= ((uint32_t(xs) >> 7) & 127u) << (8 * (t % 4));
+        words[2][t / 4] |= ((uint32_t(xs) >> 14) & 255u) << (8 * (t % 4));
     }
     if (!safe) { for (int p = 0; p < 3; ++p) for (int q = 0; q < 4; ++q) words[p][q] = 0; atomicOr(mask + b / 32, 1u << (b % 32)); }
 #pragma unroll

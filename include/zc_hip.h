@@ -68,6 +68,10 @@ zc_status zc_hip_destroy(zc_hip_ctx* ctx);
 /* Metal::allocate / zeros / upload (metal.hpp:61-65); download stands in for reading Buffer::data. */
 zc_status zc_hip_alloc(zc_hip_ctx* ctx, uint64_t bytes, void** out);
 zc_status zc_hip_free(zc_hip_ctx* ctx, void* ptr);
+/* Host-visible allocation (pinned, mapped into the device's address space, coherent): the
+ * stand-in for the reference's unified-memory Buffer::data (storage.hpp:54-63).  The same
+ * pointer is valid on the host and in kernels; meant for activations and small tensors. */
+zc_status zc_hip_alloc_host(zc_hip_ctx* ctx, uint64_t bytes, void** out);
 zc_status zc_hip_memset(zc_hip_ctx* ctx, void* dst, int byte, uint64_t bytes);
 zc_status zc_hip_upload(zc_hip_ctx* ctx, void* dst, const void* host_src, uint64_t bytes);
 zc_status zc_hip_download(zc_hip_ctx* ctx, void* host_dst, const void* src, uint64_t bytes);
@@ -164,9 +168,9 @@ typedef struct {       /* optional device buffers, any may be NULL */
     int32_t* ids;      /* [n_layers][tokens][topk] */
     float* weights;    /* [n_layers][tokens][topk] */
     float* outputs;    /* [n_layers][tokens][hidden] layer outputs before the glue */
-    uint64_t* clocks;  /* [n_layers][10] timestamps (100 MHz) of the persistent kernel's workgroup 0 at
-                          layer start, images built, phase R done, barrier 1, routed, phase G done,
-                          barrier 2, phase D done, barrier 3 (tuning aid; persistent path only) */
+    uint64_t* clocks;  /* [n_layers * 15][workgroups] timestamps (100 MHz) that every workgroup of the
+                          persistent kernel takes at its phase boundaries, 15 per layer (tuning aid;
+                          persistent path only; workgroups = compute units of the device) */
 } zc_stack_trace;
 zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
                               uint32_t n_layers, uint32_t max_tokens, zc_hip_stack** out);

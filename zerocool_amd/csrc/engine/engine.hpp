@@ -1,0 +1,134 @@
+// Host side of the MI355X MoE path in the reference's own vocabulary.
+//
+// The types and signatures below mirror the operator interface the reference's
+// Model::moe is written against (include/engine/storage.hpp:54-63, include/engine/metal.hpp:6-13,
+// 48-140, 154; include/engine/pipeline.hpp:6-8; include/engine/model.hpp:156), so that code
+// written against that interface -- the body of Model::moe, encode_expert_rows, the reference's
+// own tests of them -- compiles against this header unchanged apart from the shapes, which
+// the reference fixes at compile time (storage.hpp:26-27) and this path takes from a MoeShape.
+// Every method only forwards to the C ABI (include/zc_hip.h); there is no arithmetic here.
+//
+// Memory: the reference runs on unified memory where Buffer::data is CPU-visible.  Here
+// Temporary / State / Workspace / Snapshot buffers are pinned host allocations mapped into
+// the GPU (same pointer on both sides, readable after finish()); Resident / Expert buffers
+// live in HBM (data == nullptr, filled with Metal::write).
+#pragma once
+#include <atomic>
+#include <cstddef>
+#include <cstdint>
+#include <functional>
+#include <initializer_list>
+#include <memory>
+#include <span>
+#include <string>
+#include <vector>
+#include "../../../include/zc_hip.h"
+
+namespace zerocool::engine {
+
+uint64_t checked_add(uint64_t a, uint64_t b);
+uint64_t checked_mul(uint64_t a, uint64_t b);
+float bf16(uint16_t value);
+float round_bf16(float value);
+
+// storage.hpp:54-63
+struct Buffer {
+    uint64_t bytes = 0;
+    std::byte* data = nullptr;     // CPU-visible contents, or nullptr for HBM-only buffers
+    std::shared_ptr<void> owner;
+    void* metal = nullptr;         // the device address (the reference's id<MTLBuffer>)
+    static std::shared_ptr<Buffer> host(uint64_t bytes);
+    std::span<float> floats() const;
+};
+using Buf = std::shared_ptr<Buffer>;
+using Allocator = std::function<Buf(uint64_t)>;
+
+// metal.hpp:6-13
+struct Binding { Buf buffer; uint64_t offset = 0; };
+enum class AllocationClass { Temporary, Resident, State, Expert, Snapshot, Workspace };
+struct Linear {
+    Binding weight, scales, biases;
+    uint32_t input = 0, output = 0, group = 64, dtype = 0;
+    bool quantized = false;
+    uint32_t bits = 4;
+};
+// metal.hpp:17-43, the part that concerns this path
+struct KernelConfig {
+    std::string policy = "exact-int";   // "reference": literal lane kernels everywhere
+    void validate() const;
+};
+
+// The shapes storage.hpp:26-27 fixes for the reference's model.
+struct MoeShape {
+    uint32_t hidden = 2560, experts = 512, topk = 10, inter = 640, group = 64;
+    uint32_t bits_gate_up = 4, bits_down = 4, shared_bits_gate_up = 4, shared_bits_down = 4;
+    zc_moe_config abi() const;
+    uint64_t expert_bytes(bool shared = false) const;   // storage.hpp:32
+};
+
+// metal.hpp:48-140, the methods Model::moe and encode_expert_rows use
+class Metal {
+public:
+    struct Completion { std::atomic<bool> done{false}; uint64_t ticket = 0; std::string error; };
+    explicit Metal(MoeShape shape = {}, int device = 0);
+    ~Metal();
+    Metal(const Metal&) = delete;
+    Metal& operator=(const Metal&) = delete;
+    const MoeShape& shape() const { return shape_; }
+    Buf allocate(uint64_t bytes);
+    Buf allocate(uint64_t bytes, AllocationClass kind);
+    Buf zeros(uint64_t floats);
+    Buf zeros(uint64_t floats, AllocationClass kind);
+    Buf upload(std::span<const float> values);
+    void write(const Buf& destination, uint64_t offset, std::span<const std::byte> bytes);   // fills an HBM buffer
+    void read(const Buf& source, uint64_t offset, std::span<std::byte> bytes);              // drains, then copies out
+    void copy(const Buf& source, uint64_t source_offset, const Buf& destination, uint64_t destination_offset, uint64_t bytes);
+    Buf slice(const Buf& source, uint64_t offset, uint64_t bytes);
+    void budget(uint64_t bytes);
+    void configure(KernelConfig config);
+    bool direct_rows() const { return true; }
+    void label(std::string, int = -1, uint32_t = 0, uint32_t = 0, std::span<const uint32_t> = {}) {}
+    // "moe_sum" and "scatter_experts" are the two kernels the path dispatches by name (model.cpp:555, pipeline.cpp:28)
+    void dispatch(const std::string& name, std::initializer_list<Binding> buffers, std::initializer_list<uint32_t> params,
+                  uint32_t x, uint32_t y = 1, uint32_t z = 1, uint32_t tx = 32, uint32_t ty = 1, uint32_t tz = 1);
+    std::shared_ptr<Completion> submit();
+    void wait(const std::shared_ptr<Completion>& completion);
+    void reap() {}
+    void finish();
+    Buf linear(const Linear& layer, const Buf& x, uint32_t tokens, bool float_output = false);
+    void linear_into(const Linear& layer, const Buf& x, uint32_t tokens, Binding output, bool float_output = false);
+    void grouped_experts(std::span<const Buf> records, std::span<const uint32_t> positions, const Buf& x, const Buf& output, const Buf& scratch);
+    Buf gated_linear(const Linear& gate, const Linear& up, const Buf& x, uint32_t tokens, const Buf& rows = {});
+    void route(const Buf& logits, const Buf& ids, const Buf& weights, uint32_t tokens);
+    uint64_t allocated() const;
+    uint64_t peak() const;
+    std::string device_name() const;
+    zc_hip_ctx* context() const { return ctx_; }
+private:
+    MoeShape shape_;
+    zc_hip_ctx* ctx_ = nullptr;
+    uint64_t budget_ = 0;
+};
+// metal.hpp:154, metal.mm:1124-1129
+Linear expert_linear(const MoeShape& shape, const Buf& record, int projection, bool shared = false);
+
+// pipeline.hpp:6-8, pipeline.cpp:7-31
+void encode_expert_rows(Metal& gpu, const Buf& record, const Buf& input, const Buf& output, std::span<const int> positions,
+                        uint32_t tokens, uint32_t chunk, bool direct, int layer, uint32_t offset,
+                        const std::atomic<bool>* cancel = nullptr);
+
+// What Model::moe reads through Resident and the expert store for one layer.
+struct MoeLayerWeights {
+    Linear router;            // [experts][hidden] BF16, float output (model.cpp:434)
+    Linear shared_gate;       // [1][hidden] BF16 (model.cpp:485)
+    Buf shared_record;        // gate, up, down of the shared expert
+    std::function<Buf(uint32_t expert)> record;   // the expert store: record of a routed expert
+};
+// model.hpp:156, model.cpp:431-557: the reference's orchestration, one CPU readback of the ids per call.
+Buf moe(Metal& gpu, const MoeLayerWeights& weights, const Buf& x, uint32_t tokens,
+        const std::atomic<bool>* cancel = nullptr, uint32_t chunk = 128);
+// The same layer as one enqueue with routing and dispatch kept on the device (zc_hip_moe_forward);
+// records must be one buffer of experts * stride bytes.
+Buf moe_resident(Metal& gpu, const MoeLayerWeights& weights, const Buf& records, uint64_t stride, const Buf& x, uint32_t tokens);
+
+}  // namespace zerocool::engine

@@ -34,6 +34,7 @@ struct zc_hip_ctx {
     hipStream_t stream = nullptr;
     uint64_t budget = 0, allocated = 0, peak = 0;
     std::unordered_map<void*, uint64_t> blocks;
+    std::unordered_map<void*, uint64_t> host_blocks;   // pinned host allocations
     std::vector<hipEvent_t> tickets;   // live tickets: ticket t -> tickets[t - retired - 1]
     uint64_t retired = 0;              // tickets known complete and destroyed
     int32_t* moe_status = nullptr;     // device flag: an id outside [0,E) was seen
@@ -69,6 +70,7 @@ zc_status zc_hip_destroy(zc_hip_ctx* ctx) {
     for (auto e : ctx->tickets) hipEventDestroy(e);
     for (auto e : ctx->timer) if (e) hipEventDestroy(e);
     for (auto& b : ctx->blocks) hipFree(b.first);
+    for (auto& b : ctx->host_blocks) hipHostFree(b.first);
     hipFree(ctx->moe_status);
     hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -88,10 +90,30 @@ zc_status zc_hip_alloc(zc_hip_ctx* ctx, uint64_t bytes, void** out) {
     *out = p;
     return ZC_OK;
 }
+zc_status zc_hip_alloc_host(zc_hip_ctx* ctx, uint64_t bytes, void** out) {
+    ZC_REQUIRE(ctx && out, "null argument");
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    if (ctx->budget && (bytes > ctx->budget || ctx->allocated > ctx->budget - bytes))
+        return fail(ZC_BUDGET_EXCEEDED, "engine memory budget exceeded");
+    void* p = nullptr;
+    ZC_HIP(hipSetDevice(ctx->device));
+    const hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocMapped | hipHostMallocCoherent);
+    if (e != hipSuccess) { (void)hipGetLastError(); return fail(ZC_BUDGET_EXCEEDED, std::string("host allocation failed: ") + hipGetErrorString(e)); }
+    ctx->host_blocks[p] = bytes; ctx->allocated += bytes;
+    if (ctx->allocated > ctx->peak) ctx->peak = ctx->allocated;
+    *out = p;
+    return ZC_OK;
+}
 zc_status zc_hip_free(zc_hip_ctx* ctx, void* ptr) {
     ZC_REQUIRE(ctx, "null context");
     if (!ptr) return ZC_OK;
     std::lock_guard<std::mutex> lock(ctx->mutex);
+    if (auto h = ctx->host_blocks.find(ptr); h != ctx->host_blocks.end()) {
+        ZC_HIP(hipStreamSynchronize(ctx->stream));
+        ZC_HIP(hipHostFree(ptr));
+        ctx->allocated -= h->second; ctx->host_blocks.erase(h);
+        return ZC_OK;
+    }
     auto it = ctx->blocks.find(ptr);
     if (it == ctx->blocks.end()) return fail(ZC_LOGIC_ERROR, "free of a pointer this context did not allocate");
     ZC_HIP(hipStreamSynchronize(ctx->stream));   // no GPU user may outlive its buffer

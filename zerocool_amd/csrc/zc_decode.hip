@@ -167,18 +167,13 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
     const XintLayout LH{H}, LI{I};
     Barrier bar{p.sync, p.epoch, p.spin_limit, p.status, p.epoch};
     uint32_t stamp = 0;
-    auto clock = [&]() { if (p.clocks && wg == 0 && tid == 0) p.clocks[stamp] = wall_clock64(); ++stamp; };
+    // stamps of every workgroup: clocks[(stamp index) * workgroups + workgroup]
+    auto clock = [&]() { if (p.clocks && tid == 0) p.clocks[uint64_t(stamp) * nwg + wg] = wall_clock64(); ++stamp; };
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
 
     for (uint32_t layer = 0; layer < p.L; ++layer) {
         const DecodeLayer L = p.layers[layer];
-        clock();
-        if (p.clocks) {   // calibration: 1024 dependent fused multiply-adds
-            float v = __uint_as_float(p.epoch);
-            for (int i = 0; i < 1024; ++i) v = __builtin_fmaf(v, 1.0000001f, 0.5f);
-            if (v == 12345.0f) atomicOr(p.status, 8);
-        }
         clock();
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
@@ -450,6 +445,10 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
     lp.ah = lp.img_d + sb * LI.bytes();
     const uint32_t d_end = lp.ah + sb * align16(I * 2);
     lp.total = rg_end > d_end ? rg_end : d_end;
+    // One workgroup per compute unit: ask for more than half of the LDS so that the
+    // dispatcher cannot stack two workgroups on one unit and leave another idle.
+    const uint32_t exclusive = lds_limit / 2 + 1024;
+    if (lp.total < exclusive) lp.total = exclusive;
     return lp;
 }
 

@@ -62,9 +62,9 @@ struct DecodeParams {
     uint32_t* maxabs;                // [L][T] bit patterns of max |layer output|
     int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][T][topk], [L][T][topk], [L][T][H]
     uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
-    unsigned long long* clocks;      // optional [L][kDecodeStamps] 100 MHz timestamps of workgroup 0
+    unsigned long long* clocks;      // optional [L * kDecodeStamps][workgroups] 100 MHz timestamps, one per workgroup
 };
-constexpr uint32_t kDecodeStamps = 13;
+constexpr uint32_t kDecodeStamps = 15;
 struct DecodeLdsPlan {
     uint32_t ids, weights, gatev, head, next, experts, misc, region, total;
     uint32_t img_rg, xh, img_d, ah, otile, slots_per_batch;

@@ -235,12 +235,8 @@ __device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16
                     const v4i b0 = expand(codes[j].x, codes[j].y), b1 = expand(codes[j].z, codes[j].w);
                     const uint8_t* a_at = planes + a_first + d * a_span;
                     const v4i a0 = *reinterpret_cast<const v4i*>(a_at), a1 = *reinterpret_cast<const v4i*>(a_at + a_next);
-#ifdef ZC_PROBE_NO_MFMA
-                    const v4i r0 = a0 + b0 + zero, r1 = a1 + b1;
-#else
                     const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
                     const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, zero, 0, 0, 0);
-#endif
                     const float4 fi = *reinterpret_cast<const float4*>(info + 8 * d + 2 * G);   // {2^e, sum} of blocks 2G, 2G+1
                     dot[j][0] = float(r0[0] + (r0[1] << 7) + (r0[2] << 14)) * fi.x; bsum[j][0] = fi.y;
                     dot[j][1] = float(r1[0] + (r1[1] << 7) + (r1[2] << 14)) * fi.z; bsum[j][1] = fi.w;
@@ -249,11 +245,7 @@ __device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16
             // pass 2: blocks 8d + 2G + h of spans d0 .. d0+7 sit in mask words d0/4, d0/4 + 1
             const uint32_t mine = 0x03030303u << (2 * G);
             const uint32_t u0 = mask[d0 / 4] & mine, u1 = R == 8 ? mask[d0 / 4 + 1] & mine : 0u;
-#ifdef ZC_PROBE_NO_FALLBACK
-            if (false) {
-#else
             if (__builtin_expect(__ballot((u0 | u1) != 0) != 0, 0)) {
-#endif
 #pragma unroll
                 for (int j = 0; j < R; ++j) {
                     const uint32_t d = d0 + j;

@@ -54,7 +54,7 @@ def run_stack(ctx, cfg, stack, x_dev, T, L, layered):
     return r
 
 
-def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1)):
+def _check_stack(ctx, cfg, L, tokens, seed, skew, persistent):
     layers = [workload.LayerWeights(ctx, cfg, seed + l, skew) for l in range(L)]
     hosts = [l.host() for l in layers]
     stack = ctx.stack_create(cfg, [l.layer for l in layers], max(tokens))
@@ -62,7 +62,7 @@ def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1)):
         x_dev = workload.hidden_rows(ctx, T, cfg.hidden, seed * 131 + T)
         x = x_dev.numpy(f32)
         want = oracle_stack(cfg, hosts, x, T)
-        assert ctx.stack_is_persistent(stack, T) == (T <= 8)
+        assert ctx.stack_is_persistent(stack, T) == (persistent and T <= 8)
         for layered in (True, False):
             got = run_stack(ctx, cfg, stack, x_dev, T, L, layered)
             name = "layered" if layered else "persistent"
@@ -79,12 +79,20 @@ def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1)):
             ctx.free(b)
 
 
-def test_tiny_stack(ctx):
-    check_stack(ctx, workload.tiny_config(hidden=512, experts=32, topk=4, inter=512), 3, [1, 2, 3, 5, 8, 11])
+def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1), persistent=True):
+    return _check_stack(ctx, cfg, L, tokens, seed, skew, persistent)
 
 
-def test_small_stack_many_experts(ctx):
-    check_stack(ctx, workload.tiny_config(hidden=1024, experts=128, topk=10, inter=512), 4, [1, 8])
+def test_few_experts_stack(ctx):  # the single-layer shape (hidden 2048 / intermediate 512) with few experts
+    check_stack(ctx, workload.tiny_config(hidden=2048, experts=32, topk=4, inter=512), 3, [1, 2, 3, 5, 8, 11])
+
+
+def test_single_layer_shape_stack(ctx):
+    check_stack(ctx, workload.tiny_config(hidden=2048, experts=128, topk=10, inter=512), 3, [1, 8])
+
+
+def test_other_shapes_take_the_layered_path(ctx):
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512), 2, [1, 4], persistent=False)
 
 
 def test_stand_in_stack_shape(ctx):  # hidden 3072 / intermediate 1024, two layers of the 48
@@ -92,7 +100,7 @@ def test_stand_in_stack_shape(ctx):  # hidden 3072 / intermediate 1024, two laye
 
 
 def test_stack_reports_invalid_router_output(ctx):
-    cfg = workload.tiny_config(hidden=512, experts=32, topk=4, inter=512)
+    cfg = workload.tiny_config(hidden=2048, experts=32, topk=4, inter=512)
     layers = [workload.LayerWeights(ctx, cfg, 77 + l, None) for l in range(2)]
     stack = ctx.stack_create(cfg, [l.layer for l in layers], 2)
     bad = ctx.upload(np.full(2 * cfg.hidden, np.nan, f32)); out = ctx.alloc(2 * cfg.hidden * 4)

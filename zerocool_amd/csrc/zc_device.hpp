@@ -70,6 +70,7 @@ __device__ __forceinline__ uint4 ldg_u4(const void* p, uint32_t index = 0) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ uint16_t ldg_u16(const void* p, uint32_t index = 0) { return as_global<uint16_t>(p)[index]; }
+__device__ __forceinline__ uint32_t ldg_u32(const void* p, uint32_t index = 0) { return as_global<uint32_t>(p)[index]; }
 __device__ __forceinline__ float ldg_f32(const void* p, uint32_t index = 0) { return as_global<float>(p)[index]; }
 
 // DPP moves inside rows of 16 lanes.  row_shr:1 hands lane i the value of lane i-1

@@ -91,8 +91,12 @@ def test_single_layer_shape_stack(ctx):
     check_stack(ctx, workload.tiny_config(hidden=2048, experts=128, topk=10, inter=512), 3, [1, 8])
 
 
-def test_other_shapes_take_the_layered_path(ctx):
-    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512), 2, [1, 4], persistent=False)
+def test_small_hidden_stack(ctx):
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512), 2, [1, 4])
+
+
+def test_other_shapes_take_the_layered_path(ctx):  # hidden not a multiple of 512
+    check_stack(ctx, workload.tiny_config(hidden=768, experts=64, topk=10, inter=512), 2, [1, 4], persistent=False)
 
 
 def test_stand_in_stack_shape(ctx):  # hidden 3072 / intermediate 1024, two layers of the 48

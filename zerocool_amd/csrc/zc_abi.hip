@@ -480,7 +480,7 @@ struct zc_hip_stack {
 namespace {
 bool persistent_shape(const zc_moe_config& c) {
     return c.bits_gate_up == 4 && c.bits_down == 4 && c.shared_bits_gate_up == 4 && c.shared_bits_down == 4 && c.group == 64 &&
-           zc::decode_stack_shape(c.hidden, c.inter) && c.experts <= 1024 && c.topk <= 64;
+           c.hidden % 512 == 0 && c.inter % 512 == 0 && c.hidden <= 3072 && c.inter <= 1024 && c.experts <= 1024 && c.topk <= 64;
 }
 uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : 8; }   // kernel variant; LDS is sized by the real token count
 }  // namespace
@@ -559,7 +559,7 @@ static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, 
     *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
     if (plan->total > st->lds_limit || plan->slots_per_batch == 0) return false;
     int per_cu = 0;
-    if (zc::decode_stack_occupancy(*nt, st->cfg.hidden, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+    if (zc::decode_stack_occupancy(*nt, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
     (void)ctx;
     return per_cu >= 1;
 }

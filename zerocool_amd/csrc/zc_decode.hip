@@ -150,20 +150,18 @@ __device__ __forceinline__ void route_token(const float* logits, uint32_t E, uin
     if (lane < topk) weights[lane] = v * inverse;
 }
 
-constexpr int kRing = 8;         // sixteen-byte router pieces in flight per lane
-// SH = hidden / 512 and SI = intermediate / 512 are the spans per wave and tile; tiles in flight per wave are chosen
-// so that about eight to eighteen spans (1 KB each per wave) are on their way.
-template <int S> constexpr int kTilesInFlight = S >= 4 ? 3 : S == 3 ? 4 : S == 2 ? 6 : 8;
-#define ZC_RUN_HIDDEN(...) xint_run_split<SH, kTilesInFlight<SH>, NT == 1, LdsBf16>(__VA_ARGS__)
-#define ZC_RUN_INTER(...) xint_run_split<SI, kTilesInFlight<SI>, NT == 1, LdsBf16>(__VA_ARGS__)
+constexpr int kRing = 8;         // 128-element spans of a tile in flight per lane (four when the span count is odd in eights)
+#define ZC_RUN_TILE(SPANS, ...) do { if ((SPANS) % 8 == 0) xint_run_tile<PT, 8>(__VA_ARGS__); else xint_run_tile<PT, 4>(__VA_ARGS__); } while (0)
+constexpr int kMaxTokens = 8;
 
-// NT = 1: single-token decode.  NT = 8: up to eight tokens (router accumulators per token).
-template <int NT, int SH, int SI>
+// NT = 1: single-token decode.  NT = 8: up to eight tokens, tiles take four at a time.
+template <int NT>
 __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
+    constexpr int PT = NT < 4 ? NT : 4;   // tokens per tile pass
     extern __shared__ __align__(16) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wg = blockIdx.x, nwg = gridDim.x;
     const uint32_t H = p.H, E = p.E, I = p.I, k = p.topk, T = p.T, n = T * k;
-    const uint32_t col = lane & 15u;
+    const uint32_t col = lane & 15u, G = lane >> 4;
     int32_t* ids = reinterpret_cast<int32_t*>(lds + lp.ids);
     float* weights = reinterpret_cast<float*>(lds + lp.weights);
     float* gatev = reinterpret_cast<float*>(lds + lp.gatev);
@@ -180,10 +178,6 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };   // after the slowest wave of the workgroup
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
-    // byte offsets of the lane's gate (columns 0-7) or up (columns 8-15) projection inside a record: codes, scales, biases
-    const bool up_lane = col >= 8;
-    const uint64_t ro_w = up_lane ? p.ro[3] : p.ro[0], ro_s = up_lane ? p.ro[4] : p.ro[1], ro_b = up_lane ? p.ro[5] : p.ro[2];
-    const uint64_t so_w = up_lane ? p.so[3] : p.so[0], so_s = up_lane ? p.so[4] : p.so[1], so_b = up_lane ? p.so[5] : p.so[2];
 
     for (uint32_t layer = 0; layer < p.L; ++layer) {
         const DecodeLayer L = p.layers[layer];
@@ -198,40 +192,27 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
             }
             __syncthreads();
             const bool glue = layer != 0;
+            // the shared-expert gate row rides along: coalesced sixteen-byte loads, used from LDS by the gate-dot waves
+            uint4 gate_piece[2];
+#pragma unroll
+            for (int q = 0; q < 2; ++q) if (tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
             const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), [&](uint32_t i, float& a, float& b) {
                 if (glue) { const float inv = gatev[(2 * i) / H]; a = bf(a * inv); b = bf(b * inv); }
             });
             if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
+#pragma unroll
+            for (int q = 0; q < 2; ++q) if (tid + q * kDecodeThreads < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
         }
         __syncthreads();
         xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
         clock();
-        float* part = reinterpret_cast<float*>(lds + lp.part);
-        {   // shared gate/up tiles: the whole workgroup runs a tile, tiles go round the workgroups
-            constexpr uint32_t tiles = SI * 64;   // I / 8
-            const uint8_t* rec = L.shared_record;
-            auto unit_of = [&](uint32_t i) {
-                const uint32_t row = (wg + i * nwg) * 8 + (col & 7u);
-                return XintRows{rec + so_w + row * (H / 2), reinterpret_cast<const uint16_t*>(rec + so_s) + row * (H / 64),
-                                reinterpret_cast<const uint16_t*>(rec + so_b) + row * (H / 64)};
-            };
-            auto pass_of = [&](uint32_t, uint32_t pass, const uint8_t*& planes, LdsBf16& src, uint32_t& token) {
-                if (pass >= T) return false;
-                planes = lds + lp.img_rg + pass * LH.bytes(); src = LdsBf16{xh_all + pass * H}; token = pass;
-                return true;
-            };
-            auto emit = [&](uint32_t i, uint32_t token, uint32_t column, float v, float up) {
-                if (column < 8) st_f32(p.shared_act + uint64_t(token) * I + (wg + i * nwg) * 8 + column, swiglu_bf(v, up));
-            };
-            const uint32_t count = wg < tiles ? (tiles - wg + nwg - 1) / nwg : 0;
-            ZC_RUN_HIDDEN(count, unit_of, pass_of, emit, LH, part, lane, wave);
-        }
-        {   // one-wave units, handed out from the last workgroup down: shared-expert gate dots, then router rows
-            const uint32_t router_units = (E + 3) / 4, gate_units = (T + 1) / 2;
-            for (uint32_t u = (nwg - 1 - wg) + nwg * wave; u < gate_units + router_units; u += nwg * kDecodeWaves) {
-                if (u >= gate_units) {
+        {
+            const uint32_t router_units = (E + 3) / 4, shared_units = I / 8, gate_units = (T + 1) / 2;
+            const uint32_t units = router_units + shared_units + gate_units;
+            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
+                if (u < router_units) {
                     // four experts x sixteen K partitions; k-ascending fused chain per partition
-                    const uint32_t e = (u - gate_units) * 4 + lane / 16, split = lane % 16, P = H / 16;
+                    const uint32_t e = u * 4 + lane / 16, split = lane % 16, P = H / 16;
                     const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
                     const uint32_t pieces = P / 8;   // sixteen-byte pieces of the partition, kRing in flight
                     uint4 wv[kRing];
@@ -271,19 +252,29 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                         for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c[t];
                         if (split == 15 && e < E) st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + offset : sum);
                     }
+                } else if (u < router_units + shared_units) {
+                    const uint32_t tile = u - router_units, row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                    const uint8_t* rec = L.shared_record;
+                    const uint8_t* w_row = rec + p.so[pr] + uint64_t(row) * (H / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64);
+                    for (uint32_t t0 = 0; t0 < T; t0 += PT) {
+                        const uint8_t* img[PT]; LdsBf16 src[PT];
+#pragma unroll
+                        for (int t = 0; t < PT; ++t) {
+                            const uint32_t tt = t0 + t < T ? t0 + t : 0;
+                            img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
+                        }
+                        auto emit = [&](int t, float v) {
+                            const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                            if (G == 0 && col < 8) st_f32(p.shared_act + uint64_t(t0 + t) * I + row, swiglu_bf(v, up));
+                        };
+                        ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, int(min(uint32_t(PT), T - t0)), emit);
+                    }
                 } else {
                     // shared_expert_gate: reference lane chain k = lane + 32 j (qwen.metal:499-506); two tokens per wave
-                    const uint32_t t = u * 2 + (lane >> 5), l32 = lane & 31u;
-                    // the weight row goes through LDS: coalesced sixteen-byte loads, all in flight at once
-                    uint16_t* gw = reinterpret_cast<uint16_t*>(lds + lp.gatew);   // waves that share it write the same bytes
-                    for (uint32_t i0 = 0; i0 < H / 8; i0 += 64 * 8) {
-                        uint4 piece[8];
-#pragma unroll
-                        for (int q = 0; q < 8; ++q) if (i0 + q * 64 + lane < H / 8) piece[q] = ldg_u4(L.shared_gate, i0 + q * 64 + lane);
-#pragma unroll
-                        for (int q = 0; q < 8; ++q) if (i0 + q * 64 + lane < H / 8) reinterpret_cast<uint4*>(gw)[i0 + q * 64 + lane] = piece[q];
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    const uint32_t t = (u - router_units - shared_units) * 2 + (lane >> 5), l32 = lane & 31u;
+                    const uint16_t* gw = reinterpret_cast<const uint16_t*>(lds + lp.gatew);   // staged with the input rows
                     float sum = 0;
                     if (t < T)
                         for (uint32_t kk = l32; kk < H; kk += 32) sum += b16(xh_all[t * H + kk]) * b16(gw[kk]);
@@ -333,28 +324,31 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
         const uint32_t U = uint32_t(uniform(misc[0]));
         clock();
         {
-            constexpr uint32_t tiles = SI * 64;   // I / 8
-            const uint32_t units = U * tiles;
-            int32_t cursor = -1;
-            auto unit_of = [&](uint32_t i) {
-                const uint32_t u = wg + i * nwg, e = uint32_t(uniform(experts[u / tiles])), row = (u % tiles) * 8 + (col & 7u);
+            const uint32_t tiles = I / 8, units = U * tiles;
+            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
+                const uint32_t e = uint32_t(uniform(experts[u / tiles])), tile = u % tiles;
+                const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                 const uint8_t* rec = L.records + uint64_t(e) * L.stride;
-                return XintRows{rec + ro_w + row * (H / 2), reinterpret_cast<const uint16_t*>(rec + ro_s) + row * (H / 64),
-                                reinterpret_cast<const uint16_t*>(rec + ro_b) + row * (H / 64)};
-            };
-            auto pass_of = [&](uint32_t i, uint32_t pass, const uint8_t*& planes, LdsBf16& src, uint32_t& slot) {   // the expert's slots, one per pass
-                if (pass == 0) cursor = uniform(head[uniform(experts[(wg + i * nwg) / tiles])]);
-                if (cursor < 0) return false;
-                slot = uint32_t(cursor); cursor = uniform(next[cursor]);
-                const uint32_t tt = NT == 1 ? 0u : slot / k;
-                planes = lds + lp.img_rg + tt * LH.bytes(); src = LdsBf16{xh_all + tt * H};
-                return true;
-            };
-            auto emit = [&](uint32_t i, uint32_t slot, uint32_t column, float v, float up) {
-                if (column < 8) st_f32(p.act + uint64_t(slot) * I + ((wg + i * nwg) % tiles) * 8 + column, swiglu_bf(v, up));
-            };
-            const uint32_t count = wg < units ? (units - wg + nwg - 1) / nwg : 0;
-            ZC_RUN_HIDDEN(count, unit_of, pass_of, emit, LH, part, lane, wave);
+                const uint8_t* w_row = rec + p.ro[pr] + uint64_t(row) * (H / 2);
+                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64);
+                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64);
+                int32_t s = uniform(head[e]);
+                while (s >= 0) {   // the expert's slots, PT at a time
+                    const uint8_t* img[PT]; LdsBf16 src[PT]; int32_t slot[PT]; int nt = 0;
+#pragma unroll
+                    for (int t = 0; t < PT; ++t) { slot[t] = s; if (s >= 0) { nt = t + 1; s = uniform(next[s]); } }
+#pragma unroll
+                    for (int t = 0; t < PT; ++t) {
+                        const uint32_t tt = t < nt ? uint32_t(slot[t]) / k : 0;
+                        img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
+                    }
+                    auto emit = [&](int t, float v) {
+                        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                        if (G == 0 && col < 8) st_f32(p.act + uint64_t(slot[t]) * I + row, swiglu_bf(v, up));
+                    };
+                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, nt, emit);
+                }
+            }
         }
         clock_all();
         bar.wait();
@@ -379,28 +373,33 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 if (s0 == 0) clock();
                 xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
                 if (s0 == 0) clock();
-                {   // units: the selected experts in list order, then the shared expert
-                    int32_t cursor = -1;
-                    auto unit_of = [&](uint32_t i) {
-                        const bool routed = i < U;
-                        const uint8_t* rec = routed ? L.records + uint64_t(uint32_t(uniform(experts[i < U ? i : 0]))) * L.stride : L.shared_record;
-                        const uint64_t ow = routed ? p.ro[6] : p.so[6], os = routed ? p.ro[7] : p.so[7], ob = routed ? p.ro[8] : p.so[8];
-                        return XintRows{rec + ow + row * (I / 2), reinterpret_cast<const uint16_t*>(rec + os) + row * (I / 64),
-                                        reinterpret_cast<const uint16_t*>(rec + ob) + row * (I / 64)};
-                    };
-                    auto pass_of = [&](uint32_t i, uint32_t pass, const uint8_t*& planes, LdsBf16& src, uint32_t& slot) {   // the unit's slots that lie in the batch
-                        if (pass == 0) cursor = i < U ? uniform(head[uniform(experts[i])]) : int32_t(n);
-                        for (;;) {
-                            if (i < U ? cursor < 0 : uint32_t(cursor) >= n + T) return false;
-                            const int32_t s = cursor;
-                            cursor = i < U ? uniform(next[cursor]) : cursor + 1;
-                            if (uint32_t(s) >= s0 && uint32_t(s) < s0 + sn) { slot = uint32_t(s); break; }
+                for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
+                    const uint8_t* rec; const uint64_t* off; int32_t s;
+                    if (u < U) { const uint32_t e = uint32_t(uniform(experts[u])); s = uniform(head[e]); rec = L.records + uint64_t(e) * L.stride; off = p.ro; }
+                    else { s = int32_t(n); rec = L.shared_record; off = p.so; }
+                    const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
+                    while (u < U ? s >= 0 : uint32_t(s) < n + T) {
+                        // next PT slots of this unit that lie in the batch
+                        int32_t slot[PT]; int nt = 0;
+#pragma unroll
+                        for (int t = 0; t < PT; ++t) slot[t] = int32_t(s0);
+                        while (nt < PT && (u < U ? s >= 0 : uint32_t(s) < n + T)) {
+                            if (uint32_t(s) >= s0 && uint32_t(s) < s0 + sn) {
+#pragma unroll
+                                for (int q = 0; q < PT; ++q) if (q == nt) slot[q] = s;
+                                ++nt;
+                            }
+                            s = u < U ? uniform(next[s]) : s + 1;
                         }
-                        planes = lds + lp.img_d + (slot - s0) * LI.bytes(); src = source_of(slot - s0);
-                        return true;
-                    };
-                    auto emit = [&](uint32_t, uint32_t slot, uint32_t column, float v, float) { otile[slot * 16 + column] = bf(v); };
-                    ZC_RUN_INTER(U + 1, unit_of, pass_of, emit, LI, part, lane, wave);
+                        if (!nt) break;
+                        const uint8_t* img[PT]; LdsBf16 src[PT];
+#pragma unroll
+                        for (int t = 0; t < PT; ++t) { img[t] = lds + lp.img_d + (uint32_t(slot[t]) - s0) * LI.bytes(); src[t] = source_of(uint32_t(slot[t]) - s0); }
+                        auto emit = [&](int t, float v) { if (G == 0) otile[uint32_t(slot[t]) * 16 + col] = bf(v); };
+                        ZC_RUN_TILE(I / 128, w_row, s_row, b_row, I / 128, img, src, LI, lane, nt, emit);
+                    }
                 }
             }
             __syncthreads();
@@ -446,9 +445,7 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
     uint32_t at = 0;
     auto take = [&](uint32_t bytes) { const uint32_t o = at; at += align16(bytes); return o; };
     lp.ids = take(NT * topk * 4); lp.weights = take(NT * topk * 4); lp.gatev = take(NT * 4);
-    lp.head = take(E * 4); lp.next = take(NT * topk * 4); lp.experts = take(E * 4); lp.misc = take(64);
-    lp.part = take(kXintPartBytes > H * 2 ? kXintPartBytes : H * 2);
-    lp.gatew = lp.part;   // the shared-gate row is staged after the workgroup's tiles are finished, in the same space
+    lp.head = take(E * 4); lp.next = take(NT * topk * 4); lp.experts = take(E * 4); lp.misc = take(64); lp.gatew = take(H * 2);
     lp.region = at;
     lp.img_rg = lp.region; lp.xh = lp.img_rg + NT * LH.bytes();
     const uint32_t rg_end = lp.xh + align16(NT * H * 2);
@@ -469,28 +466,24 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
     return lp;
 }
 
-// The instantiated shapes: (hidden, intermediate) = (3072, 1024) and (2048, 512).
-bool decode_stack_shape(uint32_t hidden, uint32_t inter) { return (hidden == 3072 && inter == 1024) || (hidden == 2048 && inter == 512); }
-
-template <class F> static hipError_t with_kernel(uint32_t nt, uint32_t hidden, F f) {
-    if (hidden == 3072) return nt == 1 ? f(decode_stack_kernel<1, 6, 2>) : f(decode_stack_kernel<8, 6, 2>);
-    return nt == 1 ? f(decode_stack_kernel<1, 4, 1>) : f(decode_stack_kernel<8, 4, 1>);
-}
 hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp) {
-    if (!decode_stack_shape(p.H, p.I)) return hipErrorInvalidValue;
-    return with_kernel(nt, p.H, [&](auto kernel) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(kDecodeThreads), lp.total, s, p, lp);
-        return hipGetLastError();
-    });
+#define ZC_DECODE(NT)                                                                                              \
+    do {                                                                                                           \
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<NT>),                  \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));             \
+        if (e != hipSuccess) return e;                                                                             \
+        hipLaunchKernelGGL((decode_stack_kernel<NT>), dim3(workgroups), dim3(kDecodeThreads), lp.total, s, p, lp);  \
+    } while (0)
+    if (nt == 1) ZC_DECODE(1); else ZC_DECODE(8);
+#undef ZC_DECODE
+    return hipGetLastError();
 }
-hipError_t decode_stack_occupancy(uint32_t nt, uint32_t hidden, uint32_t lds_bytes, int* blocks_per_cu) {
-    return with_kernel(nt, hidden, [&](auto kernel) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-        if (e != hipSuccess) return e;
-        return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, kernel, kDecodeThreads, lds_bytes);
-    });
+hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu) {
+    const void* f = nt == 1 ? reinterpret_cast<const void*>(decode_stack_kernel<1>) : reinterpret_cast<const void*>(decode_stack_kernel<8>);
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (e != hipSuccess) return e;
+    if (nt == 1) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<1>, kDecodeThreads, lds_bytes);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<8>, kDecodeThreads, lds_bytes);
 }
 
 }  // namespace zc

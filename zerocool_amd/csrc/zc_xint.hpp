@@ -285,151 +285,4 @@ __device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16
     }
 }
 
-
-// ---------------------------------------------------------------------------------------------
-// Tiles run by a whole workgroup of four waves.  Wave m owns the spans d = m, m+4, m+8, ...
-// of every tile: exactly the blocks of reference lanes 8m .. 8m+7, whose running sums never mix
-// with the other waves' until the final butterfly.  Each wave keeps its lanes' two sums per
-// (tile, input image); the four waves meet in LDS once per batch of kXintBatch such sums, and
-// every wave then finishes four of the sixteen columns.
-//
-//   unit_of(i)                       -> the lane's weight row of tile i (lane = (column, G))
-//   pass_of(i, pass, planes, src, tag) -> next input image for tile i and a tag for emit, false when there is none
-//   emit(i, tag, column, value, partner): called by one lane per column with the finished
-//       row sum; partner is the sum of the column eight to the right (or left) -- the
-//       up-projection row of a gate/up tile.
-// All four waves must call this with the same units and passes (it synchronises the
-// workgroup).  S = K / 512 spans per wave and tile; UB tiles are in flight.
-// ONE: every tile has exactly one pass (single-token decode); the code is then straight-line
-// per tile, which lets the wait for a tile's loads count precisely the younger loads in flight.
-struct XintRows { const uint8_t* w; const uint16_t* s; const uint16_t* b; };
-constexpr uint32_t kXintBatch = 8;                                   // finished together after one workgroup barrier
-constexpr uint32_t kXintPartBytes = kXintBatch * 2048 + 64;          // LDS behind `part`: sums, then {tile, tag} pairs
-
-template <int S, int UB, bool ONE, class Source, class UnitOf, class PassOf, class Emit>
-__device__ __forceinline__ void xint_run_split(uint32_t count, UnitOf unit_of, PassOf pass_of, Emit emit,
-                                               const XintLayout L, float* part, uint32_t lane, uint32_t m) {
-    const uint32_t G = lane >> 4, row_a = lane & 15u, c_a = row_a >> 2, p_a = row_a & 3u;
-    // A operand: row (c,p) of lane group G holds digit plane p of block 8d + 2c (+1) when c == G, zeros otherwise
-    const bool live = (c_a == G) && p_a < 3;
-    const uint32_t a_first = live ? (8 * m + 2 * G) * 48 + p_a * 16 : L.blocks() * 48, a_step = live ? 32 * 48 : 0, a_next = live ? 48 : 0;
-    const uint32_t first_block = 8 * m + 2 * G;           // block 8d + 2G of span d = m + 4q is first_block + 32q
-    const uint32_t shamt = (lane & 32u) ? 0u : 16u;       // group 2d + (G >> 1) is the low half of metadata dword d for G < 2
-    // finishing layout: lane = (c: 2 bits, G: 2 bits, h: 1 bit); wave m finishes columns 2m, 2m+1, 8+2m, 9+2m
-    const uint32_t fc = lane & 3u, fG = (lane >> 2) & 3u, fh = (lane >> 4) & 1u;
-    const uint32_t fcol = fc < 2 ? 2 * m + fc : 6 + 2 * m + fc;
-    const uint32_t fidx = (fG * 16 + fcol) * 2 + fh;
-    uint32_t* meta = reinterpret_cast<uint32_t*>(part + kXintBatch * 512);
-    const uint32_t M = 0x0f0f0f0fu;
-    const v4i zero = {0, 0, 0, 0};
-    auto expand = [&](uint32_t lo, uint32_t hi) { const v4i r = {int(lo & M), int((lo >> 4) & M), int(hi & M), int((hi >> 4) & M)}; return r; };
-    // Metadata: dword d of a row's scale (bias) vector holds groups 2d, 2d+1.  The four lanes of a column fetch the
-    // dwords of four different spans with one load (lane group G takes span q = G + 4r) and hand them round later.
-    constexpr int MR = (S + 3) / 4;
-    uint4 ring[UB][S]; uint32_t sring[UB][MR], bring[UB][MR];
-    auto issue = [&](int ub, uint32_t i) {
-        const XintRows r = unit_of(i);
-        const uint8_t* wb = r.w + 16 * G + 64 * m;              // span d = m + 4q: byte d * 64 of the row
-#pragma unroll
-        for (int q = 0; q < S; ++q) ring[ub][q] = ldg_u4(wb, 16 * q);
-#pragma unroll
-        for (int rr = 0; rr < MR; ++rr) {
-            const uint32_t q = min(G + 4 * rr, uint32_t(S - 1));
-            sring[ub][rr] = ldg_u32(r.s, m + 4 * q);
-            bring[ub][rr] = ldg_u32(r.b, m + 4 * q);
-        }
-    };
-    if (count == 0) return;
-#pragma unroll
-    for (int ub = 0; ub < UB; ++ub) issue(ub, min(uint32_t(ub), count - 1));   // a fixed number of loads in flight: tiles past the end repeat the last one
-    uint32_t nb = 0;   // sums waiting in the batch
-    auto flush = [&]() {
-        __syncthreads();
-#pragma clang loop unroll(disable)
-        for (uint32_t b = 0; b < nb; ++b) {
-            // reference lane sum (xor butterfly 16, 8, 4, 2, 1): strides 16 and 8 pair the waves,
-            // 4 and 2 pair lane groups, 1 pairs the two blocks of a lane
-            const float* mine = part + b * 512;
-            const float a = (mine[fidx] + mine[256 + fidx]) + (mine[128 + fidx] + mine[384 + fidx]);
-            float sum = a + __shfl_xor(a, 8);
-            sum = sum + __shfl_xor(sum, 4);
-            const float value = sum + __shfl_xor(sum, 16);
-            const float partner = __shfl_xor(value, 2);
-            if (lane < 4) emit(meta[2 * b], meta[2 * b + 1], fcol, value, partner);
-        }
-        __syncthreads();
-        nb = 0;
-    };
-    for (uint32_t i0 = 0; i0 < count; i0 += UB) {
-#pragma unroll
-        for (int ub = 0; ub < UB; ++ub) {
-            const uint32_t i = i0 + ub;
-            if (i < count) {
-                // the tile's loads must have landed HERE, not at the top of a loop that merely uses them
-#pragma unroll
-                for (int q = 0; q < S; ++q) asm volatile("" : "+v"(ring[ub][q].x), "+v"(ring[ub][q].y), "+v"(ring[ub][q].z), "+v"(ring[ub][q].w));
-#pragma unroll
-                for (int rr = 0; rr < MR; ++rr) asm volatile("" : "+v"(sring[ub][rr]), "+v"(bring[ub][rr]));
-                float sc[S], bi[S];
-#pragma unroll
-                for (int q = 0; q < S; ++q) {   // the dword of span q sits with the column's lane of group q mod 4
-                    const int from = int((lane & 15u) | (uint32_t(q & 3) << 4));
-                    sc[q] = __uint_as_float((uint32_t(__shfl(int(sring[ub][q >> 2]), from)) << shamt) & 0xffff0000u);
-                    bi[q] = __uint_as_float((uint32_t(__shfl(int(bring[ub][q >> 2]), from)) << shamt) & 0xffff0000u);
-                }
-                for (uint32_t pass = 0; !ONE || pass == 0; ++pass) {
-                    const uint8_t* planes; Source src; uint32_t tag;
-                    if (!pass_of(i, pass, planes, src, tag)) break;
-                    const float2* info = reinterpret_cast<const float2*>(planes + L.planes_bytes());
-                    const uint32_t* mask = reinterpret_cast<const uint32_t*>(planes + L.planes_bytes() + L.info_bytes());
-                    float term[S][2];      // scale*dot + sum*bias of the lane's two blocks of span q
-                    uint32_t unsafe[S], any = 0;
-#pragma unroll
-                    for (int q = 0; q < S; ++q) {
-                        const uint4 w = ring[ub][q];
-                        const v4i b0 = expand(w.x, w.y), b1 = expand(w.z, w.w);
-                        const uint8_t* a_at = planes + a_first + q * a_step;
-                        const v4i a0 = *reinterpret_cast<const v4i*>(a_at), a1 = *reinterpret_cast<const v4i*>(a_at + a_next);
-                        const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
-                        const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, zero, 0, 0, 0);
-                        const float4 fi = *reinterpret_cast<const float4*>(info + first_block + 32 * q);   // {2^e, sum} of the two blocks
-                        term[q][0] = sc[q] * (float(r0[0] + (r0[1] << 7) + (r0[2] << 14)) * fi.x) + fi.y * bi[q];
-                        term[q][1] = sc[q] * (float(r1[0] + (r1[1] << 7) + (r1[2] << 14)) * fi.z) + fi.w * bi[q];
-                        unsafe[q] = (mask[q] >> first_block) & 3u;   // blocks first_block + 32q (+1) sit in mask word q
-                        any |= unsafe[q];
-                    }
-                    if (__builtin_expect(__ballot(any != 0) != 0, 0)) {
-                        // rare blocks: ONE copy of the literal chain in a rolled loop; the span's operands are
-                        // picked out of the register arrays by a select chain on the (uniform) loop counter
-#pragma clang loop unroll(disable)
-                        for (uint32_t q = 0; q < uint32_t(S); ++q) {
-                            uint4 w = ring[ub][0]; uint32_t bits = unsafe[0]; float scq = sc[0], biq = bi[0];
-#pragma unroll
-                            for (int qq = 1; qq < S; ++qq) if (q == uint32_t(qq)) { w = ring[ub][qq]; bits = unsafe[qq]; scq = sc[qq]; biq = bi[qq]; }
-                            if (__ballot(bits != 0) == 0) continue;
-                            const float4 fi = *reinterpret_cast<const float4*>(info + first_block + 32 * q);
-                            float v0 = 0, v1 = 0;
-                            if (bits & 1u) v0 = scq * xint_literal_dot(expand(w.x, w.y), src, first_block + 32 * q) + fi.y * biq;
-                            if (bits & 2u) v1 = scq * xint_literal_dot(expand(w.z, w.w), src, first_block + 32 * q + 1) + fi.w * biq;
-#pragma unroll
-                            for (int qq = 0; qq < S; ++qq) if (q == uint32_t(qq)) {
-                                if (bits & 1u) term[qq][0] = v0;
-                                if (bits & 2u) term[qq][1] = v1;
-                            }
-                        }
-                    }
-                    float acc0 = 0, acc1 = 0;
-#pragma unroll
-                    for (int q = 0; q < S; ++q) { acc0 += term[q][0]; acc1 += term[q][1]; }
-                    *reinterpret_cast<float2*>(part + nb * 512 + (m * 64 + lane) * 2) = make_float2(acc0, acc1);
-                    if (m == 0 && lane == 0) { meta[2 * nb] = i; meta[2 * nb + 1] = tag; }
-                    if (++nb == kXintBatch) flush();
-                }
-            }
-            issue(ub, min(i + UB, count - 1));   // the slot refills while the next tiles are multiplied
-        }
-    }
-    if (nb) flush();
-}
-
 }  // namespace zc

@@ -70,9 +70,10 @@ struct Barrier {
 
 // Copies `pairs` pairs of fp32 values written by other workgroups into LDS as BF16 (high
 // halves), eight coherent 8-byte loads in flight per thread; returns whether any value
-// had low mantissa bits.  transform(pair index, a, b) may rescale the two values first.
-template <class Transform>
-__device__ __forceinline__ int stage_bf16(const float* src, uint32_t pairs, uint32_t* dst, Transform transform) {
+// had low mantissa bits.  transform(pair index, a, b) may rescale the two values first;
+// ready() runs once, after the first loads have been issued and before any value is used.
+template <class Ready, class Transform>
+__device__ __forceinline__ int stage_bf16(const float* src, uint32_t pairs, uint32_t* dst, Ready ready, Transform transform) {
     int inexact = 0;
     for (uint32_t base = 0; base < pairs; base += blockDim.x * 8) {
         uint64_t v[8];
@@ -81,6 +82,7 @@ __device__ __forceinline__ int stage_bf16(const float* src, uint32_t pairs, uint
             const uint32_t i = base + u * blockDim.x + threadIdx.x;
             v[u] = i < pairs ? __hip_atomic_load(reinterpret_cast<const uint64_t*>(src) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
         }
+        if (base == 0) ready();
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const uint32_t i = base + u * blockDim.x + threadIdx.x;
@@ -94,6 +96,23 @@ __device__ __forceinline__ int stage_bf16(const float* src, uint32_t pairs, uint
         }
     }
     return inexact;
+}
+// Copies `count` 8-byte words written by other workgroups into LDS, DEPTH coherent loads in flight per thread.
+template <int DEPTH>
+__device__ __forceinline__ void stage_copy(const uint64_t* src, uint32_t count, uint64_t* dst) {
+    for (uint32_t base = 0; base < count; base += blockDim.x * DEPTH) {
+        uint64_t v[DEPTH];
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            const uint32_t i = base + u * blockDim.x + threadIdx.x;
+            v[u] = i < count ? __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+        }
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            const uint32_t i = base + u * blockDim.x + threadIdx.x;
+            if (i < count) dst[i] = v[u];
+        }
+    }
 }
 
 // Top-k of one token by one wavefront.  Lane l holds experts l*per .. l*per+per-1, so the
@@ -178,6 +197,15 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };   // after the slowest wave of the workgroup
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
+    // SwiGLU of a finished gate/up tile (gate rows in columns 0-7, up rows in 8-15), stored as packed BF16 pairs:
+    // the lane of an even row writes rows r and r+1 of activation row `slot_row` as one word.
+    auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {
+        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+        const uint32_t a = __float_as_uint(swiglu_bf(v, up));
+        const uint32_t other = uint32_t(__shfl_xor(int(a), 1));
+        if (lane < 8 && !(lane & 1u))
+            ZC_ST(reinterpret_cast<uint32_t*>(buffer) + (uint64_t(slot_row) * I + row) / 2, (a >> 16) | (other & 0xffff0000u));
+    };
 
     for (uint32_t layer = 0; layer < p.L; ++layer) {
         const DecodeLayer L = p.layers[layer];
@@ -186,22 +214,39 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
         __syncthreads();
         {
             uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
-            if (layer && tid < T) {   // the glue's scale per token, kept where the gate values go later
-                const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
-                gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
-            }
-            __syncthreads();
             const bool glue = layer != 0;
+            // the glue's scale per token, 1 / max|y| of the previous layer: one token fetches it together with the row,
+            // several tokens go through LDS (one more round trip, fewer registers)
+            uint32_t peak = 0; float inv = 1.0f;
+            if constexpr (NT == 1) {
+                if (glue) peak = ZC_LD(p.maxabs + (layer - 1) * T);
+            } else {
+                if (glue && tid < T) {
+                    const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
+                    gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+                }
+                __syncthreads();
+            }
             // the shared-expert gate row rides along: coalesced sixteen-byte loads, used from LDS by the gate-dot waves
             uint4 gate_piece[2];
 #pragma unroll
-            for (int q = 0; q < 2; ++q) if (tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
-            const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), [&](uint32_t i, float& a, float& b) {
-                if (glue) { const float inv = gatev[(2 * i) / H]; a = bf(a * inv); b = bf(b * inv); }
-            });
+            for (int q = 0; q < 2; ++q) if (NT == 1 && tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
+            const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh),
+                [&]() {
+                    if constexpr (NT == 1) { const float m = __uint_as_float(peak); inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f; }
+                },
+                [&](uint32_t i, float& a, float& b) {
+                    if (glue) {
+                        const float scale = NT == 1 ? inv : gatev[(2 * i) / H];
+                        a = bf(a * scale); b = bf(b * scale);
+                    }
+                });
             if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
 #pragma unroll
-            for (int q = 0; q < 2; ++q) if (tid + q * kDecodeThreads < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
+            for (int q = 0; q < 2; ++q) if (tid + q * kDecodeThreads < H / 8) {
+                if constexpr (NT != 1) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);   // several tokens: after the rows, to spare registers
+                reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
+            }
         }
         __syncthreads();
         xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
@@ -265,10 +310,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                             const uint32_t tt = t0 + t < T ? t0 + t : 0;
                             img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
                         }
-                        auto emit = [&](int t, float v) {
-                            const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
-                            if (G == 0 && col < 8) st_f32(p.shared_act + uint64_t(t0 + t) * I + row, swiglu_bf(v, up));
-                        };
+                        auto emit = [&](int t, float v) { store_act(p.shared_act, t0 + t, row, v); };
                         ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, int(min(uint32_t(PT), T - t0)), emit);
                     }
                 } else {
@@ -293,7 +335,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
             if (E == 512) route_token<8>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
             else route_token<16>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
         }
-        if (tid < T) gatev[tid] = load_shared_f32(p.gate + tid);
+        if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
         for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
         __syncthreads();
         clock();
@@ -342,10 +384,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                         const uint32_t tt = t < nt ? uint32_t(slot[t]) / k : 0;
                         img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
                     }
-                    auto emit = [&](int t, float v) {
-                        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
-                        if (G == 0 && col < 8) st_f32(p.act + uint64_t(slot[t]) * I + row, swiglu_bf(v, up));
-                    };
+                    auto emit = [&](int t, float v) { store_act(p.act, uint32_t(slot[t]), row, v); };
                     ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, nt, emit);
                 }
             }
@@ -364,9 +403,9 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
                 {   // rows s0 .. s0+sn-1 of [act ; shared_act]: contiguous except across the seam between the two buffers
                     const uint32_t routed = s0 < n ? min(sn, n - s0) : 0;
-                    if (routed) stage_bf16(p.act + uint64_t(s0) * I, routed * I / 2, reinterpret_cast<uint32_t*>(ah), [](uint32_t, float&, float&) {});
-                    if (sn > routed) stage_bf16(p.shared_act + uint64_t(s0 + routed - n) * I, (sn - routed) * I / 2,
-                                                reinterpret_cast<uint32_t*>(ah + routed * I), [](uint32_t, float&, float&) {});
+                    if (routed) stage_copy<NT == 1 ? 12 : 6>(reinterpret_cast<const uint64_t*>(p.act) + uint64_t(s0) * I / 4, routed * I / 4, reinterpret_cast<uint64_t*>(ah));
+                    if (sn > routed) stage_copy<NT == 1 ? 12 : 6>(reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(s0 + routed - n) * I / 4, (sn - routed) * I / 4,
+                                                reinterpret_cast<uint64_t*>(ah + routed * I));
                 }
                 __syncthreads();
                 auto source_of = [&](uint32_t q) { return LdsBf16{ah + q * I}; };
@@ -410,15 +449,21 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 float partial[8];
 #pragma unroll
                 for (int q = 0; q < 8; ++q) partial[q] = 0;
-                for (uint32_t kk = 0; kk < k; ++kk) {
-                    const int32_t e = ids[t * k + kk];
-                    const float value = (e >= 0 && e < int32_t(E)) ? otile[(t * k + kk) * 16 + c] : 0.0f;
-                    const float product = value * weights[t * k + kk];
-                    if (kk < 8) partial[kk] = product; else partial[kk % 8] = partial[kk % 8] + product;
+                for (uint32_t base = 0; base < k; base += 8) {   // eight independent products at a time, partial j takes slots j, j+8, ...
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t kk = base + j;
+                        if (kk < k) {
+                            const int32_t e = ids[t * k + kk];
+                            const float value = (e >= 0 && e < int32_t(E)) ? otile[(t * k + kk) * 16 + c] : 0.0f;
+                            const float product = value * weights[t * k + kk];
+                            partial[j] = base == 0 ? product : partial[j] + product;
+                        }
+                    }
                 }
                 float sum = partial[0];
                 for (uint32_t kk = 1; kk < 8 && kk < k; ++kk) sum += partial[kk];
-                const float g = bf(sigmoid_bf(gatev[t]));
+                const float g = gatev[t];
                 const float y = bf(bf(sum) + bf(g * otile[(n + t) * 16 + c]));
                 const uint64_t at = uint64_t(t) * H + rt * 16 + c;
                 st_f32(p.layer_out + at, y);

@@ -74,6 +74,13 @@ struct LdsF32 {      // fp32 copy of an arbitrary row
 
 // Builds one 16-block `b` of an image: digit planes, {2^e, bias sum}, unsafe bit.
 // The image's mask words must have been zeroed (xint_prepare_begin) before.
+//
+// e = exponent field of the smallest non-zero magnitude; every element times 2^(134-e) is then
+// an integer X (8-bit significand shifted left by its exponent distance), obtained with one
+// exact scaling and one conversion.  The block is safe when 15 * sum|X| < 2^24, i.e.
+// sum|X| <= 1118481: that bound also keeps every |X| below 2^21 (three digit planes), rules out
+// infinities and NaN (the sum is then not below the bound), and exponent distances above 13.
+// A block whose smallest element is subnormal is left to the literal chain.
 template <class Source>
 __device__ __forceinline__ void xint_prepare_block(const Source x, const XintLayout L, uint8_t* lds, uint32_t b) {
     uint8_t* planes = lds;
@@ -81,44 +88,56 @@ __device__ __forceinline__ void xint_prepare_block(const Source x, const XintLay
     uint32_t* mask = reinterpret_cast<uint32_t*>(lds + L.planes_bytes() + L.info_bytes());
     uint32_t bits[16];
     x.block(b, bits);
-    // bias sum: BF16 rounding after each addition of four inputs (reference: qwen.metal:55)
+    // bias sum: BF16 rounding after each addition of four inputs (reference: qwen.metal:55).  For BF16-valued
+    // inputs the rounding needs no NaN case: a NaN keeps being a NaN under the integer form of the rounding.
+    auto round16 = [](float v) {
+        if constexpr (Source::kExactProducts) {
+            const uint32_t u = __float_as_uint(v);
+            return __uint_as_float((u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u);
+        } else {
+            return bf(v);
+        }
+    };
     float sum = 0;
 #pragma unroll
     for (int i = 0; i < 16; i += 4)
-        sum += bf(bf(bf(__uint_as_float(bits[i]) + __uint_as_float(bits[i + 1])) + __uint_as_float(bits[i + 2])) + __uint_as_float(bits[i + 3]));
-    uint32_t emin = 255, lowbits = 0, special = 0;
+        sum += round16(round16(round16(__uint_as_float(bits[i]) + __uint_as_float(bits[i + 1])) + __uint_as_float(bits[i + 2])) + __uint_as_float(bits[i + 3]));
+    // smallest non-zero magnitude: (bits << 1) - 1 wraps zeros to the top of the unsigned range
+    uint32_t tmin = 0xffffffffu, lowbits = 0;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const uint32_t e = (bits[i] >> 23) & 255u, m = bits[i] & 0x7fffffu;
-        lowbits |= bits[i] & 0xffffu;
-        special |= (e == 255u);
-        if (e | m) emin = min(emin, max(e, 1u));
+        tmin = min(tmin, (bits[i] << 1) - 1u);
+        if constexpr (!Source::kExactProducts) lowbits |= bits[i] & 0xffffu;
     }
-    if (emin == 255) emin = 1;   // all zero
-    uint32_t sumabs = 0, over = 0;
-    uint32_t mag[16];
+    const uint32_t smallest = tmin + 1u;                 // (bits << 1) of that element, 0 when the block is all zeros
+    const bool subnormal = smallest != 0u && smallest < (1u << 24);
+    const uint32_t emin = max(smallest >> 24, 1u);
+    // integers on the common exponent, and the sum of their magnitudes (exact while it matters)
+    int32_t xs[16];
+    float sumabs = 0;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const uint32_t e = (bits[i] >> 23) & 255u;
-        const uint32_t sig = ((e ? 128u : 0u) | ((bits[i] >> 16) & 127u));
-        const uint32_t shift = sig ? max(e, 1u) - emin : 0u;   // zeros put no demand on the range
-        over |= (shift > 13u);
-        mag[i] = sig << min(shift, 13u);
-        sumabs += mag[i];
+        const float scaled = __builtin_ldexpf(__uint_as_float(bits[i]), 134 - int(emin));
+        sumabs += __builtin_fabsf(scaled);
+        xs[i] = int32_t(scaled);
     }
-    const bool safe = !lowbits && !special && !over && 15u * sumabs < (1u << 24);
+    const bool safe = !lowbits && !subnormal && sumabs <= 1118481.0f;
     // digits of the signed integer Xs in two's complement: Xs = d0 + 2^7 d1 + 2^14 d2 with
-    // d0, d1 in [0,127] and d2 = Xs >> 14 in [-128,127] (|Xs| < 2^21)
-    uint32_t words[3][4] = {};
+    // d0, d1 in [0,127] and d2 = Xs >> 14 in [-128,127]
+    uint32_t words[3][4];
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-        const uint32_t i = xint_element_of_byte(t);
-        const int32_t xs = (bits[i] >> 31) ? -int32_t(mag[i]) : int32_t(mag[i]);
-        words[0][t / 4] |= (uint32_t(xs) & 127u) << (8 * (t % 4));
-        words[1][t / 4] |= ((uint32_t(xs) >> 7) & 127u) << (8 * (t % 4));
-        words[2][t / 4] |= ((uint32_t(xs) >> 14) & 255u) << (8 * (t % 4));
+    for (int j = 0; j < 4; ++j) {
+        uint32_t w0 = 0, w1 = 0, w2 = 0;
+#pragma unroll
+        for (int q = 3; q >= 0; --q) {
+            const uint32_t v = uint32_t(xs[xint_element_of_byte(4 * j + q)]);
+            w0 = (w0 << 8) | (v & 127u);
+            w1 = (w1 << 8) | ((v >> 7) & 127u);
+            w2 = (w2 << 8) | ((v >> 14) & 255u);
+        }
+        words[0][j] = safe ? w0 : 0u; words[1][j] = safe ? w1 : 0u; words[2][j] = safe ? w2 : 0u;
     }
-    if (!safe) { for (int p = 0; p < 3; ++p) for (int q = 0; q < 4; ++q) words[p][q] = 0; atomicOr(mask + b / 32, 1u << (b % 32)); }
+    if (!safe) atomicOr(mask + b / 32, 1u << (b % 32));
 #pragma unroll
     for (int p = 0; p < 3; ++p)
         *reinterpret_cast<uint4*>(planes + b * 48 + p * 16) = make_uint4(words[p][0], words[p][1], words[p][2], words[p][3]);

@@ -21,6 +21,9 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
+# HBM bytes per launch of the default workload (48 layers, batch 1) from the FETCH_SIZE / WRITE_SIZE counter runs summarised
+# in profiles/decode_stack_kernel_F48_batch1_pmc.txt (counters cannot be read from inside this process).
+MEASURED_TRAFFIC = 2_989_960_000
 sys.path.insert(0, ROOT)
 
 
@@ -33,6 +36,7 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extra", action="store_true", help="also time decode batch 8 and the single-layer configurations")
+    ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
@@ -57,6 +61,12 @@ def main():
         ids, w = ctx.alloc(L * n * 4), ctx.alloc(L * n * 4)
         ctx.stack_decode(stack, x, tokens, out, z.StackTrace(ids.ptr, w.ptr, None, None))
         ctx.moe_check()
+        # parity gate before any timing: the single-launch kernel and the layer-by-layer operator path must agree byte for byte
+        fused = out.numpy(np.float32).tobytes()
+        ctx.stack_decode(stack, x, tokens, out, layered=True)
+        ctx.moe_check()
+        if out.numpy(np.float32).tobytes() != fused:
+            raise SystemExit("bench.py: persistent kernel and layer-by-layer path disagree; refusing to time")
         unique = [len(np.unique(r)) for r in ids.numpy(np.int32).reshape(L, n)]
         nbytes = sum(workload.layer_bytes(cfg, u, tokens, ctx) for u in unique)
         for _ in range(warmup):
@@ -71,6 +81,13 @@ def main():
             ctx.free(b)
         return ms, nbytes, unique
 
+    if args.calibrate:
+        gib = 1 << 30
+        a, b = ctx.alloc(gib), ctx.alloc(gib)
+        ctx.fill(a, 1)
+        ctx.copy(b, a, gib)
+        ctx.finish()
+        ctx.free(a); ctx.free(b)
     ms, nbytes, unique = run(T, args.steps, args.warmup)
     persistent = ctx.stack_is_persistent(stack, T)
     achieved = nbytes / (ms * 1e-3) / 1e9
@@ -84,9 +101,10 @@ def main():
                                "Zipf(1.1) router offsets, one seed per layer",
                    "layers": L, "decode_batch": T, "hbm_resident_bytes": int(ctx.allocated),
                    "distinct_experts_per_layer": float(np.mean(unique)),
-                   "path": "persistent single-launch kernel" if persistent else "layer by layer"},
+                   "path": "persistent single-launch kernel" if persistent else "layer by layer",
+                   "parity_gate": "output bytes equal the layer-by-layer operator path on this input (checked before timing)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s", "frac": achieved / 8000.0,
-                     "traffic": None, "kernel": "zc::decode_stack_kernel (one launch = one step)",
+                     "traffic": MEASURED_TRAFFIC if (L, T) == (48, 1) else None, "kernel": "zc::decode_stack_kernel (one launch = one step)",
                      "algorithmic_bytes_per_launch": int(nbytes), "launch_us": ms * 1e3},
     }
 

@@ -126,6 +126,10 @@ class Context:
     def fill(self, buf, byte):
         self._call("zc_hip_memset", _ptr(buf), C.c_int(byte), C.c_uint64(buf.nbytes))
 
+    def copy(self, dst, src, nbytes):
+        """Device-to-device copy on the context's stream."""
+        self._call("zc_hip_copy", _ptr(dst), _ptr(src), C.c_uint64(nbytes))
+
     def upload(self, array, into=None):
         a = np.ascontiguousarray(array)
         b = into or self.alloc(max(a.nbytes, 4))

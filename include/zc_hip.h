@@ -181,6 +181,45 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* stack, const float*
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* stack, uint32_t tokens);
 zc_status zc_hip_stack_glue(zc_hip_ctx* ctx, const float* y, uint32_t tokens, uint32_t hidden, float* x_next);
 
+/* ---- Expert store: ExpertStore + ExpertCache (include/engine/storage.hpp:168-269; src/engine/storage.cpp:493-725)
+ * with the SSD replaced by pinned host memory and the slots living in HBM.  Every record has a home in pinned host
+ * memory (zc_hip_store_backing: write the record there before its first use); `slots` HBM slots cache the records in
+ * use and are filled by hipMemcpyAsync on the store's own side stream.  The rules are the reference's: a lease pins
+ * its slot until it is released (release it only after the GPU work that reads the slot has finished, e.g. after
+ * zc_hip_wait on a later ticket); victims are chosen by CLOCK second chance and are never pinned or still loading;
+ * prefetch() fills speculatively without a lease and never evicts a pinned or loading slot; counters as
+ * CacheStats (storage.hpp:183-192).  With slots >= layers * experts the store is HBM-resident after the first touch.
+ * A NULL context gives a store with host-memory slots whose fills can be held back (zc_hip_store_hold): the
+ * policy, loading joins included, can then be tested without a GPU.  One coordinator thread owns a store. */
+typedef struct zc_hip_store zc_hip_store;
+typedef struct { uint64_t hits, misses, evictions, bytes, ready_hits, loading_joins, prefetches, prefetch_claims, prefetch_unclaimed; } zc_store_stats;
+typedef struct {
+    uint64_t lease;      /* pass to wait / release */
+    void* record;        /* the slot: device address of the record (valid for GPU work enqueued after zc_hip_store_wait) */
+    int32_t acquisition; /* 0 new miss, 1 ready hit, 2 loading join (Lease::acquisition, storage.cpp:600-602) */
+} zc_store_lease;
+zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots, zc_hip_store** out);
+zc_status zc_hip_store_destroy(zc_hip_store* store);
+void* zc_hip_store_backing(zc_hip_store* store, uint32_t layer, uint32_t expert);   /* HOST pointer: the record's home */
+uint64_t zc_hip_store_stride(const zc_hip_store* store);
+uint64_t zc_hip_store_capacity(const zc_hip_store* store);
+uint64_t zc_hip_store_occupancy(const zc_hip_store* store);
+/* ExpertCache::acquire (storage.cpp:628-676).  ZC_RUNTIME_ERROR "expert cache exhausted by outstanding leases; ..." when
+ * every slot is pinned or loading. */
+zc_status zc_hip_store_acquire(zc_hip_store* store, uint32_t layer, uint32_t expert, zc_store_lease* out);
+/* Lease::wait (storage.cpp:588-591) without blocking the host: the context's stream waits for the slot's fill. */
+zc_status zc_hip_store_wait(zc_hip_store* store, uint64_t lease);
+zc_status zc_hip_store_release(zc_hip_store* store, uint64_t lease);   /* Lease::~Lease */
+/* ExpertCache::prefetch (storage.cpp:677-692): *issued = 0 when the record is present or no slot is free to take. */
+zc_status zc_hip_store_prefetch(zc_hip_store* store, uint32_t layer, uint32_t expert, int* issued);
+int zc_hip_store_ready(zc_hip_store* store, uint32_t layer, uint32_t expert);   /* ExpertCache::ready */
+zc_status zc_hip_store_clear(zc_hip_store* store);                    /* ZC_LOGIC_ERROR while a lease is out */
+zc_status zc_hip_store_resize(zc_hip_store* store, uint64_t slots);   /* survivors keep their bytes; ZC_LOGIC_ERROR while a lease is out */
+zc_status zc_hip_store_stats(const zc_hip_store* store, zc_store_stats* out);
+zc_status zc_hip_store_layer_stats(const zc_hip_store* store, uint32_t layer, uint64_t* hits, uint64_t* misses);
+/* Stores without a context only: fills of this record stay "loading" while held (what a slow read is to the reference's tests). */
+zc_status zc_hip_store_hold(zc_hip_store* store, uint32_t layer, uint32_t expert, int hold);
+
 /* Counter-based synthetic tensors: element i depends only on (seed, i).
  * kind 0: uint32 words of uniform bits (Q4/Q8 codes), count = words
  * kind 1: BF16 scale in [lo, lo+span) and BF16 bias = scale*factor, interleaved

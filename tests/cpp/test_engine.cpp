@@ -214,8 +214,54 @@ static void test_moe_layer() {   // model.cpp:431-557 against the CPU oracle
     CHECK_THROWS(moe_resident(gpu, w, records, stride, x, 1));
     gpu.budget(gpu.allocated() + 16); CHECK_THROWS(gpu.allocate(1 << 20)); gpu.budget(0);   // "engine memory budget exceeded"
 }
+static void test_expert_cache() {   // :336-348 on the GPU, and moe() reading its records through leases
+    TEST("expert cache: leases pin HBM slots; a layer through a few slots equals the resident layer");
+    const MoeShape s = small_shape(); Metal gpu(s);
+    ExpertCache cache(gpu, 1, s.topk + 2);
+    const uint64_t stride = (s.expert_bytes() + 255) / 256 * 256;
+    std::vector<std::byte> all(stride * s.experts);
+    for (uint32_t e = 0; e < s.experts; ++e) {
+        auto r = expert_fixture(s, 300 + e);
+        std::memcpy(all.data() + e * stride, r.data(), r.size());
+        std::memcpy(cache.home({0, e}).data(), r.data(), r.size());
+    }
+    {
+        std::vector<ExpertCache::Lease> leases;
+        for (uint32_t e = 0; e < s.topk + 2; ++e) leases.push_back(cache.acquire({0, e}));
+        CHECK_THROWS(cache.acquire({0, s.topk + 2}));   // "expert cache exhausted by outstanding leases; ..."
+        CHECK_THROWS(cache.clear()); CHECK_THROWS(cache.resize(64));
+        CHECK(std::string(leases[0].acquisition()) == "new_miss");
+        auto again = cache.acquire({0, 0});
+        CHECK(std::string(again.acquisition()) != "new_miss"); CHECK(again.wait()->metal == leases[0].wait()->metal);
+        CHECK((leases[3].key() == ExpertKey{0, 3}));
+    }
+    CHECK_THROWS(cache.acquire({0, s.experts})); CHECK_THROWS(cache.acquire({1, 0}));
+    auto shared_host = expert_fixture(s, 7, true);
+    auto records = to_hbm(gpu, all); auto shared_record = to_hbm(gpu, shared_host);
+    std::vector<uint16_t> router(size_t(s.experts) * s.hidden), sgate(s.hidden);
+    for (size_t i = 0; i < router.size(); ++i) router[i] = uint16_t(std::bit_cast<uint32_t>(round_bf16(float(int((i * 2246822519u >> 9) % 401) - 200) / 4096)) >> 16);
+    for (size_t i = 0; i < sgate.size(); ++i) sgate[i] = uint16_t(std::bit_cast<uint32_t>(round_bf16(float(int(i % 29) - 14) / 512)) >> 16);
+    auto router_buf = gpu.allocate(router.size() * 2, AllocationClass::Resident), sgate_buf = gpu.allocate(sgate.size() * 2, AllocationClass::Resident);
+    gpu.write(router_buf, 0, std::as_bytes(std::span(router))); gpu.write(sgate_buf, 0, std::as_bytes(std::span(sgate)));
+    MoeLayerWeights w;
+    w.router = Linear{{router_buf}, {}, {}, s.hidden, s.experts, 64, 0, false};
+    w.shared_gate = Linear{{sgate_buf}, {}, {}, s.hidden, 1, 64, 0, false};
+    w.shared_record = shared_record;
+    std::vector<ExpertCache::Lease> held;      // pinned until the layer's GPU work has finished
+    w.record = [&](uint32_t e) { held.push_back(cache.acquire({0, e})); return held.back().wait(); };
+    for (uint32_t step = 0; step < 6; ++step) {
+        auto x = gpu.zeros(s.hidden);
+        for (size_t i = 0; i < x->floats().size(); ++i) x->floats()[i] = round_bf16(float(int(((i * 40503u + step * 977u) >> 3) % 255) - 127) / 64);
+        auto a = moe(gpu, w, x, 1); gpu.finish(); held.clear();
+        auto b = moe_resident(gpu, w, records, stride, x, 1);
+        CHECK(std::memcmp(a->data, b->data, a->bytes) == 0);
+    }
+    const auto st = cache.stats();
+    CHECK(st.misses >= s.topk); CHECK(st.hits + st.misses >= 6 * s.topk); CHECK(st.bytes == st.misses * s.expert_bytes());
+    cache.clear(); CHECK(cache.occupancy() == 0);
+}
 int main() {
-    test_bf16(); test_q4_matmul(); test_route(); test_moe_sum(); test_direct_rows(); test_grouped(); test_heavy_rows(); test_moe_layer();
+    test_bf16(); test_q4_matmul(); test_route(); test_moe_sum(); test_direct_rows(); test_grouped(); test_heavy_rows(); test_moe_layer(); test_expert_cache();
     std::printf("%d checks, %d failures\n", checks, failures);
     return failures ? 1 : 0;
 }

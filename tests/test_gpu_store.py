@@ -1,0 +1,83 @@
+"""Expert store on the GPU: records travel from their pinned-host home into HBM slots on the side stream, and a layer
+computed through a small number of slots equals the layer computed from HBM-resident records byte for byte."""
+import numpy as np
+import pytest
+import zerocool_amd as z
+from zerocool_amd import workload
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = z.Context(0)
+    yield c
+    c.close()
+
+
+def test_slots_hold_the_records_they_were_asked_for(ctx):
+    record, experts = 4096 + 64, 40
+    s = z.Store(ctx, 2, experts, record, 4)
+    rng = np.random.default_rng(5)
+    for l in range(2):
+        for e in range(experts):
+            s.backing(l, e)[:] = rng.integers(0, 256, record, dtype=np.uint8)
+    for step in range(200):
+        l, e = int(rng.integers(0, 2)), int(rng.integers(0, experts))
+        lease = s.acquire(l, e)
+        slot = s.wait(lease)
+        got = slot.numpy(np.uint8)          # a download on the compute stream: ordered after the fill by the wait above
+        assert got.tobytes() == s.backing(l, e).tobytes(), (step, l, e)
+        s.release(lease)
+    st = s.stats()
+    assert st.hits + st.misses == 200 and st.evictions >= st.misses - 4 and st.bytes == st.misses * record
+    assert sum(s.layer_stats(l)[1] for l in range(2)) == st.misses
+    with pytest.raises(z.ZcError):
+        s.hold(0, 0)                        # only stores without a context can hold fills back
+    s.close()
+
+
+def test_leases_pin_slots_on_the_gpu(ctx):
+    s = z.Store(ctx, 1, 8, 1024, 2)
+    for e in range(8):
+        s.backing(0, e)[:] = e + 1
+    a, b = s.acquire(0, 0), s.acquire(0, 1)
+    with pytest.raises(z.ZcError) as err:
+        s.acquire(0, 2)
+    assert "exhausted by outstanding leases" in str(err.value)
+    s.release(b)
+    c = s.acquire(0, 2)
+    assert s.wait(a).numpy(np.uint8)[0] == 1 and s.wait(c).numpy(np.uint8)[0] == 3
+    s.release(a); s.release(c)
+    assert s.prefetch(0, 5) is True
+    ctx.finish()
+    hit = s.acquire(0, 5)
+    assert hit.acquisition in (1, 2) and s.stats().prefetch_claims == 1
+    assert s.wait(hit).numpy(np.uint8)[0] == 6
+    s.release(hit)
+    s.resize(4)
+    assert s.ready(0, 5) and s.wait(s.acquire(0, 5)).numpy(np.uint8)[0] == 6   # survivors keep their bytes across a resize
+    s.close()
+
+
+@pytest.mark.parametrize("tokens", [1, 5])
+def test_layer_through_capped_slots_equals_resident_layer(ctx, tokens):
+    cfg = workload.tiny_config(hidden=512, experts=32, topk=4, inter=128)
+    seeds = [41, 42]
+    capped = workload.StoreBackedStack(ctx, cfg, seeds, ("normal", 0.5), slots=6)   # 64 records, six slots
+    for l, seed in enumerate(seeds):
+        resident = workload.LayerWeights(ctx, cfg, seed, ("normal", 0.5))
+        for step in range(3):
+            x = workload.hidden_rows(ctx, tokens, cfg.hidden, 900 + 10 * l + step)
+            want = ctx.alloc(tokens * cfg.hidden * 4)
+            ws = ctx.alloc(ctx.moe_workspace_bytes(cfg, tokens))
+            ids = ctx.alloc(tokens * cfg.topk * 4)
+            ctx.moe_forward(cfg, resident.layer, x, tokens, want, ws, z.Trace(None, ids.ptr, None, None, None, None))
+            ctx.moe_check()
+            got, host_ids = capped.layer_forward(l, x, tokens)
+            assert host_ids.tobytes() == ids.numpy(np.int32).tobytes()
+            assert got.numpy(f32).tobytes() == want.numpy(f32).tobytes()
+    st = capped.store.stats()
+    assert st.misses > 6 and st.evictions > 0 and st.hits + st.misses > 0
+    capped.close()

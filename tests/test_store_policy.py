@@ -1,0 +1,182 @@
+"""Slot-cache policy of the expert store, on a store with host-memory slots (no GPU): the reference's cache tests
+(tests/test_qwen.cpp:93-100, 336-348, 415-430) restated through the C ABI, plus the prefetch rules of
+ExpertCache::prefetch (src/engine/storage.cpp:677-692)."""
+import numpy as np
+import pytest
+import zerocool_amd as z
+
+RECORD = 128
+
+
+def make(slots, layers=2, experts=512):
+    s = z.Store(None, layers, experts, RECORD, slots)
+    return s
+
+
+def put(s, layer, expert):
+    s.backing(layer, expert)[:] = np.frombuffer(np.full(RECORD // 4, float(layer * s.experts + expert), np.float32).tobytes(), np.uint8)
+
+
+def value(s, lease):
+    return float(s.slot_bytes(lease).view(np.float32)[0])
+
+
+def use(s, layer, expert):
+    put(s, layer, expert)
+    lease = s.acquire(layer, expert)
+    s.wait(lease)
+    v = value(s, lease)
+    s.release(lease)
+    return v
+
+
+def test_clock_leases_protect_in_flight_data():   # test_qwen.cpp:336-348
+    s = make(2)
+    put(s, 0, 1); put(s, 0, 2); put(s, 0, 3)
+    a, b = s.acquire(0, 1), s.acquire(0, 2)
+    s.wait(a); s.wait(b)
+    assert value(s, a) == 1 and value(s, b) == 2
+    with pytest.raises(z.ZcError) as err:
+        s.acquire(0, 3)
+    assert "exhausted by outstanding leases" in str(err.value)
+    with pytest.raises(z.ZcError):
+        s.clear()
+    with pytest.raises(z.ZcError):
+        s.resize(4)
+    s.release(b)
+    c = s.acquire(0, 3); s.wait(c)
+    assert value(s, c) == 3 and value(s, a) == 1
+    hit = s.acquire(0, 1)
+    assert hit.record == a.record and hit.acquisition == 1
+    for lease in (hit, a, c):
+        s.release(lease)
+    s.resize(4)
+    for i in range(32):
+        assert use(s, 1, i % 8) == 512 + i % 8
+    assert s.stats().evictions > 0
+    with pytest.raises(z.ZcError):
+        s.release(a)   # released twice
+    s.close()
+
+
+def test_resizing_preserves_survivors_and_refuses_leases():   # test_qwen.cpp:93-100
+    s = make(64)
+    for i in range(64):
+        use(s, 0, i)
+    assert s.occupancy == 64
+    lease = s.acquire(0, 63)
+    with pytest.raises(z.ZcError):
+        s.resize(32)
+    assert s.capacity == 64
+    s.release(lease)
+    s.resize(32)
+    assert s.capacity == 32 and s.occupancy == 32 and s.stats().evictions == 32
+    assert s.ready(0, 63)
+    misses = s.stats().misses
+    assert use(s, 0, 63) == 63 and s.stats().misses == misses   # a survivor keeps its bytes: a hit, not a reload
+    s.close()
+
+
+def test_loading_joins_count_separately():   # test_qwen.cpp:415-430
+    s = make(3)
+    put(s, 0, 0)
+    s.hold(0, 0)
+    a = s.acquire(0, 0)
+    join = s.acquire(0, 0)
+    st = s.stats()
+    assert st.loading_joins == 1 and st.ready_hits == 0 and a.acquisition == 0 and join.acquisition == 2
+    assert not s.ready(0, 0)
+    with pytest.raises(z.ZcError):
+        s.wait(a)           # (a held fill cannot finish; the reference would block here)
+    s.hold(0, 0, False)
+    s.wait(a); s.wait(join)
+    assert a.record == join.record and value(s, a) == 0
+    s.release(a); s.release(join)
+    use(s, 0, 1); use(s, 0, 2)
+    s.resize(2)
+    assert s.stats().evictions == 1
+    assert sum(s.ready(0, e) for e in range(3)) == 2
+    before = s.stats().misses
+    s.resize(4)
+    for e in range(3):
+        if s.ready(0, e):
+            assert use(s, 0, e) == e
+    assert s.stats().misses == before
+    s.close()
+
+
+def test_loading_slots_are_never_victims():
+    s = make(2)
+    put(s, 0, 0); put(s, 0, 1); put(s, 0, 2)
+    s.hold(0, 0)
+    a = s.acquire(0, 0)
+    s.release(a)                       # lease gone, but the fill is still in flight: the slot must not be taken
+    use(s, 0, 1)
+    assert use(s, 0, 2) == 2           # takes the slot of expert 1 (finished), not the loading one
+    assert not s.ready(0, 1)
+    s.hold(0, 0, False)
+    hit = s.acquire(0, 0)
+    assert hit.acquisition == 1
+    s.wait(hit)
+    assert value(s, hit) == 0
+    s.release(hit)
+    s.close()
+
+
+def test_prefetch_rules():   # storage.cpp:677-692
+    s = make(2)
+    for e in range(4):
+        put(s, 0, e)
+    assert s.prefetch(0, 0) is True
+    assert s.prefetch(0, 0) is False                 # present
+    st = s.stats()
+    assert st.prefetches == 1 and st.misses == 0
+    claimed = s.acquire(0, 0)                        # demand claims the guess: a hit
+    st = s.stats()
+    assert claimed.acquisition == 1 and st.prefetch_claims == 1 and st.hits == 1
+    other = s.acquire(0, 1)
+    assert s.prefetch(0, 2) is False                 # both slots pinned: a guess never evicts a lease
+    s.hold(0, 2)
+    s.release(other)
+    assert s.prefetch(0, 2) is True                  # takes the unpinned, finished slot ...
+    assert s.prefetch(0, 3) is False                 # ... and now one slot is pinned, the other still loading: nothing to take
+    s.hold(0, 2, False)
+    s.release(claimed)
+    s.close()
+
+
+def test_unclaimed_guess_is_the_next_victim():
+    s = make(3)
+    for e in range(4):
+        put(s, 0, e)
+    use(s, 0, 0); use(s, 0, 1)
+    assert s.prefetch(0, 2) is True                  # into the free slot, born unreferenced
+    assert use(s, 0, 3) == 3                         # the sweep gives 0 and 1 their second chance and takes the guess
+    st = s.stats()
+    assert st.prefetch_unclaimed == 1 and st.evictions == 1
+    assert s.ready(0, 0) and s.ready(0, 1) and s.ready(0, 3) and not s.ready(0, 2)
+    s.close()
+
+
+def test_admission_waits_for_a_loading_guess():   # storage.cpp:650-658
+    s = make(1)
+    put(s, 0, 0); put(s, 0, 1)
+    assert s.prefetch(0, 0) is True                  # the only slot holds a guess whose fill has finished
+    lease = s.acquire(0, 1)                          # demand for another record takes it
+    s.wait(lease)
+    assert value(s, lease) == 1 and s.stats().prefetch_unclaimed == 1
+    s.release(lease)
+    s.close()
+
+
+def test_ids_are_checked():
+    s = make(2, layers=1, experts=4)
+    with pytest.raises(z.ZcError) as err:
+        s.acquire(0, 4)
+    assert "invalid expert id" in str(err.value)
+    with pytest.raises(z.ZcError):
+        s.prefetch(1, 0)
+    with pytest.raises(z.ZcError):
+        z.Store(None, 1, 4, RECORD, 0)
+    assert s.layer_stats(0) == (0, 0)
+    s.close()

@@ -285,4 +285,50 @@ Buf moe_resident(Metal& gpu, const MoeLayerWeights& w, const Buf& records, uint6
     return out;
 }
 
+// ---- expert cache (storage.cpp:525-725 over zc_hip_store_*)
+ExpertCache::ExpertCache(Metal& gpu, uint32_t layers, size_t slots) : gpu_(gpu), record_bytes_(gpu.shape().expert_bytes()) {
+    check(zc_hip_store_create(gpu.context(), layers, gpu.shape().experts, record_bytes_, slots, &store_));
+}
+ExpertCache::~ExpertCache() { zc_hip_store_destroy(store_); }
+std::span<std::byte> ExpertCache::home(ExpertKey key) {
+    void* p = zc_hip_store_backing(store_, key.layer, key.expert);
+    if (!p) throw std::out_of_range("invalid expert id");
+    return {static_cast<std::byte*>(p), size_t(record_bytes_)};
+}
+ExpertCache::Lease ExpertCache::acquire(ExpertKey key) {
+    Lease lease;
+    check(zc_hip_store_acquire(store_, key.layer, key.expert, &lease.lease_));
+    lease.store_ = store_; lease.key_ = key;
+    lease.slot_ = std::make_shared<Buffer>();
+    lease.slot_->bytes = record_bytes_; lease.slot_->metal = lease.lease_.record;
+    return lease;
+}
+bool ExpertCache::prefetch(ExpertKey key) { int issued = 0; check(zc_hip_store_prefetch(store_, key.layer, key.expert, &issued)); return issued != 0; }
+bool ExpertCache::ready(ExpertKey key) const { return zc_hip_store_ready(store_, key.layer, key.expert) != 0; }
+void ExpertCache::clear() { check(zc_hip_store_clear(store_)); }
+void ExpertCache::resize(size_t slots) { check(zc_hip_store_resize(store_, slots)); }
+size_t ExpertCache::capacity() const { return zc_hip_store_capacity(store_); }
+size_t ExpertCache::occupancy() const { return zc_hip_store_occupancy(store_); }
+CacheStats ExpertCache::stats() const {
+    zc_store_stats s{}; check(zc_hip_store_stats(store_, &s));
+    return CacheStats{s.hits, s.misses, s.evictions, s.bytes, s.ready_hits, s.loading_joins, s.prefetches, s.prefetch_claims, s.prefetch_unclaimed};
+}
+ExpertCache::Lease::~Lease() { if (store_) zc_hip_store_release(store_, lease_.lease); }
+ExpertCache::Lease::Lease(Lease&& o) noexcept : store_(o.store_), lease_(o.lease_), key_(o.key_), slot_(std::move(o.slot_)) { o.store_ = nullptr; }
+ExpertCache::Lease& ExpertCache::Lease::operator=(Lease&& o) noexcept {
+    if (this != &o) {
+        if (store_) zc_hip_store_release(store_, lease_.lease);
+        store_ = o.store_; lease_ = o.lease_; key_ = o.key_; slot_ = std::move(o.slot_); o.store_ = nullptr;
+    }
+    return *this;
+}
+bool ExpertCache::Lease::ready() const { return store_ && zc_hip_store_ready(store_, key_.layer, key_.expert) != 0; }
+const Buf& ExpertCache::Lease::wait() const {
+    if (!store_) throw std::logic_error("empty expert lease");
+    check(zc_hip_store_wait(store_, lease_.lease));
+    return slot_;
+}
+ExpertKey ExpertCache::Lease::key() const { if (!store_) throw std::logic_error("empty expert lease"); return key_; }
+const char* ExpertCache::Lease::acquisition() const { return lease_.acquisition == 0 ? "new_miss" : lease_.acquisition == 1 ? "ready_hit" : "loading_join"; }
+
 }  // namespace zerocool::engine

@@ -117,6 +117,55 @@ void encode_expert_rows(Metal& gpu, const Buf& record, const Buf& input, const B
                         uint32_t tokens, uint32_t chunk, bool direct, int layer, uint32_t offset,
                         const std::atomic<bool>* cancel = nullptr);
 
+// storage.hpp:168-172, 183-192, 198-269: the expert cache, with the reference's names.  The records' home is pinned host
+// memory (home()), the slots are HBM, fills run on the store's side stream (zc_hip_store_*).  A Lease pins its slot
+// until it is destroyed: keep it until the GPU work that reads the slot has finished, as the reference does.
+struct ExpertKey {
+    uint32_t layer = 0, expert = 0;
+    bool operator==(const ExpertKey&) const = default;
+};
+struct CacheStats {
+    uint64_t hits = 0, misses = 0, evictions = 0, bytes = 0, ready_hits = 0, loading_joins = 0;
+    uint64_t prefetches = 0, prefetch_claims = 0, prefetch_unclaimed = 0;
+};
+class ExpertCache {
+public:
+    class Lease {
+    public:
+        Lease() = default;
+        ~Lease();
+        Lease(Lease&& other) noexcept;
+        Lease& operator=(Lease&& other) noexcept;
+        Lease(const Lease&) = delete;
+        bool ready() const;
+        const Buf& wait() const;            // the compute stream waits for the slot's fill; the host does not block
+        ExpertKey key() const;
+        const char* acquisition() const;    // "new_miss", "ready_hit", "loading_join"
+    private:
+        friend class ExpertCache;
+        zc_hip_store* store_ = nullptr;
+        zc_store_lease lease_{};
+        ExpertKey key_{};
+        Buf slot_;
+    };
+    ExpertCache(Metal& gpu, uint32_t layers, size_t slots);
+    ~ExpertCache();
+    ExpertCache(const ExpertCache&) = delete;
+    std::span<std::byte> home(ExpertKey key);   // where the record lives (pinned host memory): write it before first use
+    Lease acquire(ExpertKey key);
+    bool prefetch(ExpertKey key);
+    bool ready(ExpertKey key) const;
+    void clear();
+    void resize(size_t slots);
+    size_t capacity() const;
+    size_t occupancy() const;
+    CacheStats stats() const;
+private:
+    Metal& gpu_;
+    zc_hip_store* store_ = nullptr;
+    uint64_t record_bytes_ = 0;
+};
+
 // What Model::moe reads through Resident and the expert store for one layer.
 struct MoeLayerWeights {
     Linear router;            // [experts][hidden] BF16, float output (model.cpp:434)

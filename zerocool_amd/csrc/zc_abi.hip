@@ -13,6 +13,10 @@
 namespace {
 thread_local std::string g_error;
 zc_status fail(zc_status code, std::string text) { g_error = std::move(text); return code; }
+}  // namespace
+// Sets the calling thread's error text (shared with the other translation units of the library).
+zc_status zc_fail(zc_status code, const std::string& text) { return fail(code, text); }
+namespace {
 
 #define ZC_HIP(call)                                                                         \
     do {                                                                                     \

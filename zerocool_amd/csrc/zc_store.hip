@@ -1,0 +1,226 @@
+// Expert store: every record has a home in pinned host memory; a fixed pool of HBM slots caches the records in
+// use.  Fills are hipMemcpyAsync on a side stream of the store's own, each followed by an event; a compute stream
+// that is about to read a slot waits on that event (no host blocking).  The policy (which record, which slot)
+// is zc::SlotCache.  With as many slots as records the store is simply HBM-resident after the first touch.
+//
+// A store created without a context keeps its slots in ordinary host memory and finishes a fill when the caller
+// says so (zc_hip_store_hold): the policy can then be tested without a GPU, loading states included.
+#include <hip/hip_runtime.h>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <unordered_set>
+#include <vector>
+#include "../../include/zc_hip.h"
+#include "zc_store.hpp"
+
+zc_status zc_fail(zc_status code, const std::string& text);
+
+struct zc_hip_store {
+    zc_hip_ctx* ctx = nullptr;          // nullptr: host-memory slots
+    uint32_t layers = 0, experts = 0;
+    uint64_t record_bytes = 0, stride = 0;
+    uint8_t* backing = nullptr;         // [layers * experts] records, pinned host memory (or plain, without a context)
+    uint8_t* pool = nullptr;            // [capacity] slots, HBM (or plain host memory)
+    hipStream_t side = nullptr;
+    std::vector<hipEvent_t> filled;     // per slot: recorded after the slot's last fill
+    std::vector<uint64_t> pending;      // host-memory store: per slot, the key of a fill that waits for its release, or ~0
+    std::unordered_set<uint64_t> held;  // host-memory store: keys whose fills wait
+    std::unique_ptr<zc::SlotCache> cache;
+    std::vector<uint64_t> layer_hits, layer_misses;
+};
+
+namespace {
+constexpr uint64_t kNone = ~0ull;
+uint64_t key_of(const zc_hip_store* s, uint32_t layer, uint32_t expert) { return uint64_t(layer) * s->experts + expert; }
+
+template <class F> zc_status guarded(F f) {
+    try { return f(); }
+    catch (const std::invalid_argument& e) { return zc_fail(ZC_INVALID_ARGUMENT, e.what()); }
+    catch (const std::out_of_range& e) { return zc_fail(ZC_OUT_OF_RANGE, e.what()); }
+    catch (const std::logic_error& e) { return zc_fail(ZC_LOGIC_ERROR, e.what()); }
+    catch (const std::exception& e) { return zc_fail(ZC_RUNTIME_ERROR, e.what()); }
+}
+#define ZC_STORE_HIP(call) do { const hipError_t e_ = (call); if (e_ != hipSuccess) throw std::runtime_error(std::string("HIP execution: ") + hipGetErrorString(e_) + " in " #call); } while (0)
+
+void finish_host_fill(zc_hip_store* s, size_t slot) {
+    const uint64_t key = s->pending[slot];
+    if (key == kNone) return;
+    std::memcpy(s->pool + slot * s->stride, s->backing + key * s->stride, s->record_bytes);
+    s->pending[slot] = kNone;
+}
+zc::SlotCache::Hooks hooks_of(zc_hip_store* s) {
+    zc::SlotCache::Hooks h;
+    if (s->ctx) {
+        h.start = [s](size_t slot, uint64_t key) {
+            ZC_STORE_HIP(hipMemcpyAsync(s->pool + slot * s->stride, s->backing + key * s->stride, s->record_bytes, hipMemcpyHostToDevice, s->side));
+            ZC_STORE_HIP(hipEventRecord(s->filled[slot], s->side));
+        };
+        h.done = [s](size_t slot) {
+            const hipError_t e = hipEventQuery(s->filled[slot]);
+            if (e == hipErrorNotReady) return false;
+            ZC_STORE_HIP(e);
+            return true;
+        };
+        h.wait = [s](size_t slot) { ZC_STORE_HIP(hipEventSynchronize(s->filled[slot])); };
+        h.move = [s](size_t from, size_t to) {
+            ZC_STORE_HIP(hipMemcpyAsync(s->pool + to * s->stride, s->pool + from * s->stride, s->record_bytes, hipMemcpyDeviceToDevice, s->side));
+            ZC_STORE_HIP(hipEventRecord(s->filled[to], s->side));
+        };
+    } else {
+        h.start = [s](size_t slot, uint64_t key) { s->pending[slot] = key; if (!s->held.count(key)) finish_host_fill(s, slot); };
+        h.done = [s](size_t slot) { return s->pending[slot] == kNone; };
+        h.wait = [s](size_t slot) {
+            if (s->pending[slot] != kNone && s->held.count(s->pending[slot])) throw std::logic_error("waiting for a fill that the test still holds");
+            finish_host_fill(s, slot);
+        };
+        h.move = [s](size_t from, size_t to) { std::memcpy(s->pool + to * s->stride, s->pool + from * s->stride, s->record_bytes); };
+    }
+    return h;
+}
+// Slot storage for `slots` slots; keeps the bytes of the first `keep` slots.
+void provide_pool(zc_hip_store* s, uint64_t slots, uint64_t keep) {
+    uint8_t* fresh = nullptr;
+    if (s->ctx) {
+        void* p = nullptr;
+        if (zc_hip_alloc(s->ctx, slots * s->stride, &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
+        fresh = static_cast<uint8_t*>(p);
+        if (s->pool && keep) { ZC_STORE_HIP(hipMemcpyAsync(fresh, s->pool, keep * s->stride, hipMemcpyDeviceToDevice, s->side)); ZC_STORE_HIP(hipStreamSynchronize(s->side)); }
+        if (s->pool) zc_hip_free(s->ctx, s->pool);
+        while (s->filled.size() > slots) { (void)hipEventDestroy(s->filled.back()); s->filled.pop_back(); }
+        while (s->filled.size() < slots) {
+            hipEvent_t e; ZC_STORE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            ZC_STORE_HIP(hipEventRecord(e, s->side));   // a slot that was never filled counts as finished
+            s->filled.push_back(e);
+        }
+    } else {
+        fresh = new uint8_t[slots * s->stride]();
+        if (s->pool && keep) std::memcpy(fresh, s->pool, keep * s->stride);
+        delete[] s->pool;
+        s->pending.resize(slots, kNone);
+    }
+    s->pool = fresh;
+}
+}  // namespace
+
+extern "C" {
+
+zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots, zc_hip_store** out) {
+    if (!out || !layers || !experts || !record_bytes || !slots) return zc_fail(ZC_INVALID_ARGUMENT, "empty expert cache");
+    auto s = std::make_unique<zc_hip_store>();
+    s->ctx = ctx; s->layers = layers; s->experts = experts; s->record_bytes = record_bytes; s->stride = (record_bytes + 255) / 256 * 256;
+    s->layer_hits.assign(layers, 0); s->layer_misses.assign(layers, 0);
+    const zc_status status = guarded([&] {
+        const uint64_t home = uint64_t(layers) * experts * s->stride;
+        if (ctx) {
+            void* p = nullptr;
+            if (zc_hip_alloc_host(ctx, home, &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
+            s->backing = static_cast<uint8_t*>(p);
+            ZC_STORE_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));   // default priority
+        } else {
+            s->backing = new uint8_t[home]();
+        }
+        provide_pool(s.get(), slots, 0);
+        s->cache = std::make_unique<zc::SlotCache>(slots, record_bytes, hooks_of(s.get()));
+        return ZC_OK;
+    });
+    if (status != ZC_OK) { zc_hip_store_destroy(s.release()); return status; }
+    *out = s.release();
+    return ZC_OK;
+}
+zc_status zc_hip_store_destroy(zc_hip_store* s) {
+    if (!s) return ZC_OK;
+    if (s->ctx) {
+        if (s->side) { (void)hipStreamSynchronize(s->side); }
+        for (hipEvent_t e : s->filled) (void)hipEventDestroy(e);
+        if (s->side) (void)hipStreamDestroy(s->side);
+        if (s->pool) zc_hip_free(s->ctx, s->pool);
+        if (s->backing) zc_hip_free(s->ctx, s->backing);
+    } else {
+        delete[] s->pool; delete[] s->backing;
+    }
+    delete s;
+    return ZC_OK;
+}
+void* zc_hip_store_backing(zc_hip_store* s, uint32_t layer, uint32_t expert) {
+    if (!s || layer >= s->layers || expert >= s->experts) return nullptr;
+    return s->backing + key_of(s, layer, expert) * s->stride;
+}
+uint64_t zc_hip_store_stride(const zc_hip_store* s) { return s ? s->stride : 0; }
+uint64_t zc_hip_store_capacity(const zc_hip_store* s) { return s ? s->cache->capacity() : 0; }
+uint64_t zc_hip_store_occupancy(const zc_hip_store* s) { return s ? s->cache->occupancy() : 0; }
+
+zc_status zc_hip_store_acquire(zc_hip_store* s, uint32_t layer, uint32_t expert, zc_store_lease* out) {
+    if (!s || !out) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    if (layer >= s->layers || expert >= s->experts) return zc_fail(ZC_OUT_OF_RANGE, "invalid expert id");
+    return guarded([&] {
+        const auto lease = s->cache->acquire(key_of(s, layer, expert));
+        if (lease.acquisition == zc::SlotCache::NewMiss) ++s->layer_misses[layer]; else ++s->layer_hits[layer];
+        out->lease = lease.slot; out->record = s->pool + lease.slot * s->stride; out->acquisition = int32_t(lease.acquisition);
+        return ZC_OK;
+    });
+}
+zc_status zc_hip_store_wait(zc_hip_store* s, uint64_t lease) {
+    if (!s || lease >= s->cache->capacity() || !s->cache->pins(lease)) return zc_fail(ZC_LOGIC_ERROR, "empty expert lease");
+    return guarded([&] {
+        if (s->ctx) ZC_STORE_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(zc_hip_stream(s->ctx)), s->filled[lease], 0));
+        else if (s->pending[lease] != kNone) {
+            if (s->held.count(s->pending[lease])) throw std::logic_error("waiting for a fill that the test still holds");
+            finish_host_fill(s, lease);
+        }
+        return ZC_OK;
+    });
+}
+zc_status zc_hip_store_release(zc_hip_store* s, uint64_t lease) {
+    if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    return guarded([&] { s->cache->release(lease); return ZC_OK; });
+}
+zc_status zc_hip_store_prefetch(zc_hip_store* s, uint32_t layer, uint32_t expert, int* issued) {
+    if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    if (layer >= s->layers || expert >= s->experts) return zc_fail(ZC_OUT_OF_RANGE, "invalid expert id");
+    return guarded([&] { const bool did = s->cache->prefetch(key_of(s, layer, expert)); if (issued) *issued = did; return ZC_OK; });
+}
+int zc_hip_store_ready(zc_hip_store* s, uint32_t layer, uint32_t expert) {
+    if (!s || layer >= s->layers || expert >= s->experts) return 0;
+    try { return s->cache->ready(key_of(s, layer, expert)) ? 1 : 0; } catch (...) { return 0; }
+}
+zc_status zc_hip_store_clear(zc_hip_store* s) {
+    if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    return guarded([&] { s->cache->clear(); return ZC_OK; });
+}
+zc_status zc_hip_store_resize(zc_hip_store* s, uint64_t slots) {
+    if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    return guarded([&] {
+        if (!slots) throw std::invalid_argument("empty expert cache");
+        if (s->cache->leased()) throw std::logic_error("cannot resize leased expert slots");   // before any storage moves
+        const uint64_t before = s->cache->capacity();
+        if (slots > before) { provide_pool(s, slots, before); s->cache->resize(slots); }   // grow: storage first
+        else { s->cache->resize(slots); if (slots < before) provide_pool(s, slots, slots); }   // shrink: survivors are compacted to the front first
+        return ZC_OK;
+    });
+}
+zc_status zc_hip_store_stats(const zc_hip_store* s, zc_store_stats* out) {
+    if (!s || !out) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    const auto& c = s->cache->stats();
+    *out = zc_store_stats{c.hits, c.misses, c.evictions, c.bytes, c.ready_hits, c.loading_joins, c.prefetches, c.prefetch_claims, c.prefetch_unclaimed};
+    return ZC_OK;
+}
+zc_status zc_hip_store_layer_stats(const zc_hip_store* s, uint32_t layer, uint64_t* hits, uint64_t* misses) {
+    if (!s || layer >= s->layers) return zc_fail(ZC_OUT_OF_RANGE, "invalid layer");
+    if (hits) *hits = s->layer_hits[layer];
+    if (misses) *misses = s->layer_misses[layer];
+    return ZC_OK;
+}
+zc_status zc_hip_store_hold(zc_hip_store* s, uint32_t layer, uint32_t expert, int hold) {
+    if (!s || s->ctx) return zc_fail(ZC_LOGIC_ERROR, "fills can only be held in a store without a context");
+    if (layer >= s->layers || expert >= s->experts) return zc_fail(ZC_OUT_OF_RANGE, "invalid expert id");
+    const uint64_t key = key_of(s, layer, expert);
+    if (hold) s->held.insert(key);
+    else {
+        s->held.erase(key);
+        for (size_t slot = 0; slot < s->pending.size(); ++slot) if (s->pending[slot] == key) finish_host_fill(s, slot);
+    }
+    return ZC_OK;
+}
+
+}  // extern "C"

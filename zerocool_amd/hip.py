@@ -52,12 +52,109 @@ def load_library():
     lib.zc_hip_last_error.restype = C.c_char_p
     lib.zc_hip_version.restype = C.c_char_p
     for name in ("zc_hip_allocated", "zc_hip_peak", "zc_hip_moe_workspace_bytes", "zc_hip_projection_bytes",
-                 "zc_hip_record_bytes"):
+                 "zc_hip_record_bytes", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy"):
         getattr(lib, name).restype = C.c_uint64
     lib.zc_hip_stream.restype = C.c_void_p
+    lib.zc_hip_store_backing.restype = C.c_void_p
+    for name in ("zc_hip_store_backing", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy"):
+        getattr(lib, name).argtypes = [C.c_void_p] + ([C.c_uint32, C.c_uint32] if name.endswith("backing") else [])
     lib.zc_hip_projection_bytes.argtypes = [C.c_uint32] * 4
     _lib = lib
     return lib
+
+
+class StoreStats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("hits", "misses", "evictions", "bytes", "ready_hits", "loading_joins",
+                                          "prefetches", "prefetch_claims", "prefetch_unclaimed")]
+
+
+class StoreLease(C.Structure):
+    _fields_ = [("lease", C.c_uint64), ("record", C.c_void_p), ("acquisition", C.c_int32)]
+
+
+class Store:
+    """Expert store (zc_hip_store_*): records live in pinned host memory, `slots` HBM slots cache them.  ctx=None gives a
+    store with host-memory slots whose fills can be held back, for tests of the policy without a GPU."""
+
+    ACQUISITIONS = ("new_miss", "ready_hit", "loading_join")
+
+    def __init__(self, ctx, layers, experts, record_bytes, slots):
+        self.lib = load_library()
+        self.ctx, self.layers, self.experts, self.record_bytes = ctx, layers, experts, record_bytes
+        self.handle = C.c_void_p()
+        self._check(self.lib.zc_hip_store_create(ctx.handle if ctx else None, C.c_uint32(layers), C.c_uint32(experts),
+                                                 C.c_uint64(record_bytes), C.c_uint64(slots), C.byref(self.handle)))
+
+    def _check(self, status):
+        if status:
+            raise ZcError(status, self.lib.zc_hip_last_error().decode())
+
+    def close(self):
+        if self.handle:
+            self.lib.zc_hip_store_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def backing(self, layer, expert):
+        """The record's home in (pinned) host memory as a writable numpy byte array."""
+        p = self.lib.zc_hip_store_backing(self.handle, layer, expert)
+        if not p:
+            raise IndexError("invalid expert id")
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(self.record_bytes,))
+
+    def acquire(self, layer, expert):
+        lease = StoreLease()
+        self._check(self.lib.zc_hip_store_acquire(self.handle, C.c_uint32(layer), C.c_uint32(expert), C.byref(lease)))
+        return lease
+
+    def wait(self, lease):
+        self._check(self.lib.zc_hip_store_wait(self.handle, C.c_uint64(lease.lease)))
+        return DevBuf(self.ctx, lease.record, self.record_bytes) if self.ctx else lease.record
+
+    def release(self, lease):
+        self._check(self.lib.zc_hip_store_release(self.handle, C.c_uint64(lease.lease)))
+
+    def prefetch(self, layer, expert):
+        issued = C.c_int(0)
+        self._check(self.lib.zc_hip_store_prefetch(self.handle, C.c_uint32(layer), C.c_uint32(expert), C.byref(issued)))
+        return bool(issued.value)
+
+    def ready(self, layer, expert):
+        return bool(self.lib.zc_hip_store_ready(self.handle, C.c_uint32(layer), C.c_uint32(expert)))
+
+    def hold(self, layer, expert, hold=True):
+        self._check(self.lib.zc_hip_store_hold(self.handle, C.c_uint32(layer), C.c_uint32(expert), C.c_int(int(hold))))
+
+    def clear(self):
+        self._check(self.lib.zc_hip_store_clear(self.handle))
+
+    def resize(self, slots):
+        self._check(self.lib.zc_hip_store_resize(self.handle, C.c_uint64(slots)))
+
+    @property
+    def capacity(self):
+        return self.lib.zc_hip_store_capacity(self.handle)
+
+    @property
+    def occupancy(self):
+        return self.lib.zc_hip_store_occupancy(self.handle)
+
+    @property
+    def stride(self):
+        return self.lib.zc_hip_store_stride(self.handle)
+
+    def stats(self):
+        st = StoreStats()
+        self._check(self.lib.zc_hip_store_stats(self.handle, C.byref(st)))
+        return st
+
+    def layer_stats(self, layer):
+        h, m = C.c_uint64(), C.c_uint64()
+        self._check(self.lib.zc_hip_store_layer_stats(self.handle, C.c_uint32(layer), C.byref(h), C.byref(m)))
+        return h.value, m.value
+
+    def slot_bytes(self, lease):
+        """Host-memory stores: the slot's current bytes."""
+        return np.ctypeslib.as_array(C.cast(lease.record, C.POINTER(C.c_uint8)), shape=(self.record_bytes,))
 
 
 class DevBuf:

@@ -78,3 +78,70 @@ def layer_bytes(cfg, unique_experts, tokens, ctx):
     H, E, k = cfg.hidden, cfg.experts, cfg.topk
     return (2 * H * E + 2 * H + unique_experts * ctx.record_bytes(cfg) + ctx.record_bytes(cfg, shared=True)
             + tokens * 4 * H + tokens * k * 8)
+
+
+class StoreBackedStack:
+    """A stack of layers whose routed records live in an expert store: the home of every record is pinned host
+    memory, `slots` HBM slots cache the records in use (the capped-HBM run of the 48-layer configuration).  The layer
+    step is the reference's orchestration (src/engine/model.cpp:431-557): router, route, ONE readback of the ids,
+    leases for the selected experts (fills on the store's side stream), per-expert gate/up + down into the expert's
+    slots, shared expert, weighted combine; leases are released once the step's GPU work has finished."""
+
+    def __init__(self, ctx, cfg, seeds, skew, slots):
+        from .hip import Store, DevBuf
+        self.ctx, self.cfg = ctx, cfg
+        self.store = Store(ctx, len(seeds), cfg.experts, ctx.record_bytes(cfg), slots)
+        assert self.store.stride == record_stride(ctx, cfg)
+        self.layers = []
+        for l, seed in enumerate(seeds):
+            home = self.store.lib.zc_hip_store_backing(self.store.handle, l, 0)
+            # the generator kernel writes the records straight into their pinned-host home (mapped into the GPU)
+            records = DevBuf(ctx, home, cfg.experts * self.store.stride)
+            self.layers.append(LayerWeights(ctx, cfg, seed, skew, records=records))
+        ctx.finish()
+
+    def close(self):
+        self.store.close()
+
+    def layer_forward(self, l, x, T):
+        ctx, cfg, w = self.ctx, self.cfg, self.layers[l]
+        H, E, k, I = cfg.hidden, cfg.experts, cfg.topk, cfg.inter
+        logits = ctx.router_logits(w.router, x, T, H, E, w.offsets)
+        ids, weights = ctx.route(logits, T, E, k)
+        host_ids = ids.numpy(np.int32)                      # the one readback (model.cpp:446)
+        if ((host_ids < 0) | (host_ids >= E)).any():
+            raise RuntimeError("invalid router output")     # model.cpp:459
+        order = np.argsort(host_ids, kind="stable")          # slots grouped by expert, ascending slot inside an expert
+        selected, starts = np.unique(host_ids[order], return_index=True)
+        expert_out = ctx.alloc(T * k * H * 4)
+        temporaries = [logits, ids, weights, expert_out]
+        bounds = list(starts) + [len(order)]
+        group = max(1, min(int(self.store.capacity), 32))   # leases out at once (pipeline.cpp:71-220 works in such groups)
+        for g0 in range(0, len(selected), group):
+            batch = range(g0, min(g0 + group, len(selected)))
+            leases = [self.store.acquire(l, int(selected[j])) for j in batch]   # fills start on the side stream
+            for j, lease in zip(batch, leases):
+                record = self.store.wait(lease)              # the compute stream waits for the slot's fill, the host does not
+                slots = order[bounds[j]:bounds[j + 1]].astype(np.int32)
+                rows = ctx.upload((slots // k).astype(np.int32))
+                act = ctx.gated_linear(ctx.expert_linear(cfg, record, 0), ctx.expert_linear(cfg, record, 1), x, T, len(slots), rows)
+                if len(slots) == 1:                          # direct rows (model.cpp:527-531)
+                    ctx.linear(ctx.expert_linear(cfg, record, 2), act, 1, out=expert_out.view(int(slots[0]) * H * 4, H * 4))
+                    temporaries += [rows, act]
+                else:                                        # encode_expert_rows (pipeline.cpp:7-31)
+                    y = ctx.linear(ctx.expert_linear(cfg, record, 2), act, len(slots))
+                    positions = ctx.upload(slots)
+                    ctx.scatter_experts(y, positions, len(slots), H, expert_out)
+                    temporaries += [rows, act, y, positions]
+            ctx.finish()                                     # GPU users of the slots are done: the leases may go
+            for lease in leases:
+                self.store.release(lease)
+        sact = ctx.gated_linear(ctx.expert_linear(cfg, w.shared_record, 0, shared=True), ctx.expert_linear(cfg, w.shared_record, 1, shared=True), x, T, T)
+        shared = ctx.linear(ctx.expert_linear(cfg, w.shared_record, 2, shared=True), sact, T)
+        from .hip import Linear
+        gate = ctx.linear(Linear(w.shared_gate.ptr, None, None, H, 1, 64, 0, 0, 4), x, T)
+        out = ctx.moe_sum(expert_out, weights, shared, gate, T, H, k)
+        ctx.finish()
+        for b in temporaries + [sact, shared, gate]:
+            ctx.free(b)
+        return out, host_ids

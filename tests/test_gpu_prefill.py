@@ -1,0 +1,99 @@
+"""Prefill path (BASELINE config 3 at reduced and full size): sorted tokens + grouped GEMM on the bf16 matrix cores.
+Routing ids, softmax weights and the dispatch must equal the exact path bit for bit; expert outputs and the layer
+output are checked against the exact path (itself byte-equal to the CPU oracle) within max relative error 2e-3."""
+import numpy as np
+import pytest
+import oracle
+import zerocool_amd as z
+from zerocool_amd import workload
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+TOLERANCE = 2e-3   # max |got - want| / max |want|
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = z.Context(0)
+    yield c
+    c.close()
+
+
+def run_both(ctx, cfg, weights, x, T):
+    n = T * cfg.topk
+    outs = []
+    for prefill in (False, True):
+        out = ctx.alloc(T * cfg.hidden * 4)
+        size = ctx.moe_prefill_workspace_bytes(cfg, T) if prefill else ctx.moe_workspace_bytes(cfg, T)
+        assert size > 0
+        ws = ctx.alloc(size)
+        ids, w = ctx.alloc(n * 4), ctx.alloc(n * 4)
+        eo, sh = ctx.alloc(n * cfg.hidden * 4), ctx.alloc(T * cfg.hidden * 4)
+        trace = z.Trace(None, ids.ptr, w.ptr, eo.ptr, sh.ptr, None)
+        (ctx.moe_prefill if prefill else ctx.moe_forward)(cfg, weights.layer, x, T, out, ws, trace)
+        ctx.moe_check()
+        outs.append(dict(out=out.numpy(f32), ids=ids.numpy(np.int32), weights=w.numpy(f32), expert_out=eo.numpy(f32), shared=sh.numpy(f32)))
+        for b in (out, ws, ids, w, eo, sh):
+            ctx.free(b)
+    return outs
+
+
+def rel(got, want):
+    return float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+
+
+ONE_BF16_STEP = 2.0 ** -7   # the spacing of BF16 numbers relative to their magnitude, at most
+
+
+@pytest.mark.parametrize("shape,tokens", [((512, 32, 4, 128), 1), ((512, 32, 4, 128), 37), ((512, 32, 4, 128), 300),
+                                          ((1024, 64, 10, 256), 129), ((2048, 512, 10, 512), 96)])
+def test_prefill_matches_the_exact_path(ctx, shape, tokens):
+    cfg = workload.tiny_config(*shape)
+    weights = workload.LayerWeights(ctx, cfg, 61 + tokens, ("normal", 0.5))
+    x = workload.hidden_rows(ctx, tokens, cfg.hidden, 700 + tokens)
+    exact, fast = run_both(ctx, cfg, weights, x, tokens)
+    assert fast["ids"].tobytes() == exact["ids"].tobytes()
+    assert fast["weights"].tobytes() == exact["weights"].tobytes()
+    # The two paths differ only by the order of fp32 additions, so a BF16-rounded value can at most tip over to the
+    # neighbouring BF16 number where its fp32 sum sits on a rounding boundary.  Intermediates: no error larger than one
+    # such step of the largest value; layer output: within the stated tolerance, and nearly all values identical.
+    assert rel(fast["shared"], exact["shared"]) <= ONE_BF16_STEP
+    assert rel(fast["expert_out"], exact["expert_out"]) <= ONE_BF16_STEP
+    print(f"T={tokens} {shape}: layer output max rel err {rel(fast['out'], exact['out']):.3g}, "
+          f"identical {np.mean(fast['out'].view(np.uint32) == exact['out'].view(np.uint32)):.5f}, "
+          f"expert outputs identical {np.mean(fast['expert_out'].view(np.uint32) == exact['expert_out'].view(np.uint32)):.5f}")
+    assert rel(fast["out"], exact["out"]) <= TOLERANCE
+    same = np.mean(fast["out"].view(np.uint32) == exact["out"].view(np.uint32))
+    assert same > 0.98, same
+    for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, x):
+        ctx.free(b)
+
+
+def test_prefill_against_the_cpu_oracle(ctx):
+    cfg = workload.tiny_config(512, 32, 4, 128)
+    T = 70
+    weights = workload.LayerWeights(ctx, cfg, 91, ("zipf", 1.1))
+    x = workload.hidden_rows(ctx, T, cfg.hidden, 92)
+    h = weights.host()
+    ocfg = oracle.Config(*[getattr(cfg, n) for n, _ in z.Config._fields_])
+    want, tr = oracle.moe_layer(ocfg, h["router"], h["shared_gate"], h["shared_record"], h["records"], h["stride"],
+                                x.numpy(f32), T, router_offsets=h["offsets"], threads=8, trace=True)
+    _, fast = run_both(ctx, cfg, weights, x, T)
+    assert fast["ids"].tobytes() == tr["ids"].tobytes()
+    assert rel(fast["out"].reshape(T, cfg.hidden), want) <= TOLERANCE
+
+
+def test_prefill_rejects_what_it_cannot_run(ctx):
+    mixed = workload.tiny_config(512, 32, 4, 128, bits=(4, 8, 8, 8))
+    assert ctx.moe_prefill_workspace_bytes(mixed, 64) == 0
+    cfg = workload.tiny_config(512, 32, 4, 128)
+    weights = workload.LayerWeights(ctx, cfg, 93, None)
+    T = 40
+    x = ctx.upload(np.full(T * cfg.hidden, 1.0000001, f32))     # not BF16-valued
+    out, ws = ctx.alloc(T * cfg.hidden * 4), ctx.alloc(ctx.moe_prefill_workspace_bytes(cfg, T))
+    ctx.moe_prefill(cfg, weights.layer, x, T, out, ws)
+    with pytest.raises(z.ZcError) as err:
+        ctx.moe_check()
+    assert "BF16" in str(err.value)
+    with pytest.raises(z.ZcError):
+        ctx.moe_prefill(mixed, weights.layer, x, T, out, ws)

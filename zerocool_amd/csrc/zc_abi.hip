@@ -444,6 +444,116 @@ zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     }
     return ZC_OK;
 }
+// Prefill: the same layer with the expert products as a sorted-token grouped GEMM on the bf16 matrix cores.
+namespace {
+struct PrefillSpace {
+    Workspace base;
+    uint16_t *xb, *actb, *sactb; float *xsum, *asum, *ssum;
+    int32_t *tile_expert, *tile_first, *tile_rows, *tile_count, *stile_expert, *stile_first, *stile_rows, *stile_count;
+    uint32_t max_tiles, max_shared_tiles;
+    uint64_t bytes;
+};
+PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
+    PrefillSpace w{};
+    w.base = carve(c, T, base);
+    uint64_t at = w.base.bytes;
+    auto take = [&](uint64_t bytes) { void* p = base ? static_cast<uint8_t*>(base) + at : nullptr; at += align_up(bytes, 256); return p; };
+    const uint64_t n = uint64_t(T) * c->topk;
+    w.max_tiles = uint32_t(n / 32 + c->experts); w.max_shared_tiles = (T + 31) / 32;
+    w.xb = (uint16_t*)take(uint64_t(T) * c->hidden * 2); w.xsum = (float*)take(uint64_t(T) * (c->hidden / 64) * 4);
+    w.actb = (uint16_t*)take(n * c->inter * 2); w.asum = (float*)take(n * (c->inter / 64) * 4);
+    w.sactb = (uint16_t*)take(uint64_t(T) * c->inter * 2); w.ssum = (float*)take(uint64_t(T) * (c->inter / 64) * 4);
+    w.tile_expert = (int32_t*)take(w.max_tiles * 4ull); w.tile_first = (int32_t*)take(w.max_tiles * 4ull); w.tile_rows = (int32_t*)take(w.max_tiles * 4ull);
+    w.tile_count = (int32_t*)take(4);
+    w.stile_expert = (int32_t*)take(w.max_shared_tiles * 4ull); w.stile_first = (int32_t*)take(w.max_shared_tiles * 4ull);
+    w.stile_rows = (int32_t*)take(w.max_shared_tiles * 4ull); w.stile_count = (int32_t*)take(4);
+    w.bytes = at;
+    return w;
+}
+bool prefill_config(const zc_moe_config* c) {
+    return c->bits_gate_up == 4 && c->bits_down == 4 && c->shared_bits_gate_up == 4 && c->shared_bits_down == 4 && c->group == 64 &&
+           zc::prefill_shape(c->hidden, c->inter, c->experts);
+}
+}  // namespace
+uint64_t zc_hip_moe_prefill_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens) {
+    if (validate_config(cfg) != ZC_OK || !tokens || !prefill_config(cfg)) return 0;
+    return carve_prefill(cfg, tokens, nullptr).bytes;
+}
+zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
+                             float* out, void* workspace, const zc_moe_trace* trace) {
+    if (const zc_status s = validate_config(c)) return s;
+    ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 group 64 with hidden and intermediate sizes that are multiples of 128");
+    ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
+    ZC_REQUIRE(l->router && l->shared_gate && l->shared_record && l->expert_records, "missing MoE layer weights");
+    ZC_REQUIRE(l->record_stride >= zc_hip_record_bytes(c, 0) && l->record_stride % 16 == 0, "expert record stride is too small or not a multiple of 16");
+    ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(workspace) % 256 == 0 &&
+               reinterpret_cast<uintptr_t>(l->router) % 16 == 0 && reinterpret_cast<uintptr_t>(l->expert_records) % 16 == 0 &&
+               reinterpret_cast<uintptr_t>(l->shared_record) % 16 == 0, "MoE layer operands are misaligned");
+    ZC_REQUIRE(x != out, "invalid or overlapping linear output");
+    const PrefillSpace w = carve_prefill(c, T, workspace);
+    hipStream_t s = ctx->stream;
+    const uint32_t H = c->hidden, I = c->inter, E = c->experts, k = c->topk;
+    const uint64_t n = uint64_t(T) * k;
+    // exact kernels: router logits, top-k + softmax, dispatch (model.cpp:434-479), shared gate
+    zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
+    zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
+    zc::launch_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, w.base.selected, w.base.count, ctx->moe_status);
+    zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
+    // operands of the matrix cores: bf16 rows and their group sums; work lists
+    zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, ctx->moe_status);
+    zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
+    zc::launch_prefill_tiles(s, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
+    auto offsets_of = [&](const void* record, int shared, uint64_t* off, int first, int count) {
+        for (int q = 0; q < count; ++q) {
+            zc_linear lin; zc_hip_expert_linear(c, shared, record, first + q, &lin);
+            const auto base = reinterpret_cast<uintptr_t>(record);
+            off[3 * q] = reinterpret_cast<uintptr_t>(lin.weight) - base; off[3 * q + 1] = reinterpret_cast<uintptr_t>(lin.scales) - base;
+            off[3 * q + 2] = reinterpret_cast<uintptr_t>(lin.biases) - base;
+        }
+    };
+    {   // routed gate/up + SwiGLU on gathered rows (pipeline.cpp:18-24), then down scattered to the slots (pipeline.cpp:25-29)
+        zc::PrefillGemm g{};
+        g.a = w.xb; g.asum = w.xsum; g.a_rows = w.base.slots; g.a_div = k; g.out_rows = nullptr;
+        g.records = static_cast<const uint8_t*>(l->expert_records); g.stride = l->record_stride; offsets_of(l->expert_records, 0, g.off, 0, 2);
+        g.tile_expert = w.tile_expert; g.tile_first = w.tile_first; g.tile_rows = w.tile_rows; g.tile_count = w.tile_count;
+        g.K = H; g.N = I; g.out_b = w.actb;
+        zc::launch_prefill_gemm(s, g, true, w.max_tiles);
+        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum);
+        zc::PrefillGemm d{};
+        d.a = w.actb; d.asum = w.asum; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
+        d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
+        d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
+        d.K = I; d.N = H; d.out_f = w.base.expert_out;
+        zc::launch_prefill_gemm(s, d, false, w.max_tiles);
+    }
+    {   // shared expert (model.cpp:482-485): one group of all the tokens
+        zc::PrefillGemm g{};
+        g.a = w.xb; g.asum = w.xsum; g.a_rows = nullptr; g.a_div = 1;
+        g.records = static_cast<const uint8_t*>(l->shared_record); g.stride = 0; offsets_of(l->shared_record, 1, g.off, 0, 2);
+        g.tile_expert = w.stile_expert; g.tile_first = w.stile_first; g.tile_rows = w.stile_rows; g.tile_count = w.stile_count;
+        g.K = H; g.N = I; g.out_b = w.sactb;
+        zc::launch_prefill_gemm(s, g, true, w.max_shared_tiles);
+        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum);
+        zc::PrefillGemm d{};
+        d.a = w.sactb; d.asum = w.ssum; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
+        d.records = g.records; d.stride = 0; offsets_of(l->shared_record, 1, d.off, 2, 1);
+        d.tile_expert = w.stile_expert; d.tile_first = w.stile_first; d.tile_rows = w.stile_rows; d.tile_count = w.stile_count;
+        d.K = I; d.N = H; d.out_f = w.base.shared;
+        zc::launch_prefill_gemm(s, d, false, w.max_shared_tiles);
+    }
+    // weighted combine (model.cpp:553-556)
+    zc::launch_moe_sum(s, w.base.expert_out, w.base.weights, w.base.shared, w.base.gate, T, H, k, out);
+    ZC_LAUNCHED();
+    if (trace) {
+        if (trace->logits) ZC_HIP(hipMemcpyAsync(trace->logits, w.base.logits, uint64_t(T) * E * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->ids) ZC_HIP(hipMemcpyAsync(trace->ids, w.base.ids, n * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->weights) ZC_HIP(hipMemcpyAsync(trace->weights, w.base.weights, n * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->expert_out) ZC_HIP(hipMemcpyAsync(trace->expert_out, w.base.expert_out, n * H * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->shared) ZC_HIP(hipMemcpyAsync(trace->shared, w.base.shared, uint64_t(T) * H * 4, hipMemcpyDeviceToDevice, s));
+        if (trace->gate) ZC_HIP(hipMemcpyAsync(trace->gate, w.base.gate, uint64_t(T) * 4, hipMemcpyDeviceToDevice, s));
+    }
+    return ZC_OK;
+}
 zc_status zc_hip_moe_check(zc_hip_ctx* ctx) {
     ZC_REQUIRE(ctx, "null context");
     int32_t flag = 0;

@@ -245,8 +245,60 @@ __global__ __launch_bounds__(256) void router_kernel(const uint16_t* w, const fl
         if (split == 0 && e < E && t0 + t < T) out[uint64_t(t0 + t) * E + e] = offsets ? sum + offsets[e] : sum;
     }
 }
+// The same chains for long batches, register-tiled: a lane owns one K partition for 4 tokens x 4 experts, so every
+// sixteen-byte weight piece and every eight inputs feed sixteen multiply-accumulate chains.  A workgroup covers
+// 16 tokens x 16 experts; lane = (partition, token group, expert group).
+__global__ __launch_bounds__(256) void router_tiled_kernel(const uint16_t* w, const float* x, uint32_t T, uint32_t K,
+                                                           uint32_t E, const float* offsets, float* out) {
+    const uint32_t split = threadIdx.x % 16, pair = threadIdx.x / 16, tg = pair % 4, eg = pair / 4;
+    const uint32_t t0 = blockIdx.y * 16 + tg * 4, e0 = blockIdx.x * 16 + eg * 4, P = K / 16;
+    float c[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c[t][e] = 0;
+    const float* xr[4]; const uint16_t* wr[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) xr[t] = x + uint64_t(min(t0 + t, T - 1)) * K + split * P;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wr[e] = w + uint64_t(min(e0 + e, E - 1)) * K + split * P;
+    for (uint32_t i = 0; i < P; i += 8) {
+        float xv[4][8], wv[4][8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float4 a = *reinterpret_cast<const float4*>(xr[t] + i), b = *reinterpret_cast<const float4*>(xr[t] + i + 4);
+            xv[t][0] = a.x; xv[t][1] = a.y; xv[t][2] = a.z; xv[t][3] = a.w; xv[t][4] = b.x; xv[t][5] = b.y; xv[t][6] = b.z; xv[t][7] = b.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint4 v = *reinterpret_cast<const uint4*>(wr[e] + i);
+            const uint32_t ww[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int k = 0; k < 8; ++k) wv[e][k] = __uint_as_float((k & 1) ? (ww[k / 2] & 0xffff0000u) : (ww[k / 2] << 16));
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) c[t][e] = __builtin_fmaf(xv[t][k], wv[e][k], c[t][e]);
+    }
+    const uint32_t base = (threadIdx.x & 63u) & ~15u;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float sum = 0;
+            for (uint32_t sidx = 0; sidx < 16; ++sidx) sum += __shfl(c[t][e], base + sidx);
+            if (split == 0 && e0 + e < E && t0 + t < T) out[uint64_t(t0 + t) * E + e0 + e] = offsets ? sum + offsets[e0 + e] : sum;
+        }
+}
 void launch_router(hipStream_t s, const void* w, const float* x, uint32_t T, uint32_t K, uint32_t E,
                    const float* offsets, float* out) {
+    if (T >= 64 && K % 128 == 0) {
+        hipLaunchKernelGGL(router_tiled_kernel, dim3((E + 15) / 16, (T + 15) / 16), dim3(256), 0, s, (const uint16_t*)w, x, T, K, E, offsets, out);
+        return;
+    }
     const uint32_t gx = (E + 15) / 16;
     if (T >= 4) hipLaunchKernelGGL(router_kernel<4>, dim3(gx, (T + 3) / 4), dim3(256), 0, s, (const uint16_t*)w, x, T, K, E, offsets, out);
     else hipLaunchKernelGGL(router_kernel<1>, dim3(gx, T), dim3(256), 0, s, (const uint16_t*)w, x, T, K, E, offsets, out);
@@ -366,10 +418,65 @@ __global__ __launch_bounds__(1024) void dispatch_kernel(const int32_t* ids, uint
         }
     }
 }
+// The same sort for many slots (prefill), spread over the device: one wavefront per expert counts, one workgroup
+// scans, one wavefront per expert places.  offsets[1 + e] doubles as the count array between the first two steps.
+__global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* ids, uint32_t n, uint32_t E, int32_t* offsets, int32_t* status) {
+    const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blockIdx.x == 0) {
+        int bad = 0;
+        for (uint32_t p = threadIdx.x; p < n; p += blockDim.x) bad |= (ids[p] < 0 || ids[p] >= int32_t(E));
+        if (bad) atomicOr(status, 1);
+    }
+    if (e >= E) return;
+    int32_t c = 0;
+    for (uint32_t p0 = 0; p0 < n; p0 += 64) {
+        const uint32_t p = p0 + lane;
+        c += __popcll(__ballot(p < n && ids[p] == int32_t(e)));
+    }
+    if (lane == 0) offsets[1 + e] = c;
+}
+__global__ __launch_bounds__(64) void dispatch_scan_kernel(uint32_t E, int32_t* offsets, int32_t* selected, int32_t* count) {
+    const uint32_t lane = threadIdx.x;
+    int32_t running = 0, picked = 0;
+    if (lane == 0) offsets[0] = 0;
+    for (uint32_t base = 0; base < E; base += 64) {
+        const uint32_t e = base + lane;
+        const int32_t c = e < E ? offsets[1 + e] : 0;
+        int32_t incl = c;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { const int32_t up = __shfl_up(incl, o); if (int(lane) >= o) incl += up; }
+        if (e < E) offsets[e + 1] = running + incl;
+        const uint64_t mask = __ballot(c > 0);
+        if (c > 0) selected[picked + __popcll(mask & ((1ull << lane) - 1))] = int32_t(e);
+        picked += __popcll(mask);
+        running += __shfl(incl, 63);
+    }
+    if (lane == 0) *count = picked;
+}
+__global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* ids, uint32_t n, uint32_t topk, uint32_t E, const int32_t* offsets,
+                                                             int32_t* slots, int32_t* rows) {
+    const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (e >= E) return;
+    int32_t pos = offsets[e];
+    if (offsets[e + 1] == pos) return;
+    for (uint32_t p0 = 0; p0 < n; p0 += 64) {
+        const uint32_t p = p0 + lane;
+        const bool m = p < n && ids[p] == int32_t(e);
+        const uint64_t mask = __ballot(m);
+        if (m) { const int32_t at = pos + __popcll(mask & ((1ull << lane) - 1)); slots[at] = int32_t(p); if (rows) rows[at] = int32_t(p / topk); }
+        pos += __popcll(mask);
+    }
+}
 void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets,
                      int32_t* slots, int32_t* rows, int32_t* selected, int32_t* count, int32_t* status) {
-    hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(1024), size_t(E + 1) * 4, s, ids, tokens * topk, topk, E, offsets,
-                       slots, rows, selected, count, status);
+    const uint32_t n = tokens * topk;
+    if (n <= 1024) {   // decode: one launch
+        hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(1024), size_t(E + 1) * 4, s, ids, n, topk, E, offsets, slots, rows, selected, count, status);
+        return;
+    }
+    hipLaunchKernelGGL(dispatch_count_kernel, dim3((E + 3) / 4), dim3(256), 0, s, ids, n, E, offsets, status);
+    hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(64), 0, s, E, offsets, selected, count);
+    hipLaunchKernelGGL(dispatch_place_kernel, dim3((E + 3) / 4), dim3(256), 0, s, ids, n, topk, E, offsets, slots, rows);
 }
 
 // ---------------------------------------------------------------------------

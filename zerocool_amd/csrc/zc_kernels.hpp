@@ -74,4 +74,25 @@ hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt
 hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu);
 constexpr uint32_t kDecodeSyncBytes = (32 * 1024 + 16 * 64) * 4;
 
+// ---- prefill: sorted-token grouped GEMM on the bf16 matrix cores (zc_prefill.hip)
+struct PrefillGemm {
+    const uint16_t* a;        // bf16 rows [.][K]
+    const float* asum;        // per (row, group of 64): sum of the blocks' BF16-rounded sum-of-four chains
+    const int32_t* a_rows;    // row of `a` for sorted position pos: a_rows ? a_rows[pos] / a_div : pos
+    uint32_t a_div;
+    const int32_t* out_rows;  // output row for sorted position pos: out_rows ? out_rows[pos] : pos   (down projection)
+    const uint8_t* records; uint64_t stride;   // expert e's record at records + e * stride
+    uint64_t off[6];          // byte offsets in a record: codes, scales, biases of the (gate | down) projection, then of up
+    const int32_t *tile_expert, *tile_first, *tile_rows, *tile_count;
+    uint32_t K, N;            // reduction length, rows of ONE projection
+    uint16_t* out_b;          // gate/up: SwiGLU activations as bf16 [sorted position][N]
+    float* out_f;             // down: BF16-rounded fp32 [output row][N]
+};
+void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status);
+void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums);
+void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
+                          int32_t* tile_rows, int32_t* tile_count);
+void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles);
+bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts);
+
 }  // namespace zc

@@ -1,0 +1,242 @@
+// Prefill path of the MoE layer: tokens sorted by expert, then a grouped GEMM on the bf16 matrix cores with
+// fp32 accumulation (the reference batches the same work per expert in encode_expert_rows, src/engine/pipeline.cpp:7-31,
+// over q4_mm / q4_gate_up, kernels/metal/qwen.metal:289-376).
+//
+// Arithmetic.  The reference evaluates, per 16-element block, scale * sum(x q) + bias * sum'(x) with sum' the
+// BF16-rounded sum-of-four chain (qwen.metal:46-62).  Here the products x * q run on v_mfma_f32_16x16x32_bf16: x is
+// BF16-valued (exact as a bf16 operand), q in 0..15 is exact in bf16, products are exact and accumulate in fp32 over one
+// scale group of 64; per group the accumulator is folded as  total += scale * dot + bias * chain_sum  with the chain
+// sums precomputed per (row, group) exactly as the reference rounds them.  Only the order of the fp32 additions
+// differs from the reference, so results agree to a few fp32 ulps before the BF16 rounding of the outputs; this path is
+// tolerance-checked (max relative error 2e-3 of the layer output), not bit-exact.  Routing, dispatch and the combine use
+// the exact kernels.
+//
+// Tiling.  One workgroup (4 waves) owns 32 sorted token rows of ONE expert and 128 weight rows (gate/up: 64 gate rows
+// and the 64 up rows of the same indices, so SwiGLU is fused in registers), and walks K in steps of 64 = one scale
+// group: the 4-bit codes of the step are expanded to bf16 once per workgroup into LDS, the token rows are gathered into
+// LDS as bf16, both double-buffered.  Each wave multiplies a 16-row half of the tokens by 4 of the 8 column tiles.
+#include "zc_kernels.hpp"
+#include "zc_device.hpp"
+
+namespace zc {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kTileRows = 32, kTileCols = 128, kStepK = 64, kPitch = 72;   // LDS row pitch in bf16 elements (144 bytes)
+
+// fp32 rows holding BF16 values -> bf16 rows, plus per (row, group of 64) the sum of the four blocks' BF16-rounded
+// sum-of-four chains.  One thread per (row, group).  status bit 4: a value was not BF16-valued.
+__global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status) {
+    const uint32_t groups = K / 64, i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * groups) return;
+    const uint32_t r = i / groups, g = i % groups;
+    const float4* src = reinterpret_cast<const float4*>(x + uint64_t(r) * K + g * 64);
+    uint32_t low = 0;
+    float total = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        float sum = 0;
+        uint32_t packed[8];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 v = src[b * 4 + q];
+            sum += bf(bf(bf(v.x + v.y) + v.z) + v.w);
+            const uint32_t u0 = __float_as_uint(v.x), u1 = __float_as_uint(v.y), u2 = __float_as_uint(v.z), u3 = __float_as_uint(v.w);
+            low |= (u0 | u1 | u2 | u3) & 0xffffu;
+            packed[2 * q] = (u0 >> 16) | (u1 & 0xffff0000u); packed[2 * q + 1] = (u2 >> 16) | (u3 & 0xffff0000u);
+        }
+        total += sum;
+        uint4* dst = reinterpret_cast<uint4*>(xb + uint64_t(r) * K + g * 64 + b * 16);
+        dst[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+        dst[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
+    }
+    sums[i] = total;
+    if (low) atomicOr(status, 4);
+}
+// The same sums for rows that are already bf16 (the SwiGLU activations).
+__global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums) {
+    const uint32_t groups = K / 64, i = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t rows = rows_ptr ? min(uint32_t(*rows_ptr), rows_max) : rows_max;
+    if (i >= rows * groups) return;
+    const uint32_t r = i / groups, g = i % groups;
+    const uint4* src = reinterpret_cast<const uint4*>(xb + uint64_t(r) * K + g * 64);
+    float total = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const uint4 lo = src[2 * b], hi = src[2 * b + 1];
+        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        float sum = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float a = __uint_as_float(w[2 * q] << 16), c = __uint_as_float(w[2 * q] & 0xffff0000u);
+            const float d = __uint_as_float(w[2 * q + 1] << 16), e = __uint_as_float(w[2 * q + 1] & 0xffff0000u);
+            sum += bf(bf(bf(a + c) + d) + e);
+        }
+        total += sum;
+    }
+    sums[i] = total;
+}
+
+// Work list: tile t = (expert, first sorted position, rows).  offsets[e] .. offsets[e+1] are the expert's sorted
+// positions (the dispatch kernel's output); a null offsets pointer means ONE group of `rows` rows (the shared expert).
+__global__ __launch_bounds__(1024) void prefill_tiles_kernel(const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert,
+                                                            int32_t* tile_first, int32_t* tile_rows, int32_t* tile_count) {
+    __shared__ int32_t scan[1024];
+    const uint32_t e = threadIdx.x;
+    const int32_t first = offsets ? (e < experts ? offsets[e] : 0) : 0, count = offsets ? (e < experts ? offsets[e + 1] - offsets[e] : 0) : (e == 0 ? int32_t(rows) : 0);
+    const int32_t tiles = (count + int32_t(kTileRows) - 1) / int32_t(kTileRows);
+    scan[e] = tiles;
+    __syncthreads();
+    for (uint32_t step = 1; step < 1024; step <<= 1) {
+        const int32_t add = e >= step ? scan[e - step] : 0;
+        __syncthreads();
+        scan[e] += add;
+        __syncthreads();
+    }
+    const int32_t begin = scan[e] - tiles;
+    for (int32_t t = 0; t < tiles; ++t) {
+        tile_expert[begin + t] = int32_t(e); tile_first[begin + t] = first + t * int32_t(kTileRows);
+        tile_rows[begin + t] = min(int32_t(kTileRows), count - t * int32_t(kTileRows));
+    }
+    if (e == 1023) *tile_count = scan[1023];
+}
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
+    __shared__ __align__(16) uint16_t a_s[2][kTileRows * kPitch];
+    __shared__ __align__(16) uint16_t b_s[2][kTileCols * kPitch];
+    __shared__ float scale_s[2][kTileCols], bias_s[2][kTileCols], sum_s[2][kTileRows];
+    const uint32_t tile = blockIdx.y;
+    if (tile >= uint32_t(*p.tile_count)) return;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, j = lane & 15u, g4 = lane >> 4;
+    const uint32_t expert = uint32_t(p.tile_expert[tile]), first = uint32_t(p.tile_first[tile]), rows = uint32_t(p.tile_rows[tile]);
+    const uint32_t K = p.K, N = p.N, groups = K / 64;
+    const uint32_t n0 = blockIdx.x * (GATED ? 64u : 128u);
+    const uint8_t* record = p.records + uint64_t(expert) * p.stride;
+
+    // what this thread fetches every step
+    const uint32_t a_r = tid >> 3, a_c = tid & 7u;                       // token row of the tile, 16-byte chunk of the step
+    const uint32_t a_pos = first + min(a_r, rows - 1);                   // rows past the end repeat the last one (never stored)
+    const uint32_t a_row = p.a_rows ? uint32_t(p.a_rows[a_pos]) / p.a_div : a_pos;
+    const uint16_t* a_src = p.a + uint64_t(a_row) * K + a_c * 8;
+    const uint32_t b_r = tid >> 1, b_h = tid & 1u;                       // weight row of the tile, half of the step (32 codes)
+    const uint32_t b_proj = GATED ? b_r >> 6 : 0u, b_n = n0 + (GATED ? (b_r & 63u) : b_r);
+    const uint8_t* b_src = record + p.off[b_proj * 3] + uint64_t(b_n) * (K / 2) + b_h * 16;
+    const uint32_t m_r = tid & 127u;                                     // metadata row (threads 0..127)
+    const uint32_t m_proj = GATED ? m_r >> 6 : 0u, m_n = n0 + (GATED ? (m_r & 63u) : m_r);
+    const uint16_t* s_src = reinterpret_cast<const uint16_t*>(record + p.off[m_proj * 3 + 1]) + uint64_t(m_n) * groups;
+    const uint16_t* o_src = reinterpret_cast<const uint16_t*>(record + p.off[m_proj * 3 + 2]) + uint64_t(m_n) * groups;
+    const uint32_t x_pos = first + min(tid & 31u, rows - 1);
+    const uint32_t x_row = p.a_rows ? uint32_t(p.a_rows[x_pos]) / p.a_div : x_pos;
+    const float* x_src = p.asum + uint64_t(x_row) * groups;
+
+    uint4 a_next, b_next; uint16_t s_next = 0, o_next = 0; float x_next = 0;
+    auto fetch = [&](uint32_t g) {
+        a_next = *reinterpret_cast<const uint4*>(a_src + g * 64);
+        b_next = ldg_u4(b_src + g * 32);
+        if (tid < 128) { s_next = ldg_u16(s_src, g); o_next = ldg_u16(o_src, g); }
+        else if (tid < 160) x_next = x_src[g];
+    };
+    auto stash = [&](uint32_t buf) {
+        *reinterpret_cast<uint4*>(&a_s[buf][a_r * kPitch + a_c * 8]) = a_next;
+        // 32 codes -> 32 bf16: nibble i of a word is element 8w+i
+        const uint32_t words[4] = {b_next.x, b_next.y, b_next.z, b_next.w};
+        uint32_t out[16];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t even = words[w] & 0x0f0f0f0fu, odd = (words[w] >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x2 pair = {float((even >> (8 * q)) & 0xffu), float((odd >> (8 * q)) & 0xffu)};
+                out[4 * w + q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+            }
+        }
+        uint4* dst = reinterpret_cast<uint4*>(&b_s[buf][b_r * kPitch + b_h * 32]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dst[q] = make_uint4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
+        if (tid < 128) { scale_s[buf][m_r] = b16(s_next); bias_s[buf][m_r] = b16(o_next); }
+        else if (tid < 160) sum_s[buf][tid & 31u] = x_next;
+    };
+
+    const uint32_t wm = wave & 1u, wn = wave >> 1;
+    // the wave's four column tiles (rows of b_s): gate/up: two gate tiles and the up tiles of the same rows
+    uint32_t col_row[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) col_row[q] = (GATED ? ((q >> 1) * 64u + (2 * wn + (q & 1)) * 16u) : (4 * wn + q) * 16u) + j;
+    f32x4 total[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) total[q] = f32x4{0, 0, 0, 0};
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (uint32_t g = 0; g < groups; ++g) {
+        const uint32_t buf = g & 1u;
+        if (g + 1 < groups) fetch(g + 1);
+        f32x4 dot[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dot[q] = f32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&a_s[buf][(16 * wm + j) * kPitch + kk * 32 + g4 * 8]));
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&b_s[buf][col_row[q] * kPitch + kk * 32 + g4 * 8]));
+                dot[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, dot[q], 0, 0, 0);
+            }
+        }
+        float sums[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sums[r] = sum_s[buf][16 * wm + 4 * g4 + r];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float scale = scale_s[buf][col_row[q]], bias = bias_s[buf][col_row[q]];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) total[q][r] = __builtin_fmaf(scale, dot[q][r], __builtin_fmaf(bias, sums[r], total[q][r]));
+        }
+        if (g + 1 < groups) stash(buf ^ 1u);
+        __syncthreads();
+    }
+    // epilogue: row m of the tile is sorted position first + m
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t m = 16 * wm + 4 * g4 + r;
+        if (m >= rows) continue;
+        const uint32_t pos = first + m;
+        if constexpr (GATED) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const uint32_t n = n0 + (2 * wn + q) * 16 + j;
+                p.out_b[uint64_t(pos) * N + n] = uint16_t(__float_as_uint(swiglu_bf(total[q][r], total[2 + q][r])) >> 16);
+            }
+        } else {
+            const uint32_t out_row = p.out_rows ? uint32_t(p.out_rows[pos]) : pos;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) p.out_f[uint64_t(out_row) * N + n0 + (4 * wn + q) * 16 + j] = bf(total[q][r]);
+        }
+    }
+}
+
+void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status) {
+    const uint32_t items = rows * (K / 64);
+    hipLaunchKernelGGL(prefill_rows_kernel, dim3((items + 255) / 256), dim3(256), 0, s, x, rows, K, xb, sums, status);
+}
+void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums) {
+    const uint32_t items = rows_max * (K / 64);
+    hipLaunchKernelGGL(prefill_sums_kernel, dim3((items + 255) / 256), dim3(256), 0, s, xb, rows_ptr, rows_max, K, sums);
+}
+void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
+                          int32_t* tile_rows, int32_t* tile_count) {
+    hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(1024), 0, s, offsets, experts, rows, tile_expert, tile_first, tile_rows, tile_count);
+}
+void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles) {
+    const dim3 grid(gated ? p.N / 64 : p.N / 128, max_tiles);
+    if (gated) hipLaunchKernelGGL(prefill_gemm_kernel<true>, grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(prefill_gemm_kernel<false>, grid, dim3(256), 0, s, p);
+}
+bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts) { return hidden % 128 == 0 && inter % 128 == 0 && experts <= 1024; }
+
+}  // namespace zc

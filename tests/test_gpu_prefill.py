@@ -54,9 +54,10 @@ def test_prefill_matches_the_exact_path(ctx, shape, tokens):
     exact, fast = run_both(ctx, cfg, weights, x, tokens)
     assert fast["ids"].tobytes() == exact["ids"].tobytes()
     assert fast["weights"].tobytes() == exact["weights"].tobytes()
-    # The two paths differ only by the order of fp32 additions, so a BF16-rounded value can at most tip over to the
-    # neighbouring BF16 number where its fp32 sum sits on a rounding boundary.  Intermediates: no error larger than one
-    # such step of the largest value; layer output: within the stated tolerance, and nearly all values identical.
+    # The two paths differ only by the order of fp32 additions, so a BF16-rounded value could at most tip over to the
+    # neighbouring BF16 number where its fp32 sum sits on a rounding boundary; the prefill path recomputes exactly the
+    # sums that land near such a boundary.  Intermediates: no error larger than one such step of the largest value;
+    # layer output: within the stated tolerance, and all but a sliver of the values identical.
     assert rel(fast["shared"], exact["shared"]) <= ONE_BF16_STEP
     assert rel(fast["expert_out"], exact["expert_out"]) <= ONE_BF16_STEP
     print(f"T={tokens} {shape}: layer output max rel err {rel(fast['out'], exact['out']):.3g}, "
@@ -64,7 +65,7 @@ def test_prefill_matches_the_exact_path(ctx, shape, tokens):
           f"expert outputs identical {np.mean(fast['expert_out'].view(np.uint32) == exact['expert_out'].view(np.uint32)):.5f}")
     assert rel(fast["out"], exact["out"]) <= TOLERANCE
     same = np.mean(fast["out"].view(np.uint32) == exact["out"].view(np.uint32))
-    assert same > 0.98, same
+    assert same > 0.9999, same
     for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, x):
         ctx.free(b)
 

@@ -451,6 +451,7 @@ struct PrefillSpace {
     uint16_t *xb, *actb, *sactb; float *xsum, *asum, *ssum;
     int32_t *tile_expert, *tile_first, *tile_rows, *tile_count, *stile_expert, *stile_first, *stile_rows, *stile_count;
     uint32_t max_tiles, max_shared_tiles;
+    uint32_t* near_bits;      // one bit per product element: recompute exactly
     uint64_t bytes;
 };
 PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
@@ -467,6 +468,7 @@ PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
     w.tile_count = (int32_t*)take(4);
     w.stile_expert = (int32_t*)take(w.max_shared_tiles * 4ull); w.stile_first = (int32_t*)take(w.max_shared_tiles * 4ull);
     w.stile_rows = (int32_t*)take(w.max_shared_tiles * 4ull); w.stile_count = (int32_t*)take(4);
+    w.near_bits = (uint32_t*)take(n * std::max(c->hidden, c->inter) / 8);
     w.bytes = at;
     return w;
 }
@@ -484,6 +486,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     if (const zc_status s = validate_config(c)) return s;
     ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 group 64 with hidden and intermediate sizes that are multiples of 128");
     ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
+    ZC_REQUIRE(uint64_t(T) * c->topk * std::max(c->hidden, c->inter) < (1ull << 32), "too many product elements for one prefill call");
     ZC_REQUIRE(l->router && l->shared_gate && l->shared_record && l->expert_records, "missing MoE layer weights");
     ZC_REQUIRE(l->record_stride >= zc_hip_record_bytes(c, 0) && l->record_stride % 16 == 0, "expert record stride is too small or not a multiple of 16");
     ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(workspace) % 256 == 0 &&
@@ -500,6 +503,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     zc::launch_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, w.base.selected, w.base.count, ctx->moe_status);
     zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
     // operands of the matrix cores: bf16 rows and their group sums; work lists
+    const float margin = zc::kPrefillMargin;
     zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, ctx->moe_status);
     zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
     zc::launch_prefill_tiles(s, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
@@ -517,14 +521,18 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.records = static_cast<const uint8_t*>(l->expert_records); g.stride = l->record_stride; offsets_of(l->expert_records, 0, g.off, 0, 2);
         g.tile_expert = w.tile_expert; g.tile_first = w.tile_first; g.tile_rows = w.tile_rows; g.tile_count = w.tile_count;
         g.K = H; g.N = I; g.out_b = w.actb;
+        g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(n) * I / 32); g.near_margin = margin; g.ids = w.base.ids; g.slots = w.base.slots;
         zc::launch_prefill_gemm(s, g, true, w.max_tiles);
+        zc::launch_prefill_patch(s, g, true);
         zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum);
         zc::PrefillGemm d{};
         d.a = w.actb; d.asum = w.asum; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
         d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
         d.K = I; d.N = H; d.out_f = w.base.expert_out;
+        d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(n) * H / 32); d.near_margin = margin; d.ids = w.base.ids; d.slots = w.base.slots;
         zc::launch_prefill_gemm(s, d, false, w.max_tiles);
+        zc::launch_prefill_patch(s, d, false);
     }
     {   // shared expert (model.cpp:482-485): one group of all the tokens
         zc::PrefillGemm g{};
@@ -532,14 +540,18 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.records = static_cast<const uint8_t*>(l->shared_record); g.stride = 0; offsets_of(l->shared_record, 1, g.off, 0, 2);
         g.tile_expert = w.stile_expert; g.tile_first = w.stile_first; g.tile_rows = w.stile_rows; g.tile_count = w.stile_count;
         g.K = H; g.N = I; g.out_b = w.sactb;
+        g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(T) * I / 32); g.near_margin = margin; g.ids = nullptr; g.slots = nullptr;
         zc::launch_prefill_gemm(s, g, true, w.max_shared_tiles);
+        zc::launch_prefill_patch(s, g, true);
         zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum);
         zc::PrefillGemm d{};
         d.a = w.sactb; d.asum = w.ssum; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
         d.records = g.records; d.stride = 0; offsets_of(l->shared_record, 1, d.off, 2, 1);
         d.tile_expert = w.stile_expert; d.tile_first = w.stile_first; d.tile_rows = w.stile_rows; d.tile_count = w.stile_count;
         d.K = I; d.N = H; d.out_f = w.base.shared;
+        d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(T) * H / 32); d.near_margin = margin; d.ids = nullptr; d.slots = nullptr;
         zc::launch_prefill_gemm(s, d, false, w.max_shared_tiles);
+        zc::launch_prefill_patch(s, d, false);
     }
     // weighted combine (model.cpp:553-556)
     zc::launch_moe_sum(s, w.base.expert_out, w.base.weights, w.base.shared, w.base.gate, T, H, k, out);

@@ -87,12 +87,20 @@ struct PrefillGemm {
     uint32_t K, N;            // reduction length, rows of ONE projection
     uint16_t* out_b;          // gate/up: SwiGLU activations as bf16 [sorted position][N]
     float* out_f;             // down: BF16-rounded fp32 [output row][N]
+    // Sums that land within near_margin * (sum of term magnitudes) of a BF16 rounding boundary are marked in a bit map
+    // (bit sorted position * N + row; near_words 32-bit words, all written by the product kernel)
+    // and recomputed afterwards with the reference's exact lane arithmetic (launch_prefill_patch).
+    uint32_t* near_bits; uint32_t near_words; float near_margin;
+    const int32_t* ids;       // expert of sorted position pos: ids ? ids[slots[pos]] : 0 (used by the recomputation)
+    const int32_t* slots;
 };
+constexpr float kPrefillMargin = 0x1p-22f;  // of the summed term magnitudes: four fp32 steps at that scale
 void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status);
 void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums);
 void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
                           int32_t* tile_rows, int32_t* tile_count);
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles);
+void launch_prefill_patch(hipStream_t s, const PrefillGemm& p, bool gated);
 bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts);
 
 }  // namespace zc

@@ -27,6 +27,44 @@ MEASURED_TRAFFIC = 2_989_960_000
 sys.path.insert(0, ROOT)
 
 
+def single_layer(ctx, name, tokens, prefill, reps, warmup=3):
+    """One MoE layer of a single-layer configuration (hidden 2048, 512 experts, top-10, intermediate 512), timed with
+    weights and inputs resident.  FLOP count: 2 * tokens * hidden * intermediate * 3 projections * (top-k + shared)
+    + the router product."""
+    from zerocool_amd import workload
+    c = workload.config(name)
+    lw = workload.LayerWeights(ctx, c, workload.BASE_SEED + 77, ("zipf", 1.1))
+    x = workload.hidden_rows(ctx, tokens, c.hidden, workload.BASE_SEED + 78 + tokens)
+    out = ctx.alloc(tokens * c.hidden * 4)
+    ws = ctx.alloc(ctx.moe_prefill_workspace_bytes(c, tokens) if prefill else ctx.moe_workspace_bytes(c, tokens))
+    step = ctx.moe_prefill if prefill else ctx.moe_forward
+    for _ in range(warmup):
+        step(c, lw.layer, x, tokens, out, ws)
+    ctx.finish(); ctx.moe_check()
+    ctx.timer_start()
+    for _ in range(reps):
+        step(c, lw.layer, x, tokens, out, ws)
+    ms_layer = ctx.timer_stop() / reps
+    for b in (x, out, ws, lw.router, lw.shared_gate, lw.shared_record, lw.records):
+        ctx.free(b)
+    flops = 2.0 * tokens * c.hidden * c.inter * 3 * (c.topk + 1) + 2.0 * tokens * c.hidden * c.experts
+    return {"tokens": tokens, "us_per_layer": ms_layer * 1e3, "tokens_per_s": tokens / (ms_layer * 1e-3),
+            "TFLOPs": flops / (ms_layer * 1e-3) / 1e12, "path": "bf16 matrix-core prefill" if prefill else "exact operator path"}
+
+
+def prefill_workload(ctx, args):
+    r = single_layer(ctx, "S", 2048, True, args.steps, args.warmup)
+    print(json.dumps({
+        "metric": "moe_prefill_tokens_per_s", "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": r["us_per_layer"] * 1e-3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u4 codes as bf16 x bf16 inputs, fp32 accumulation", "data": "synthetic (seeded generator)",
+        "config": {"workload": "BASELINE configs[3]: one MoE layer, 2048-token prefill batch, hidden 2048, 512 experts, top-10, "
+                               "intermediate 512, affine Q4 group 64", "tokens": 2048},
+        "roofline": {"bound": "mfma", "achieved": r["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s", "frac": r["TFLOPs"] / 2500.0,
+                     "traffic": None, "kernel": "zc::prefill_gemm_kernel (whole-layer rate: router, routing, dispatch, "
+                                                "both grouped products, exact recomputation and combine included)"}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -36,6 +74,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extra", action="store_true", help="also time decode batch 8 and the single-layer configurations")
+    ap.add_argument("--workload", choices=("stack", "prefill"), default="stack",
+                    help="stack: the 48-layer decode stack (the headline); prefill: one 2048-token batch through one layer of "
+                         "hidden 2048 / 512 experts / top-10 / intermediate 512 on the bf16 matrix cores")
     ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -48,6 +89,8 @@ def main():
     from zerocool_amd import workload
 
     ctx = z.Context(0)
+    if args.workload == "prefill":
+        return prefill_workload(ctx, args)
     cfg = workload.config("F")
     L, T = args.layers, args.batch
     layers = [workload.LayerWeights(ctx, cfg, workload.BASE_SEED + 4 * 1000 + l, ("zipf", 1.1)) for l in range(L)]
@@ -170,6 +213,11 @@ def main():
                                "host_to_hbm_bytes_per_token_layer": (st.bytes - bytes0) / n_steps / capped_layers,
                                "evictions": int(st.evictions), "note": "Python-driven reference orchestration over zc_hip_store_*"}
         capped.close()
+        # Single-layer configurations: decode batches through the exact operator path, and batches through the
+        # sorted-token grouped product on the bf16 matrix cores.
+        extra["single_layer_q4"] = [single_layer(ctx, "S", t, False, 50) for t in (1, 8, 32, 64)]
+        extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8)]
+        extra["prefill_q4"] = [single_layer(ctx, "S", t, True, 20) for t in (32, 64, 256, 2048)]
         result["extra"] = extra
 
     print(json.dumps(result))

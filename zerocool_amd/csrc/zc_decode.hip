@@ -29,7 +29,9 @@ __device__ __forceinline__ int32_t uniform(int32_t v) { return __builtin_amdgcn_
 __device__ __forceinline__ void st_f32(float* p, float v) { ZC_ST(reinterpret_cast<uint32_t*>(p), __float_as_uint(v)); }
 __device__ __forceinline__ void st_i32(int32_t* p, int32_t v) { ZC_ST(reinterpret_cast<uint32_t*>(p), uint32_t(v)); }
 
-constexpr uint32_t kDecodeThreads = 256, kDecodeWaves = 4;
+// Workgroup size: single-token decode runs two waves per SIMD (the tile engine then fits 256 registers), several
+// tokens keep one wave per SIMD and the whole register file.
+constexpr uint32_t decode_threads(int nt) { return nt == 1 ? 512u : 256u; }
 constexpr uint32_t kFlagStride = 32, kReleaseBase = 32 * 1024, kReleaseStride = 64, kAbortWord = kReleaseBase + 8 * kReleaseStride;
 
 struct Barrier {
@@ -46,14 +48,17 @@ struct Barrier {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
-        if (blockIdx.x == 0) {
-            for (uint32_t w = threadIdx.x; w < gridDim.x; w += blockDim.x)
+        uint32_t me = blockIdx.x, thread = threadIdx.x;
+        asm volatile("" : "+s"(me));       // flag addresses are formed here, not kept in registers across the phases
+        asm volatile("" : "+v"(thread));
+        if (me == 0) {
+            for (uint32_t w = thread; w < gridDim.x; w += blockDim.x)
                 if (w) spin(mem + kFlagStride * w);
             __syncthreads();
-            if (threadIdx.x < 8) ZC_ST(mem + kReleaseBase + kReleaseStride * threadIdx.x, epoch);
-        } else if (threadIdx.x == 0) {
-            ZC_ST(mem + kFlagStride * blockIdx.x, epoch);
-            spin(mem + kReleaseBase + kReleaseStride * (blockIdx.x & 7u));
+            if (thread < 8) ZC_ST(mem + kReleaseBase + kReleaseStride * thread, epoch);
+        } else if (thread == 0) {
+            ZC_ST(mem + kFlagStride * me, epoch);
+            spin(mem + kReleaseBase + kReleaseStride * (me & 7u));
         }
         __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -169,18 +174,19 @@ __device__ __forceinline__ void route_token(const float* logits, uint32_t E, uin
     if (lane < topk) weights[lane] = v * inverse;
 }
 
-constexpr int kRing = 8;         // 128-element spans of a tile in flight per lane (four when the span count is odd in eights)
-#define ZC_RUN_TILE(SPANS, ...) do { if ((SPANS) % 8 == 0) xint_run_tile<PT, 8>(__VA_ARGS__); else xint_run_tile<PT, 4>(__VA_ARGS__); } while (0)
-constexpr int kMaxTokens = 8;
+constexpr int kRing = 8;         // sixteen-byte pieces of a router partition in flight per lane; tiles keep eight 128-element spans
+                                 // in flight with one wave per SIMD and four with two
+#define ZC_RUN_TILE(SPANS, ...) do { if (NT != 1 && (SPANS) % 8 == 0) xint_run_tile<PT, 8>(__VA_ARGS__); else xint_run_tile<PT, 4>(__VA_ARGS__); } while (0)
 
 // NT = 1: single-token decode.  NT = 8: up to eight tokens, tiles take four at a time.
 template <int NT>
-__global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
+__global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
     constexpr int PT = NT < 4 ? NT : 4;   // tokens per tile pass
+    constexpr uint32_t kDecodeThreads = decode_threads(NT), kDecodeWaves = kDecodeThreads / 64;
     extern __shared__ __align__(16) uint8_t lds[];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wg = blockIdx.x, nwg = gridDim.x;
+    uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, col = lane & 15u, G = lane >> 4;
+    const uint32_t wg = blockIdx.x, nwg = gridDim.x;
     const uint32_t H = p.H, E = p.E, I = p.I, k = p.topk, T = p.T, n = T * k;
-    const uint32_t col = lane & 15u, G = lane >> 4;
     int32_t* ids = reinterpret_cast<int32_t*>(lds + lp.ids);
     float* weights = reinterpret_cast<float*>(lds + lp.weights);
     float* gatev = reinterpret_cast<float*>(lds + lp.gatev);
@@ -209,6 +215,13 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
 
     for (uint32_t layer = 0; layer < p.L; ++layer) {
         const DecodeLayer L = p.layers[layer];
+        // Per-lane addresses and predicates derived from the thread index are recomputed in every layer: hoisted out of
+        // the layer loop they would stay live through all phases and spill.
+        auto refresh = [&]() {
+            asm volatile("" : "+v"(tid));
+            lane = tid & 63u; wave = uint32_t(uniform(int32_t(tid >> 6))); col = lane & 15u; G = lane >> 4;
+        };
+        refresh();
         clock();
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
@@ -228,12 +241,17 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 __syncthreads();
             }
             // the shared-expert gate row rides along: coalesced sixteen-byte loads, used from LDS by the gate-dot waves
-            uint4 gate_piece[2];
+            constexpr int kGatePieces = (3072 / 8 + kDecodeThreads - 1) / kDecodeThreads;   // hidden <= 3072
+            uint4 gate_piece[kGatePieces];
 #pragma unroll
-            for (int q = 0; q < 2; ++q) if (NT == 1 && tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
+            for (int q = 0; q < kGatePieces; ++q) gate_piece[q] = make_uint4(0, 0, 0, 0);
             const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh),
                 [&]() {
-                    if constexpr (NT == 1) { const float m = __uint_as_float(peak); inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f; }
+                    if constexpr (NT == 1) {
+#pragma unroll
+                        for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
+                        const float m = __uint_as_float(peak); inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+                    }
                 },
                 [&](uint32_t i, float& a, float& b) {
                     if (glue) {
@@ -243,7 +261,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
                 });
             if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
 #pragma unroll
-            for (int q = 0; q < 2; ++q) if (tid + q * kDecodeThreads < H / 8) {
+            for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) {
                 if constexpr (NT != 1) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);   // several tokens: after the rows, to spare registers
                 reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
             }
@@ -327,6 +345,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
         }
         clock_all();
         bar.wait();
+        refresh();
         clock();
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
         for (uint32_t t = wave; t < T; t += kDecodeWaves)
@@ -391,6 +410,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_stack_kernel(DecodePara
         }
         clock_all();
         bar.wait();
+        refresh();
         clock();
         // ---------------- phase D: down tiles per 16 output rows, combine ----------------
         float* otile = reinterpret_cast<float*>(lds + lp.otile);
@@ -517,7 +537,7 @@ hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<NT>),                  \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));             \
         if (e != hipSuccess) return e;                                                                             \
-        hipLaunchKernelGGL((decode_stack_kernel<NT>), dim3(workgroups), dim3(kDecodeThreads), lp.total, s, p, lp);  \
+        hipLaunchKernelGGL((decode_stack_kernel<NT>), dim3(workgroups), dim3(decode_threads(NT)), lp.total, s, p, lp);  \
     } while (0)
     if (nt == 1) ZC_DECODE(1); else ZC_DECODE(8);
 #undef ZC_DECODE
@@ -527,8 +547,8 @@ hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_p
     const void* f = nt == 1 ? reinterpret_cast<const void*>(decode_stack_kernel<1>) : reinterpret_cast<const void*>(decode_stack_kernel<8>);
     hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
-    if (nt == 1) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<1>, kDecodeThreads, lds_bytes);
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<8>, kDecodeThreads, lds_bytes);
+    if (nt == 1) return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<1>, decode_threads(1), lds_bytes);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<8>, decode_threads(8), lds_bytes);
 }
 
 }  // namespace zc

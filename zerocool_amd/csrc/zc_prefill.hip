@@ -27,7 +27,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kTileRows = 32, kTileCols = 128, kStepK = 64, kPitch = 72;   // LDS row pitch in bf16 elements (144 bytes)
+constexpr uint32_t kTileRows = 32, kTileCols = 128, kPitch = 72;   // LDS row pitch in bf16 elements (144 bytes)
 
 // fp32 rows holding BF16 values -> bf16 rows, plus per (row, group of 64) the sum of the four blocks' BF16-rounded
 // sum-of-four chains.  One thread per (row, group).  status bit 4: a value was not BF16-valued.

@@ -149,9 +149,11 @@ __device__ __forceinline__ void xint_prepare_block(const Source x, const XintLay
 // Clears the unsafe masks and zero slots of `count` consecutive images (stride L.bytes()).
 __device__ __forceinline__ void xint_prepare_begin(const XintLayout L, uint8_t* lds, uint32_t count) {
     const uint32_t words = L.mask_bytes() / 4;
-    for (uint32_t i = threadIdx.x; i < count * words; i += blockDim.x)
+    uint32_t first = threadIdx.x;
+    asm volatile("" : "+v"(first));   // addresses are formed here, not hoisted out of a caller's outer loop
+    for (uint32_t i = first; i < count * words; i += blockDim.x)
         reinterpret_cast<uint32_t*>(lds + (i / words) * L.bytes() + L.planes_bytes() + L.info_bytes())[i % words] = 0;
-    for (uint32_t i = threadIdx.x; i < count * 4; i += blockDim.x)
+    for (uint32_t i = first; i < count * 4; i += blockDim.x)
         reinterpret_cast<uint32_t*>(lds + (i / 4) * L.bytes() + L.blocks() * 48)[i % 4] = 0;
 }
 // Builds `count` images cooperatively: all threads call it; source_of(q) gives image q's
@@ -161,7 +163,9 @@ __device__ __forceinline__ void xint_prepare_batch(const SourceOf source_of, uin
     xint_prepare_begin(L, lds, count);
     __syncthreads();
     const uint32_t blocks = L.blocks();
-    for (uint32_t i = threadIdx.x; i < count * blocks; i += blockDim.x) {
+    uint32_t first = threadIdx.x;
+    asm volatile("" : "+v"(first));
+    for (uint32_t i = first; i < count * blocks; i += blockDim.x) {
         const uint32_t q = i / blocks;
         xint_prepare_block(source_of(q), L, lds + q * L.bytes(), i % blocks);
     }

@@ -54,8 +54,11 @@ def run_stack(ctx, cfg, stack, x_dev, T, L, layered):
     return r
 
 
-def _check_stack(ctx, cfg, L, tokens, seed, skew, persistent):
+def _check_stack(ctx, cfg, L, tokens, seed, skew, persistent, mutate=None):
     layers = [workload.LayerWeights(ctx, cfg, seed + l, skew) for l in range(L)]
+    if mutate:
+        for l in layers:
+            mutate(l)
     hosts = [l.host() for l in layers]
     stack = ctx.stack_create(cfg, [l.layer for l in layers], max(tokens))
     for T in tokens:
@@ -79,8 +82,8 @@ def _check_stack(ctx, cfg, L, tokens, seed, skew, persistent):
             ctx.free(b)
 
 
-def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1), persistent=True):
-    return _check_stack(ctx, cfg, L, tokens, seed, skew, persistent)
+def check_stack(ctx, cfg, L, tokens, seed=31, skew=("zipf", 1.1), persistent=True, mutate=None):
+    return _check_stack(ctx, cfg, L, tokens, seed, skew, persistent, mutate)
 
 
 def test_few_experts_stack(ctx):  # the single-layer shape (hidden 2048 / intermediate 512) with few experts
@@ -93,6 +96,19 @@ def test_single_layer_shape_stack(ctx):
 
 def test_small_hidden_stack(ctx):
     check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512), 2, [1, 4])
+
+
+def test_tied_logits_pick_the_lowest_ids(ctx):
+    # 512 experts whose router rows repeat in runs of twelve: every run ties exactly, so the ten picks are the ten
+    # lowest ids of the best run, in ascending order, and the softmax weights are all equal
+    cfg = workload.tiny_config(hidden=1024, experts=512, topk=10, inter=512)
+
+    def repeat_rows(layer):
+        rows = layer.router.numpy(np.uint16).reshape(cfg.experts, cfg.hidden)
+        rows = rows[(np.arange(cfg.experts) // 12) * 12]
+        layer.ctx.upload(np.ascontiguousarray(rows).reshape(-1), into=layer.router)
+
+    check_stack(ctx, cfg, 2, [1, 3], skew=None, mutate=repeat_rows)
 
 
 def test_other_shapes_take_the_layered_path(ctx):  # hidden not a multiple of 512

@@ -127,6 +127,22 @@ zc_status zc_hip_scatter_experts(zc_hip_ctx* ctx, const float* x, const int32_t*
 zc_status zc_hip_moe_sum(zc_hip_ctx* ctx, const float* experts, const float* weights,
                          const float* shared, const float* gate, uint32_t tokens,
                          uint32_t hidden, uint32_t topk, float* out);
+/* The callers' glue either side of Model::moe: Model::unary / Model::binary (model.cpp:328-336 ->
+ * dispatch("unary"), dispatch("binary"); qwen.metal:567-581).  op: 0 SiLU, 1 sigmoid, 2 SiLU(x/4),
+ * 3 2*sigmoid(x/4), 4 softplus; binary op 0 adds, any other multiplies.  Results are BF16-valued fp32. */
+zc_status zc_hip_unary(zc_hip_ctx* ctx, const float* x, uint64_t n, uint32_t op, float* y);
+zc_status zc_hip_binary(zc_hip_ctx* ctx, const float* x, const float* y, uint64_t n, uint32_t op, float* out);
+/* dispatch("hc_mix") in Model::hyper (model.cpp:343; qwen.metal:582-588): x, w [tokens][4][hidden] ->
+ * out [tokens][hidden]. */
+zc_status zc_hip_hc_mix(zc_hip_ctx* ctx, const float* x, const float* w, uint32_t tokens, uint32_t hidden, float* out);
+/* dispatch("hc_add") after attention and after the MoE layer (model.cpp:651, 662; qwen.metal:589-595):
+ * hyper [tokens][4][hidden], x [tokens][hidden], inject [tokens][4] -> out [tokens][4][hidden]. */
+zc_status zc_hip_hc_add(zc_hip_ctx* ctx, const float* hyper, const float* x, const float* inject,
+                        uint32_t tokens, uint32_t hidden, float* out);
+/* Model::norm -> dispatch("norm") / dispatch("norm_wide") (model.cpp:312-326; qwen.metal:545-566, 403-426):
+ * RMS norm over groups of `group` elements (<= 4096) of rows of `width`; w: `width` weights, dtype 0 BF16, 1 fp32. */
+zc_status zc_hip_norm(zc_hip_ctx* ctx, const float* x, const void* w, uint32_t dtype, uint32_t group,
+                      uint32_t width, uint32_t tokens, float* out);
 /* Metal::grouped_experts (metal.mm:881-912): n<=8 records (host array of device
  * pointers), distinct positions < topk (host array); scratch holds n*inter floats. */
 zc_status zc_hip_grouped_experts(zc_hip_ctx* ctx, const zc_moe_config* cfg,

@@ -50,6 +50,8 @@ def _load():
     lib.zco_projection_bytes.restype = C.c_uint64
     lib.zco_projection_bytes.argtypes = [C.c_uint32] * 4
     lib.zco_record_bytes.restype = C.c_uint64
+    lib.zco_softplus_bf.restype = f32; lib.zco_softplus_bf.argtypes = [f32]
+    lib.zco_unary.restype = f32; lib.zco_unary.argtypes = [f32, C.c_uint32]
     return lib
 
 
@@ -175,3 +177,41 @@ def moe_layer(cfg, router, shared_gate, shared_record, expert_records, record_st
     if status:
         raise RuntimeError("invalid router output")
     return (out, tr) if trace else out
+
+
+# ---- the callers' glue either side of the layer
+
+
+def unary(x, op):
+    x = np.ascontiguousarray(x, dtype=np.float32); y = np.empty_like(x)
+    lib.zco_unary_n(_p(x), C.c_uint64(x.size), C.c_uint32(op), _p(y))
+    return y
+
+
+def binary(x, y, op):
+    x = np.ascontiguousarray(x, dtype=np.float32); y = np.ascontiguousarray(y, dtype=np.float32); out = np.empty_like(x)
+    lib.zco_binary_n(_p(x), _p(y), C.c_uint64(x.size), C.c_uint32(op), _p(out))
+    return out
+
+
+def hc_mix(x, w, tokens, hidden):
+    x = np.ascontiguousarray(x, dtype=np.float32); w = np.ascontiguousarray(w, dtype=np.float32)
+    out = np.empty((tokens, hidden), np.float32)
+    lib.zco_hc_mix(_p(x), _p(w), C.c_uint32(tokens), C.c_uint32(hidden), _p(out))
+    return out
+
+
+def hc_add(hyper, x, inject, tokens, hidden):
+    a = [np.ascontiguousarray(v, dtype=np.float32) for v in (hyper, x, inject)]
+    out = np.empty((tokens, 4, hidden), np.float32)
+    lib.zco_hc_add(_p(a[0]), _p(a[1]), _p(a[2]), C.c_uint32(tokens), C.c_uint32(hidden), _p(out))
+    return out
+
+
+def norm(x, w, group, width, tokens):
+    """w: uint16 (BF16 bits) or float32 weights of length width."""
+    x = np.ascontiguousarray(x, dtype=np.float32); w = np.ascontiguousarray(w)
+    dtype = 1 if w.dtype == np.float32 else 0
+    out = np.empty(tokens * width, np.float32)
+    lib.zco_norm(_p(x), _p(w), C.c_uint32(dtype), C.c_uint32(group), C.c_uint32(width), C.c_uint32(tokens), _p(out))
+    return out

@@ -58,11 +58,85 @@ float zco_sigmoid_bf(float x) {
     return x < 0 ? y : zco_bf(1.0f - y);
 }
 
+/*
+ * log(y) for y in [1, 2], evaluated in double from basic operations only (division, fused multiply-add), so the
+ * device computes the same bits: log y = 2 atanh z, z = (y-1)/(y+1) <= 1/3, odd series to z^35.  Rounded to
+ * fp32 once.  Stands in for Metal's log in softplus_bf (qwen.metal:36-40).
+ */
+float zco_log_1to2(float y) {
+    const double z = ((double)y - 1.0) / ((double)y + 1.0), z2 = z * z;
+    double p = 1.0 / 35.0;
+    for (int k = 33; k >= 1; k -= 2) p = fma(p, z2, 1.0 / (double)k);
+    return (float)(2.0 * z * p);
+}
+/* qwen.metal:36-40 */
+float zco_softplus_bf(float x) {
+    const float e = zco_bf(zco_expf(-fabsf(x))), one = 1.0f + e;
+    const float tail = one == 1.0f ? e : e * (zco_log_1to2(one) / (one - 1.0f));
+    return zco_bf(fmaxf(x, 0.0f) + zco_bf(tail));
+}
+/* kernel unary (qwen.metal:567-577): 0 SiLU, 1 sigmoid, 2 SiLU(x/4), 3 2*sigmoid(x/4), 4 softplus */
+float zco_unary(float v, uint32_t op) {
+    if (op == 0) v = v * zco_sigmoid_bf(v);
+    if (op == 1) v = zco_sigmoid_bf(v);
+    if (op == 2) { v = zco_bf(v / 4); v = v * zco_sigmoid_bf(v); }
+    if (op == 3) v = 2 * zco_bf(zco_sigmoid_bf(zco_bf(v / 4)));
+    if (op == 4) v = zco_softplus_bf(v);
+    return zco_bf(v);
+}
+void zco_unary_n(const float* x, uint64_t n, uint32_t op, float* y) { for (uint64_t i = 0; i < n; ++i) y[i] = zco_unary(x[i], op); }
+/* kernel binary (qwen.metal:578-581): op 0 add, otherwise multiply */
+void zco_binary_n(const float* x, const float* y, uint64_t n, uint32_t op, float* out) {
+    for (uint64_t i = 0; i < n; ++i) out[i] = zco_bf(op ? x[i] * y[i] : x[i] + y[i]);
+}
+/* kernel hc_mix (qwen.metal:582-588): x, w are [tokens][4][hidden]; BF16 rounding of every product and partial sum */
+void zco_hc_mix(const float* x, const float* w, uint32_t tokens, uint32_t hidden, float* out) {
+    for (uint32_t t = 0; t < tokens; ++t)
+        for (uint32_t d = 0; d < hidden; ++d) {
+            float sum = 0;
+            for (uint32_t h = 0; h < 4; ++h) { const uint64_t k = ((uint64_t)t * 4 + h) * hidden + d; sum = zco_bf(sum + zco_bf(x[k] * w[k])); }
+            out[(uint64_t)t * hidden + d] = zco_bf(sum / 4);
+        }
+}
+/* kernel hc_add (qwen.metal:589-595): hyper [tokens][4][hidden], x [tokens][hidden], inject [tokens][4] */
+void zco_hc_add(const float* hyper, const float* x, const float* inject, uint32_t tokens, uint32_t hidden, float* out) {
+    for (uint32_t t = 0; t < tokens; ++t)
+        for (uint32_t h = 0; h < 4; ++h)
+            for (uint32_t d = 0; d < hidden; ++d) {
+                const uint64_t k = ((uint64_t)t * 4 + h) * hidden + d;
+                out[k] = zco_bf(hyper[k] + zco_bf(x[(uint64_t)t * hidden + d] * inject[t * 4 + h]));
+            }
+}
+
 /* The fixed association this oracle gives simd_sum: xor butterfly 16,8,4,2,1. */
 static float simd_sum(float* lane) {
     for (uint32_t stride = ZCO_LANES / 2; stride; stride >>= 1)
         for (uint32_t l = 0; l < stride; ++l) lane[l] = lane[l] + lane[l + stride];
     return lane[0];
+}
+/* rms_square_sum + kernel norm (qwen.metal:545-566): grouped RMS norm, D <= 4096 per group.  Each 128-element
+ * block gives every lane a sum of four squares, a lane sum, and lane block/128 keeps it; a second lane sum adds the
+ * blocks.  precise::rsqrt is taken as 1 / sqrt (two correctly rounded operations).  w: dtype 0 BF16, 1 fp32. */
+void zco_norm(const float* x, const void* w, uint32_t dtype, uint32_t D, uint32_t width, uint32_t tokens, float* out) {
+    const uint64_t groups = (uint64_t)tokens * (width / D);
+    for (uint64_t g = 0; g < groups; ++g) {
+        const float* xg = x + g * D;
+        float contribution[32] = {0};
+        for (uint32_t block = 0; block < D; block += 128) {
+            float acc[32];
+            for (uint32_t lane = 0; lane < 32; ++lane) {
+                acc[lane] = 0;
+                for (uint32_t i = 0; i < 4; ++i) { const uint32_t d = block + lane * 4 + i; if (d < D) acc[lane] += xg[d] * xg[d]; }
+            }
+            contribution[block / 128] = simd_sum(acc);
+        }
+        const float inv = 1.0f / sqrtf(simd_sum(contribution) / (float)D + 1e-6f);
+        for (uint32_t d = 0; d < D; ++d) {
+            const uint64_t i = g * D + d; const uint32_t wi = (uint32_t)(i % width);
+            const float weight = dtype == 1 ? ((const float*)w)[wi] : zco_b16(((const uint16_t*)w)[wi]);
+            out[i] = zco_bf(zco_bf(xg[d] * inv) * weight);
+        }
+    }
 }
 /* Note: lane l and lane l^stride compute the same commutative sum, so keeping
  * only the lower half at every step gives lane 0's butterfly value exactly. */

@@ -84,6 +84,17 @@ void zco_scatter_experts(const float* x, const int32_t* positions, uint32_t n, u
 void zco_moe_sum(const float* experts, const float* weights, const float* shared,
                  const float* gate, uint32_t tokens, uint32_t H, uint32_t topk, float* out);
 
+/* The callers' glue either side of the layer (model.cpp:328-351, 651, 662): element-wise operators, the
+ * four-stream mix and residual injection, grouped RMS norm. */
+float zco_log_1to2(float y);
+float zco_softplus_bf(float x);                                                       /* qwen.metal:36-40 */
+float zco_unary(float v, uint32_t op);                                                /* qwen.metal:567-577 */
+void zco_unary_n(const float* x, uint64_t n, uint32_t op, float* y);
+void zco_binary_n(const float* x, const float* y, uint64_t n, uint32_t op, float* out);   /* qwen.metal:578-581 */
+void zco_hc_mix(const float* x, const float* w, uint32_t tokens, uint32_t hidden, float* out);   /* qwen.metal:582-588 */
+void zco_hc_add(const float* hyper, const float* x, const float* inject, uint32_t tokens, uint32_t hidden, float* out);   /* qwen.metal:589-595 */
+void zco_norm(const float* x, const void* w, uint32_t dtype, uint32_t D, uint32_t width, uint32_t tokens, float* out);    /* qwen.metal:545-566 */
+
 /* A whole layer (model.cpp:431-557). */
 typedef struct {
     uint32_t hidden, experts, topk, inter, group;

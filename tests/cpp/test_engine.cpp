@@ -260,8 +260,53 @@ static void test_expert_cache() {   // :336-348 on the GPU, and moe() reading it
     CHECK(st.misses >= s.topk); CHECK(st.hits + st.misses >= 6 * s.topk); CHECK(st.bytes == st.misses * s.expert_bytes());
     cache.clear(); CHECK(cache.occupancy() == 0);
 }
+static void test_glue() {   // :53, :876-897, :1137-1145 and the glue of model.cpp:328-351, 651
+    TEST("element-wise dispatches, the stream mix / injection and the grouped norm");
+    Metal gpu; const uint32_t H = gpu.shape().hidden;
+    auto x = gpu.zeros(32), y = gpu.zeros(32);
+    for (int i = 0; i < 32; ++i) x->floats()[i] = round_bf16(float(i - 16) / 8);
+    gpu.dispatch("binary", {{x}, {x}, {y}}, {32, 0}, 32); gpu.finish();
+    for (int i = 0; i < 32; ++i) CHECK(y->floats()[i] == 2 * x->floats()[i]);
+    auto edge = gpu.zeros(2), out = gpu.zeros(2); edge->floats()[0] = -6.84375f; edge->floats()[1] = 6.84375f;
+    gpu.dispatch("unary", {{edge}, {out}}, {2, 0}, 2); gpu.finish();
+    CHECK(out->floats()[0] == -0.00726318359375f); CHECK(out->floats()[1] == 6.84375f);   // the captured exp rounding boundary
+    gpu.dispatch("unary", {{edge}, {out}}, {2, 4}, 2); gpu.finish();
+    CHECK(out->floats()[1] == 6.84375f && out->floats()[0] > 0 && out->floats()[0] < 0.0011f);
+    CHECK_THROWS(gpu.dispatch("unary", {{edge}, {out}}, {2, 9}, 2));
+    CHECK_THROWS(gpu.dispatch("binary", {{edge}, {x}, {out}}, {32, 0}, 32));
+    // four streams: mixing with unit weights averages them, injecting with zero leaves the streams alone
+    const uint32_t T = 2;
+    auto streams = gpu.zeros(uint64_t(T) * 4 * H), ones = gpu.zeros(uint64_t(T) * 4 * H), mixed = gpu.zeros(uint64_t(T) * H);
+    for (size_t i = 0; i < streams->floats().size(); ++i) { streams->floats()[i] = round_bf16(float(int(i % 23) - 11) / 16); ones->floats()[i] = 1; }
+    gpu.dispatch("hc_mix", {{streams}, {ones}, {mixed}}, {T}, H, T); gpu.finish();
+    for (uint32_t t = 0; t < T; ++t) for (uint32_t d = 0; d < H; d += 97) {
+        float sum = 0; for (uint32_t h = 0; h < 4; ++h) sum = round_bf16(sum + streams->floats()[(uint64_t(t) * 4 + h) * H + d]);
+        CHECK(mixed->floats()[uint64_t(t) * H + d] == round_bf16(sum / 4));
+    }
+    auto inject = gpu.zeros(T * 4), after = gpu.zeros(uint64_t(T) * 4 * H);
+    gpu.dispatch("hc_add", {{streams}, {mixed}, {inject}, {after}}, {T}, 4 * H, T); gpu.finish();
+    CHECK(std::memcmp(after->data, streams->data, after->bytes) == 0);
+    for (uint32_t i = 0; i < T * 4; ++i) inject->floats()[i] = float(i % 3) - 1;
+    gpu.dispatch("hc_add", {{streams}, {mixed}, {inject}, {after}}, {T}, 4 * H, T); gpu.finish();
+    CHECK(after->floats()[5 * H + 7] == round_bf16(streams->floats()[5 * H + 7] + round_bf16(mixed->floats()[H + 7] * inject->floats()[5])));
+    // grouped RMS norm: both kernel names give the same bytes, also for a group that is not a multiple of 128
+    for (auto [D, width, tokens] : std::array<std::tuple<uint32_t, uint32_t, uint32_t>, 3>{{{2560, 10240, 3}, {512, 1024, 2}, {320, 640, 1}}}) {
+        auto in = gpu.zeros(uint64_t(width) * tokens), w = gpu.allocate(width * 2), a = gpu.allocate(in->bytes), b = gpu.allocate(in->bytes);
+        for (size_t i = 0; i < in->floats().size(); ++i) in->floats()[i] = round_bf16(float(int(i * 7 % 61) - 30) / 10);
+        for (uint32_t i = 0; i < width; ++i) reinterpret_cast<uint16_t*>(w->data)[i] = 0x3f80 + uint16_t(i % 5);
+        const uint32_t threads = 32 * ((D + 127) / 128);
+        gpu.dispatch("norm", {{in}, {w}, {a}}, {D, width, tokens, 0, 1}, tokens * (width / D) * 32);
+        gpu.dispatch("norm_wide", {{in}, {w}, {b}}, {D, width, tokens, 0, 1}, tokens * (width / D) * threads, 1, 1, threads); gpu.finish();
+        CHECK(std::memcmp(a->data, b->data, a->bytes) == 0);
+        double ms = 0; for (uint32_t d = 0; d < D; ++d) ms += double(in->floats()[d]) * in->floats()[d];
+        const double want = in->floats()[3] / std::sqrt(ms / D + 1e-6) * bf16(reinterpret_cast<uint16_t*>(w->data)[3]);
+        CHECK(std::fabs(a->floats()[3] - want) <= std::fabs(want) / 64);
+    }
+    CHECK_THROWS(gpu.dispatch("norm", {{x}, {x}, {y}}, {48, 100, 1, 0, 1}, 32));
+}
+
 int main() {
-    test_bf16(); test_q4_matmul(); test_route(); test_moe_sum(); test_direct_rows(); test_grouped(); test_heavy_rows(); test_moe_layer(); test_expert_cache();
+    test_glue(); test_bf16(); test_q4_matmul(); test_route(); test_moe_sum(); test_direct_rows(); test_grouped(); test_heavy_rows(); test_moe_layer(); test_expert_cache();
     std::printf("%d checks, %d failures\n", checks, failures);
     return failures ? 1 : 0;
 }

@@ -202,6 +202,24 @@ void Metal::dispatch(const std::string& name, std::initializer_list<Binding> buf
         if (b.size() != 3 || p.size() != 1 || x != shape_.hidden || y != p[0]) throw std::invalid_argument("scatter_experts dispatch shape");
         check(zc_hip_scatter_experts(ctx_, static_cast<const float*>(at(b[0])), static_cast<const int32_t*>(at(b[1])), p[0], shape_.hidden,
                                      static_cast<float*>(at(b[2]))));
+    } else if (name == "unary") {   // model.cpp:330: {x, out}, {count, op}
+        if (b.size() != 2 || p.size() != 2 || x != p[0] || b[0].buffer->bytes - b[0].offset < uint64_t(p[0]) * 4 || b[1].buffer->bytes - b[1].offset < uint64_t(p[0]) * 4)
+            throw std::invalid_argument("unary dispatch shape");
+        check(zc_hip_unary(ctx_, static_cast<const float*>(at(b[0])), p[0], p[1], static_cast<float*>(at(b[1]))));
+    } else if (name == "binary") {   // model.cpp:335: {x, y, out}, {count, op}
+        if (b.size() != 3 || p.size() != 2 || x != p[0]) throw std::invalid_argument("binary shape mismatch");
+        for (const auto& v : b) if (v.buffer->bytes - v.offset < uint64_t(p[0]) * 4) throw std::invalid_argument("binary shape mismatch");
+        check(zc_hip_binary(ctx_, static_cast<const float*>(at(b[0])), static_cast<const float*>(at(b[1])), p[0], p[1], static_cast<float*>(at(b[2]))));
+    } else if (name == "hc_mix") {   // model.cpp:343: {n, mix, out}, {tokens}, grid hidden x tokens
+        if (b.size() != 3 || p.size() != 1 || x != shape_.hidden || y != p[0]) throw std::invalid_argument("hc_mix dispatch shape");
+        check(zc_hip_hc_mix(ctx_, static_cast<const float*>(at(b[0])), static_cast<const float*>(at(b[1])), p[0], shape_.hidden, static_cast<float*>(at(b[2]))));
+    } else if (name == "hc_add") {   // model.cpp:651: {hyper, x, inject, out}, {tokens}, grid 4*hidden x tokens
+        if (b.size() != 4 || p.size() != 1 || x != 4 * shape_.hidden || y != p[0]) throw std::invalid_argument("hc_add dispatch shape");
+        check(zc_hip_hc_add(ctx_, static_cast<const float*>(at(b[0])), static_cast<const float*>(at(b[1])), static_cast<const float*>(at(b[2])), p[0],
+                            shape_.hidden, static_cast<float*>(at(b[3]))));
+    } else if (name == "norm" || name == "norm_wide") {   // model.cpp:318-325: {x, w, out}, {group, width, tokens, dtype, grouped}
+        if (b.size() != 3 || p.size() != 5 || !p[0] || p[1] % p[0]) throw std::invalid_argument("normalization shape");
+        check(zc_hip_norm(ctx_, static_cast<const float*>(at(b[0])), at(b[1]), p[3], p[0], p[1], p[2], static_cast<float*>(at(b[2]))));
     } else throw std::invalid_argument("unknown kernel: " + name);
 }
 

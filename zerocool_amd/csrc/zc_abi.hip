@@ -331,6 +331,36 @@ zc_status zc_hip_moe_sum(zc_hip_ctx* ctx, const float* experts, const float* wei
     ZC_LAUNCHED();
     return ZC_OK;
 }
+zc_status zc_hip_unary(zc_hip_ctx* ctx, const float* x, uint64_t n, uint32_t op, float* y) {
+    ZC_REQUIRE(ctx && x && y && n && op <= 4, "invalid unary operator or buffers");
+    zc::launch_unary(ctx->stream, x, n, op, y);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_binary(zc_hip_ctx* ctx, const float* x, const float* y, uint64_t n, uint32_t op, float* out) {
+    ZC_REQUIRE(ctx && x && y && out && n, "binary shape mismatch");
+    zc::launch_binary(ctx->stream, x, y, n, op, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_hc_mix(zc_hip_ctx* ctx, const float* x, const float* w, uint32_t tokens, uint32_t hidden, float* out) {
+    ZC_REQUIRE(ctx && x && w && out && tokens && hidden && x != out && w != out, "invalid stream mix buffers");
+    zc::launch_hc_mix(ctx->stream, x, w, tokens, hidden, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_hc_add(zc_hip_ctx* ctx, const float* hyper, const float* x, const float* inject, uint32_t tokens, uint32_t hidden, float* out) {
+    ZC_REQUIRE(ctx && hyper && x && inject && out && tokens && hidden && x != out && inject != out, "invalid residual injection buffers");
+    zc::launch_hc_add(ctx->stream, hyper, x, inject, tokens, hidden, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
+zc_status zc_hip_norm(zc_hip_ctx* ctx, const float* x, const void* w, uint32_t dtype, uint32_t group, uint32_t width, uint32_t tokens, float* out) {
+    ZC_REQUIRE(ctx && x && w && out && tokens && group && width && width % group == 0 && group <= 4096 && dtype <= 1, "normalization shape");
+    zc::launch_norm(ctx->stream, x, w, dtype, group, width, tokens, out);
+    ZC_LAUNCHED();
+    return ZC_OK;
+}
 zc_status zc_hip_grouped_experts(zc_hip_ctx* ctx, const zc_moe_config* cfg, const void* const* records,
                                  const uint32_t* positions, uint32_t n, const float* x, float* out, float* scratch) {
     if (const zc_status s = validate_config(cfg)) return s;

@@ -38,6 +38,12 @@ void launch_route(hipStream_t s, const float* logits, uint32_t T, uint32_t E, ui
 void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets,
                      int32_t* slots, int32_t* rows, int32_t* selected, int32_t* count, int32_t* status);
 void launch_scatter(hipStream_t s, const float* x, const int32_t* positions, uint32_t n, uint32_t H, float* out);
+// ---- the callers' glue either side of the layer (zc_glue.hip)
+void launch_unary(hipStream_t s, const float* x, uint64_t n, uint32_t op, float* y);
+void launch_binary(hipStream_t s, const float* x, const float* y, uint64_t n, uint32_t op, float* out);
+void launch_hc_mix(hipStream_t s, const float* x, const float* w, uint32_t tokens, uint32_t hidden, float* out);
+void launch_hc_add(hipStream_t s, const float* hyper, const float* x, const float* inject, uint32_t tokens, uint32_t hidden, float* out);
+void launch_norm(hipStream_t s, const float* x, const void* w, uint32_t dtype, uint32_t D, uint32_t width, uint32_t tokens, float* out);
 void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, const float* shared, const float* gate,
                     uint32_t T, uint32_t H, uint32_t topk, float* out);
 void launch_stack_glue(hipStream_t s, const float* y, uint32_t T, uint32_t H, float* out);

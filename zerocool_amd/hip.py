@@ -303,6 +303,32 @@ class Context:
                    C.c_uint32(hidden), C.c_uint32(topk), _ptr(out))
         return out
 
+    # ---- the callers' glue either side of the layer
+    def unary(self, x, n, op, out=None):
+        out = out or self.alloc(n * 4)
+        self._call("zc_hip_unary", _ptr(x), C.c_uint64(n), C.c_uint32(op), _ptr(out))
+        return out
+
+    def binary(self, x, y, n, op, out=None):
+        out = out or self.alloc(n * 4)
+        self._call("zc_hip_binary", _ptr(x), _ptr(y), C.c_uint64(n), C.c_uint32(op), _ptr(out))
+        return out
+
+    def hc_mix(self, x, w, tokens, hidden, out=None):
+        out = out or self.alloc(tokens * hidden * 4)
+        self._call("zc_hip_hc_mix", _ptr(x), _ptr(w), C.c_uint32(tokens), C.c_uint32(hidden), _ptr(out))
+        return out
+
+    def hc_add(self, hyper, x, inject, tokens, hidden, out=None):
+        out = out or self.alloc(tokens * 4 * hidden * 4)
+        self._call("zc_hip_hc_add", _ptr(hyper), _ptr(x), _ptr(inject), C.c_uint32(tokens), C.c_uint32(hidden), _ptr(out))
+        return out
+
+    def norm(self, x, w, dtype, group, width, tokens, out=None):
+        out = out or self.alloc(tokens * width * 4)
+        self._call("zc_hip_norm", _ptr(x), _ptr(w), C.c_uint32(dtype), C.c_uint32(group), C.c_uint32(width), C.c_uint32(tokens), _ptr(out))
+        return out
+
     def grouped_experts(self, cfg, records, positions, x, out, scratch):
         n = len(records)
         recs = (C.c_void_p * max(n, 1))(*[r.ptr for r in records])

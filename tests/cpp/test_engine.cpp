@@ -2,6 +2,8 @@
 // (tests/test_qwen.cpp, cited per case): build tiny deterministic inputs through the Buffer
 // interface, run the operators, compare bytes.  The CPU oracle (oracle/zc_oracle.h) is the checker.
 #include "../../zerocool_amd/csrc/engine/engine.hpp"
+#include "../../zerocool_amd/csrc/engine/records.hpp"
+#include <unistd.h>
 #include "../../oracle/zc_oracle.h"
 #include <algorithm>
 #include <bit>
@@ -220,11 +222,17 @@ static void test_expert_cache() {   // :336-348 on the GPU, and moe() reading it
     ExpertCache cache(gpu, 1, s.topk + 2);
     const uint64_t stride = (s.expert_bytes() + 255) / 256 * 256;
     std::vector<std::byte> all(stride * s.experts);
-    for (uint32_t e = 0; e < s.experts; ++e) {
-        auto r = expert_fixture(s, 300 + e);
-        std::memcpy(all.data() + e * stride, r.data(), r.size());
-        std::memcpy(cache.home({0, e}).data(), r.data(), r.size());
+    // the records travel through a prepared directory on disk, as they would from the reference's prepare step
+    const auto dir = std::filesystem::temp_directory_path() / ("zc_engine_prepared_" + std::to_string(::getpid()));
+    write_prepared_experts(dir, s, 1, [&](ExpertKey k, std::span<std::byte> into) { auto r = expert_fixture(s, 300 + k.expert); std::memcpy(into.data(), r.data(), r.size()); });
+    {
+        PreparedExperts prepared(dir, s);
+        prepared.layer(0, all, stride);                                           // an HBM layer array's layout
+        for (uint32_t e = 0; e < s.experts; ++e) prepared.expert({0, e}, cache.home({0, e}));   // the pinned home of the slot cache
+        auto r = expert_fixture(s, 300 + 5);
+        CHECK(std::memcmp(all.data() + 5 * stride, r.data(), r.size()) == 0 && std::memcmp(cache.home({0, 5}).data(), r.data(), r.size()) == 0);
     }
+    std::filesystem::remove_all(dir);
     {
         std::vector<ExpertCache::Lease> leases;
         for (uint32_t e = 0; e < s.topk + 2; ++e) leases.push_back(cache.acquire({0, e}));

@@ -1,0 +1,112 @@
+// Tests of the on-disk expert record readers (zerocool_amd/csrc/engine/records.hpp); no GPU needed.
+// Follows the checks of the reference's PreparedArtifact / ExpertStore (src/engine/storage.cpp:316-394, 493-516).
+#include "../../zerocool_amd/csrc/engine/records.hpp"
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <unistd.h>
+
+using namespace zerocool::engine;
+static int checks = 0, failures = 0;
+#define CHECK(cond) do { ++checks; if (!(cond)) { ++failures; std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); } } while (0)
+#define CHECK_THROWS(expr) do { ++checks; bool thrown = false; try { (void)(expr); } catch (const std::exception&) { thrown = true; } \
+    if (!thrown) { ++failures; std::printf("  FAILED %s:%d: no exception from %s\n", __FILE__, __LINE__, #expr); } } while (0)
+
+static std::byte value(ExpertKey k, uint64_t i) { return std::byte((k.layer * 131 + k.expert * 31 + i * 7 + (i >> 8)) & 0xff); }
+static void fill(ExpertKey k, std::span<std::byte> into) { for (uint64_t i = 0; i < into.size(); ++i) into[i] = value(k, i); }
+static std::string slurp(const std::filesystem::path& p) { std::ifstream f(p, std::ios::binary); return {std::istreambuf_iterator<char>(f), {}}; }
+static void spit(const std::filesystem::path& p, const std::string& s) { std::ofstream f(p, std::ios::binary | std::ios::trunc); f << s; }
+static std::string replaced(std::string s, const std::string& a, const std::string& b) { const auto at = s.find(a); if (at != std::string::npos) s.replace(at, a.size(), b); return s; }
+
+int main() {
+    const auto root = std::filesystem::temp_directory_path() / ("zc_records_" + std::to_string(::getpid()));
+    std::filesystem::remove_all(root);
+    MoeShape s; s.hidden = 512; s.experts = 8; s.topk = 2; s.inter = 128;
+    const uint64_t bytes = s.expert_bytes();
+
+    std::printf("JSON reader\n");
+    const Json j = Json::parse(R"( {"a": [1, 2.5e2, {"b": "x\nA"}], "t": true, "n": null, "big": 9007199254740991} )");
+    CHECK(j.at("a").size() == 3 && j.at("a").at(0).u64() == 1 && j.at("a").at(1).u64() == 250);
+    CHECK(j.at("a").at(2).at("b").str() == "x\nA" && j.contains("t") && !j.contains("z") && j.at("big").u64() == 9007199254740991ull);
+    CHECK_THROWS(Json::parse("{\"a\": }")); CHECK_THROWS(Json::parse("[1, 2")); CHECK_THROWS(Json::parse("{} x")); CHECK_THROWS(j.at("zz"));
+    CHECK_THROWS(Json::parse("-1").u64()); CHECK_THROWS(Json::parse("1.5").u64());
+
+    std::printf("record layout\n");
+    const auto layout = expert_layout(s);
+    CHECK(layout[0].first == "gate_proj.weight" && layout[0].second == 128ull * 512 / 2 && layout[1].second == 128ull * 8 * 2);
+    CHECK(layout[6].first == "down_proj.weight" && layout[6].second == 512ull * 128 / 2 && layout[8].second == 512ull * 2 * 2);
+    MoeShape ref;   // the reference's own shape: 2,764,800 bytes at stride 2,768,896 (storage.hpp:32-33)
+    CHECK(ref.expert_bytes() == 2764800 && (ref.expert_bytes() + 16383) / 16384 * 16384 == 2768896);
+
+    std::printf("prepared directory: write, read back, reject what the reference rejects\n");
+    const auto dir = root / "prepared";
+    write_prepared_experts(dir, s, 2, fill);
+    {
+        PreparedExperts p(dir, s);
+        CHECK(p.layers() == 2 && p.stride() % 16384 == 0 && p.stride() >= bytes);
+        CHECK(std::filesystem::file_size(dir / "experts-01.bin") == p.stride() * s.experts);
+        std::vector<std::byte> record(bytes);
+        bool same = true;
+        for (uint32_t l = 0; l < 2; ++l) for (uint32_t e = 0; e < s.experts; ++e) {
+            p.expert({l, e}, record);
+            for (uint64_t i = 0; i < bytes; i += 97) same = same && record[i] == value({l, e}, i);
+            same = same && record[bytes - 1] == value({l, e}, bytes - 1);
+        }
+        CHECK(same);
+        const uint64_t stride = (bytes + 255) / 256 * 256;                // the layout of an HBM layer array
+        std::vector<std::byte> whole(stride * s.experts);
+        p.layer(1, whole, stride);
+        CHECK(whole[stride * 5 + 1234] == value({1, 5}, 1234) && whole[stride * 7 + bytes - 1] == value({1, 7}, bytes - 1));
+        CHECK_THROWS(p.expert({2, 0}, record)); CHECK_THROWS(p.expert({0, 8}, record));
+        CHECK_THROWS(p.expert({0, 0}, std::span<std::byte>(record).first(bytes - 1)));
+        CHECK_THROWS(p.layer(0, std::span<std::byte>(whole).first(whole.size() - 300), stride));
+        std::string pad = slurp(dir / "experts-00.bin");                  // the pad after the nine pieces is zero
+        bool zero = true; for (uint64_t i = bytes; i < p.stride(); ++i) zero = zero && pad[i] == 0;
+        CHECK(zero);
+    }
+    MoeShape other = s; other.inter = 256;
+    CHECK_THROWS(PreparedExperts(dir, other));                            // "unsupported prepared expert projection"
+    const std::string manifest = slurp(dir / "manifest.json");
+    spit(dir / "manifest.json", replaced(manifest, "zc-affine-records-v1", "zc-affine-records-v2")); CHECK_THROWS(PreparedExperts(dir, s));
+    spit(dir / "manifest.json", replaced(manifest, "\"alignment\": 16384", "\"alignment\": 4096")); CHECK_THROWS(PreparedExperts(dir, s));
+    spit(dir / "manifest.json", replaced(manifest, "experts-01.bin", "experts-00.bin")); CHECK_THROWS(PreparedExperts(dir, s));   // duplicate range
+    spit(dir / "manifest.json", replaced(manifest, "experts-01.bin", "../experts-01.bin")); CHECK_THROWS(PreparedExperts(dir, s));
+    spit(dir / "manifest.json", replaced(manifest, "\"group_size\": 64", "\"group_size\": 32")); CHECK_THROWS(PreparedExperts(dir, s));
+    spit(dir / "manifest.json", manifest);
+    std::filesystem::resize_file(dir / "experts-01.bin", std::filesystem::file_size(dir / "experts-01.bin") - 1); CHECK_THROWS(PreparedExperts(dir, s));
+    std::filesystem::remove(dir / "experts-01.bin"); CHECK_THROWS(PreparedExperts(dir, s));
+    CHECK_THROWS(PreparedExperts(root / "nowhere", s));
+
+    std::printf("safetensors checkpoint: nine stacked tensors per layer gathered into records\n");
+    const auto ckpt = root / "checkpoint"; std::filesystem::create_directories(ckpt);
+    {
+        // layer 0 in one file, layer 1 in another; tensor data = for each piece, the experts' slices back to back
+        for (uint32_t l = 0; l < 2; ++l) {
+            std::string header = "{\"__metadata__\": {\"format\": \"pt\"}", data; uint64_t at = 0, piece_at = 0;
+            for (int p = 0; p < 9; ++p) {
+                const uint64_t rows = p < 6 ? s.inter : s.hidden, cols = p < 6 ? s.hidden : s.inter, len = layout[p].second;
+                header += ", \"model.layers." + std::to_string(l) + ".mlp.switch_mlp." + layout[p].first + "\": {\"dtype\": \"" + (p % 3 == 0 ? "U32" : "BF16") +
+                          "\", \"shape\": [" + std::to_string(s.experts) + ", " + std::to_string(rows) + ", " + std::to_string(p % 3 == 0 ? cols / 8 : cols / 64) +
+                          "], \"data_offsets\": [" + std::to_string(at) + ", " + std::to_string(at + len * s.experts) + "]}";
+                for (uint32_t e = 0; e < s.experts; ++e) for (uint64_t i = 0; i < len; ++i) data += char(value({l, e}, piece_at + i));
+                at += len * s.experts; piece_at += len;
+            }
+            header += "}";
+            const uint64_t n = header.size(); std::string file(8, '\0'); std::memcpy(file.data(), &n, 8);
+            spit(ckpt / ("model-0000" + std::to_string(l + 1) + ".safetensors"), file + header + data);
+        }
+        SafetensorsExperts c(ckpt, s, 2);
+        std::vector<std::byte> record(bytes); bool same = true;
+        for (uint32_t l = 0; l < 2; ++l) for (uint32_t e = 0; e < s.experts; e += 3) {
+            c.expert({l, e}, record);
+            for (uint64_t i = 0; i < bytes; i += 61) same = same && record[i] == value({l, e}, i);
+        }
+        CHECK(same);                                                      // byte-identical to the prepared record of the same expert
+        CHECK_THROWS(c.expert({2, 0}, record));
+        CHECK_THROWS(SafetensorsExperts(ckpt, s, 3));                     // layer 2 is not there
+        CHECK_THROWS(SafetensorsExperts(ckpt, other, 2));                 // shapes differ
+    }
+    std::filesystem::remove_all(root);
+    std::printf("%d checks, %d failures\n", checks, failures);
+    return failures ? 1 : 0;
+}

@@ -267,6 +267,29 @@ static void test_expert_cache() {   // :336-348 on the GPU, and moe() reading it
     const auto st = cache.stats();
     CHECK(st.misses >= s.topk); CHECK(st.hits + st.misses >= 6 * s.topk); CHECK(st.bytes == st.misses * s.expert_bytes());
     cache.clear(); CHECK(cache.occupancy() == 0);
+    // next-layer prediction (model.cpp:437-445, 489-500): here the "next layer" has this layer's router and sees the
+    // same input, so every guess is exactly what the following call demands: all of them were prefetched and none misses
+    w.next_router = w.router; w.prefetch_depth = s.topk;
+    w.prefetch = [&](uint32_t e) { return cache.prefetch({0, e}); };
+    {
+        auto x = gpu.zeros(s.hidden);
+        for (size_t i = 0; i < x->floats().size(); ++i) x->floats()[i] = round_bf16(float(int((i * 2654435761u >> 7) % 255) - 127) / 64);
+        const auto before = cache.stats();
+        PredictionStats guess;
+        auto first = moe(gpu, w, x, 1, nullptr, 128, x, &guess); gpu.finish(); held.clear();
+        CHECK(guess.guesses == s.topk && guess.experts.size() == s.topk);
+        const auto mid = cache.stats();
+        CHECK(mid.prefetches - before.prefetches == guess.issued);        // already-resident guesses are not issued again
+        auto second = moe(gpu, w, x, 1); gpu.finish(); held.clear();      // demands exactly the guessed experts
+        const auto after = cache.stats();
+        CHECK(after.misses == mid.misses);
+        CHECK(std::memcmp(first->data, second->data, first->bytes) == 0);  // the hint never changes the arithmetic
+        auto plain = moe_resident(gpu, w, records, stride, x, 1);
+        CHECK(std::memcmp(first->data, plain->data, first->bytes) == 0);
+        w.prefetch_depth = 3; PredictionStats shallow; cache.clear();
+        moe(gpu, w, x, 1, nullptr, 128, x, &shallow); gpu.finish(); held.clear();
+        CHECK(shallow.guesses == s.topk && shallow.issued <= 3);
+    }
 }
 static void test_glue() {   // :53, :876-897, :1137-1145 and the glue of model.cpp:328-351, 651
     TEST("element-wise dispatches, the stream mix / injection and the grouped norm");

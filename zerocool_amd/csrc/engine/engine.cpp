@@ -262,13 +262,30 @@ void encode_expert_rows(Metal& gpu, const Buf& record, const Buf& input, const B
 }
 
 // model.cpp:431-557 without the cache, prefetch, trace and timing branches
-Buf moe(Metal& gpu, const MoeLayerWeights& w, const Buf& x, uint32_t tokens, const std::atomic<bool>* cancel, uint32_t chunk) {
+Buf moe(Metal& gpu, const MoeLayerWeights& w, const Buf& x, uint32_t tokens, const std::atomic<bool>* cancel, uint32_t chunk,
+        const Buf& predict, PredictionStats* prediction) {
     const auto& s = gpu.shape();
     auto cancelled = [&] { if (cancel && cancel->load()) throw std::runtime_error("generation cancelled"); };
     auto router = gpu.linear(w.router, x, tokens, true);
     auto ids = gpu.allocate(uint64_t(tokens) * s.topk * 4), weights = gpu.allocate(uint64_t(tokens) * s.topk * 4);
     gpu.route(router, ids, weights, tokens);
+    Buf predicted;
+    if (predict && w.next_router.weight.buffer) {   // model.cpp:437-445: shares this readback, never feeds the arithmetic
+        if (predict->bytes < uint64_t(tokens) * s.hidden * 4) throw std::invalid_argument("invalid prediction input");
+        auto logits = gpu.linear(w.next_router, predict, tokens, true);
+        predicted = gpu.allocate(uint64_t(tokens) * s.topk * 4);
+        gpu.route(logits, predicted, gpu.allocate(uint64_t(tokens) * s.topk * 4), tokens);
+    }
     gpu.finish(); cancelled();
+    if (predicted) {                                // model.cpp:489-500: the first token's guesses, distinct, depth-limited
+        PredictionStats local; PredictionStats& st = prediction ? *prediction : local; st = {};
+        const auto guesses = std::span<const int>(reinterpret_cast<const int*>(predicted->data), s.topk);
+        for (int e : guesses)
+            if (e >= 0 && e < int(s.experts) && std::find(st.experts.begin(), st.experts.end(), e) == st.experts.end()) {
+                const bool issued = st.experts.size() < w.prefetch_depth && w.prefetch && w.prefetch(uint32_t(e));
+                st.experts.push_back(e); ++st.guesses; st.issued += issued;
+            }
+    }
     std::vector<std::vector<int>> positions(s.experts);
     auto raw = std::span<const int>(reinterpret_cast<const int*>(ids->data), size_t(tokens) * s.topk);
     for (uint32_t p = 0; p < tokens * s.topk; ++p) {

@@ -30,6 +30,17 @@
  *   route softmax WEIGHT BITS and the final simd_sum association of the affine
  *   dots: parity unpinned at bit level (only an Apple GPU run could pin them);
  *   sum-to-one and tolerance checks only.
+ *
+ * The callers' glue either side of the layer (tests/test_oracle_glue.py):
+ *   softplus, unary   64-point captured softplus table, exact (…:881); ops 2 and 3
+ *                     as compositions of the pinned SiLU / sigmoid
+ *   log in softplus   correctly rounded fp32 logarithm on a 1001-point grid
+ *   binary, hc_mix,   explicit loops with a BF16 rounding after every operation
+ *   hc_add
+ *   norm              double precision within two BF16 roundings, closed forms, and
+ *                     a row whose block sums depend on the order of additions;
+ *                     precise::rsqrt (taken as 1/sqrt) and the lane-sum association:
+ *                     parity unpinned (the reference tests norm only against norm_wide)
  */
 #ifndef ZC_ORACLE_H
 #define ZC_ORACLE_H

@@ -2,7 +2,7 @@
 // (tests/test_qwen.cpp, cited per case): build tiny deterministic inputs through the Buffer
 // interface, run the operators, compare bytes.  The CPU oracle (oracle/zc_oracle.h) is the checker.
 #include "../../zerocool_amd/csrc/engine/engine.hpp"
-#include "../../zerocool_amd/csrc/engine/records.hpp"
+#include "../../zerocool_amd/csrc/engine/route_trace.hpp"
 #include <unistd.h>
 #include "../../oracle/zc_oracle.h"
 #include <algorithm>
@@ -336,8 +336,31 @@ static void test_glue() {   // :53, :876-897, :1137-1145 and the glue of model.c
     CHECK_THROWS(gpu.dispatch("norm", {{x}, {x}, {y}}, {48, 100, 1, 0, 1}, 32));
 }
 
+static void test_route_replay() {   // model.cpp:274-283, 447-448: dumped logits replayed against dumped ids
+    TEST("route dumps of another machine replay through route()");
+    Metal gpu; const auto& s = gpu.shape(); const uint32_t T = 5;
+    std::vector<float> logits(size_t(T) * s.experts); std::vector<int> want(size_t(T) * s.topk);
+    for (uint32_t t = 0; t < T; ++t) {
+        for (uint32_t e = 0; e < s.experts; ++e) logits[size_t(t) * s.experts + e] = float(int((e * 37u + t * 101u) % 199) - 99) / 8;   // many exact ties
+        std::vector<int> order(s.experts); std::iota(order.begin(), order.end(), 0);
+        std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return logits[size_t(t) * s.experts + a] > logits[size_t(t) * s.experts + b]; });
+        std::copy(order.begin(), order.begin() + s.topk, want.begin() + size_t(t) * s.topk);
+    }
+    const auto dir = std::filesystem::temp_directory_path() / ("zc_engine_dump_" + std::to_string(::getpid()));
+    write_tensor_dump(dir, 40, "router_3", std::as_bytes(std::span(logits)));
+    write_tensor_dump(dir, 40, "route_3", std::as_bytes(std::span(want)));
+    CHECK(replay_route_dump(gpu, dir, 40, 3) == 0);
+    std::swap(want[0], want[1]);
+    write_tensor_dump(dir, 40, "route_3", std::as_bytes(std::span(want)));
+    CHECK(replay_route_dump(gpu, dir, 40, 3) == 2);
+    CHECK_THROWS(replay_route_dump(gpu, dir, 40, 4)); CHECK_THROWS(replay_route_dump(gpu, dir, 41, 3));
+    write_tensor_dump(dir, 40, "route_3", std::as_bytes(std::span(want).first(7)));
+    CHECK_THROWS(replay_route_dump(gpu, dir, 40, 3));
+    std::filesystem::remove_all(dir);
+}
+
 int main() {
-    test_glue(); test_bf16(); test_q4_matmul(); test_route(); test_moe_sum(); test_direct_rows(); test_grouped(); test_heavy_rows(); test_moe_layer(); test_expert_cache();
+    test_route_replay(); test_glue(); test_bf16(); test_q4_matmul(); test_route(); test_moe_sum(); test_direct_rows(); test_grouped(); test_heavy_rows(); test_moe_layer(); test_expert_cache();
     std::printf("%d checks, %d failures\n", checks, failures);
     return failures ? 1 : 0;
 }

@@ -1,6 +1,6 @@
 // Tests of the on-disk expert record readers (zerocool_amd/csrc/engine/records.hpp); no GPU needed.
 // Follows the checks of the reference's PreparedArtifact / ExpertStore (src/engine/storage.cpp:316-394, 493-516).
-#include "../../zerocool_amd/csrc/engine/records.hpp"
+#include "../../zerocool_amd/csrc/engine/route_trace.hpp"
 #include <cstdio>
 #include <cstring>
 #include <fstream>
@@ -105,6 +105,41 @@ int main() {
         CHECK_THROWS(c.expert({2, 0}, record));
         CHECK_THROWS(SafetensorsExperts(ckpt, s, 3));                     // layer 2 is not there
         CHECK_THROWS(SafetensorsExperts(ckpt, other, 2));                 // shapes differ
+    }
+    std::printf("route trace: the reference's call-order rules, and a round trip through the reader\n");
+    {
+        const auto path = root / "routes.jsonl";
+        const uint32_t L = 3, K = 2;
+        {
+            RouteTrace t(path, "{\"model\": \"test\", \"layers\": 3}", L, K);
+            CHECK_THROWS(RouteTrace(path, "{}", L, K));                    // must be a new file
+            const int prompt[3] = {5, 6, 7}, one[1] = {9};
+            CHECK_THROWS(t.begin(1, 0, prompt, "prefill", 16));            // no request yet
+            t.request_begin("a \"quoted\" name", prompt, 4, false);
+            CHECK_THROWS(t.request_begin("again", prompt, 4, false));
+            t.begin(77, 0, prompt, "prefill", 16);
+            const int r0[6] = {1, 2, 3, 4, 5, 6}, r1[6] = {6, 5, 4, 3, 2, 1}, r2[6] = {0, 1, 0, 1, 0, 1};
+            CHECK_THROWS(t.routes(1, 0, 3, r0));                           // layers in order
+            CHECK_THROWS(t.routes(0, 0, 3, std::span<const int>(r0, 5)));  // tokens * topk ids
+            t.routes(0, 0, 3, r0); t.routes(1, 0, 3, r1);
+            CHECK_THROWS(t.commit(3));                                     // a layer is missing
+            t.routes(2, 0, 3, r2); CHECK_THROWS(t.commit(4)); t.commit(3);
+            t.begin(77, 3, one, "decode", 16); const int d[2] = {7, 8}; t.routes(0, 3, 1, d); t.abort();
+            CHECK_THROWS(t.finish());                                      // the request is still open
+            t.request_end(one, "stop", 0); t.cache_reset(); t.finish();
+        }
+        const TraceSummary sum = read_route_trace(path);
+        CHECK(sum.complete && sum.events == 13 && sum.forwards.size() == 2);
+        CHECK(sum.forwards[0].committed && sum.forwards[0].tokens == 3 && sum.forwards[0].phase == "prefill" && sum.forwards[0].routes.size() == 3);
+        CHECK(sum.forwards[0].routes[1] == (std::vector<int>{6, 5, 4, 3, 2, 1}) && !sum.forwards[1].committed && sum.forwards[1].routes.size() == 1);
+        spit(root / "broken.jsonl", replaced(slurp(path), "\"sequence\":3", "\"sequence\":4")); CHECK_THROWS(read_route_trace(root / "broken.jsonl"));
+        { RouteTrace open_ended(root / "open.jsonl", "{}", L, K); }
+        CHECK(!read_route_trace(root / "open.jsonl").complete);           // closed without finish(): "incomplete"
+        const float logits[4] = {1, 2, 3, 4};
+        write_tensor_dump(root / "dump", 12, "router_0", std::as_bytes(std::span(logits)));
+        const auto back = read_tensor_dump(root / "dump", 12, "router_0");
+        CHECK(back.size() == 16 && std::memcmp(back.data(), logits, 16) == 0 && std::filesystem::exists(root / "dump" / "step_12" / "router_0.bin"));
+        CHECK_THROWS(read_tensor_dump(root / "dump", 12, "route_0"));
     }
     std::filesystem::remove_all(root);
     std::printf("%d checks, %d failures\n", checks, failures);

@@ -225,6 +225,20 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         clock();
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
+        // One token: the wave's first router unit starts loading its weights now, so that their latency passes while the
+        // input row is staged and its image built (the weights do not depend on the input).
+        const uint32_t first_unit = wg + nwg * wave;
+        uint4 early[kRing];
+#pragma unroll
+        for (int i = 0; i < kRing; ++i) early[i] = make_uint4(0, 0, 0, 0);
+        if constexpr (NT == 1) {
+            if (first_unit < (E + 3) / 4) {
+                const uint32_t e = first_unit * 4 + lane / 16, split = lane % 16, P = H / 16;
+                const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
+#pragma unroll
+                for (int i = 0; i < kRing; ++i) if (uint32_t(i) < P / 8) early[i] = ldg_u4(wr, i);
+            }
+        }
         {
             uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
             const bool glue = layer != 0;
@@ -270,27 +284,35 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
         clock();
         {
-            const uint32_t router_units = (E + 3) / 4, shared_units = I / 8, gate_units = (T + 1) / 2;
+            // One token: the shared gate/up tiles do not wait for the routing, so they run beside it in phase G on the
+            // waves that would otherwise idle while wave 0 picks the experts; this phase then only has the router.
+            const uint32_t router_units = (E + 3) / 4, shared_units = NT == 1 ? 0 : I / 8, gate_units = (T + 1) / 2;
             const uint32_t units = router_units + shared_units + gate_units;
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
                 if (u < router_units) {
                     // four experts x sixteen K partitions; k-ascending fused chain per partition
                     const uint32_t e = u * 4 + lane / 16, split = lane % 16, P = H / 16;
                     const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
+                    constexpr int kRouterRing = kRing;
                     const uint32_t pieces = P / 8;   // sixteen-byte pieces of the partition, kRing in flight
-                    uint4 wv[kRing];
+                    uint4 wv[kRouterRing];
+                    if (NT == 1 && u == first_unit) {
 #pragma unroll
-                    for (int i = 0; i < kRing; ++i) if (uint32_t(i) < pieces) wv[i] = ldg_u4(wr, i);
+                        for (int i = 0; i < kRouterRing; ++i) wv[i] = early[i];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < kRouterRing; ++i) if (uint32_t(i) < pieces) wv[i] = ldg_u4(wr, i);
+                    }
                     float c[NT];
 #pragma unroll
                     for (int t = 0; t < NT; ++t) c[t] = 0;
-                    for (uint32_t i0 = 0; i0 < pieces; i0 += kRing) {
+                    for (uint32_t i0 = 0; i0 < pieces; i0 += kRouterRing) {
 #pragma unroll
-                        for (int j = 0; j < kRing; ++j) {
+                        for (int j = 0; j < kRouterRing; ++j) {
                             const uint32_t i = i0 + j;
                             if (i < pieces) {
                                 const uint32_t ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
-                                if (i + kRing < pieces) wv[j] = ldg_u4(wr, i + kRing);
+                                if (i + kRouterRing < pieces) wv[j] = ldg_u4(wr, i + kRouterRing);
 #pragma unroll
                                 for (int t = 0; t < NT; ++t) {
                                     if (t >= int(T)) break;
@@ -337,7 +359,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     const uint16_t* gw = reinterpret_cast<const uint16_t*>(lds + lp.gatew);   // staged with the input rows
                     float sum = 0;
                     if (t < T)
-                        for (uint32_t kk = l32; kk < H; kk += 32) sum += b16(xh_all[t * H + kk]) * b16(gw[kk]);
+                        for (uint32_t k0 = l32; k0 < H; k0 += 256) {   // eight LDS reads in flight per operand (hidden is a multiple of 512); the sum stays in k order
+                            float a[8], g[8];
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) { a[j] = b16(xh_all[t * H + k0 + 32 * j]); g[j] = b16(gw[k0 + 32 * j]); }
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) sum += a[j] * g[j];
+                        }
                     sum = lane_sum32(sum);
                     if (t < T && l32 == 0) st_f32(p.gate + t, bf(sum));
                 }
@@ -348,6 +376,19 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         refresh();
         clock();
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
+        if constexpr (NT == 1) {
+            if (wave >= 1)
+                for (uint32_t tile = wg + nwg * (wave - 1); tile < I / 8; tile += nwg * (kDecodeWaves - 1)) {
+                    const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                    const uint8_t* rec = L.shared_record;
+                    const uint8_t* w_row = rec + p.so[pr] + uint64_t(row) * (H / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64);
+                    const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
+                    auto emit = [&](int, float v) { store_act(p.shared_act, 0, row, v); };
+                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
+                }
+        }
         for (uint32_t t = wave; t < T; t += kDecodeWaves)
         {
             auto stamp = [&]() { if (t == 0) clock(); };

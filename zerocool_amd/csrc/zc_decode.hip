@@ -225,63 +225,100 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         clock();
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
-        // One token: the wave's first router unit starts loading its weights now, so that their latency passes while the
-        // input row is staged and its image built (the weights do not depend on the input).
+        // One token: the wave's first router unit starts loading its weights while the input row is staged and its image
+        // built (the weights do not depend on the input).
         const uint32_t first_unit = wg + nwg * wave;
         uint4 early[kRing];
 #pragma unroll
         for (int i = 0; i < kRing; ++i) early[i] = make_uint4(0, 0, 0, 0);
         if constexpr (NT == 1) {
-            if (first_unit < (E + 3) / 4) {
+            // One token: thread b fetches the sixteen fp32 values of block b, applies the glue's scale, writes the BF16 copy and
+            // builds the block's image pieces straight from registers; the shared gate row and the scale ride along.
+            uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
+            const bool glue = layer != 0;
+            const float* row = glue ? p.layer_out : p.x_in;
+            const uint32_t peak = glue ? ZC_LD(p.maxabs + (layer - 1) * T) : 0u;
+            uint64_t v[8];
+#pragma unroll
+            for (int w = 0; w < 8; ++w) v[w] = 0;
+            if (tid < H / 16) {
+#pragma unroll
+                for (int w = 0; w < 8; ++w) v[w] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(row) + tid * 8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            uint4 gate_piece = make_uint4(0, 0, 0, 0);
+            if (tid < H / 8) gate_piece = ldg_u4(L.shared_gate, tid);
+            if (first_unit < (E + 3) / 4) {   // issued after the input's loads: waiting for those does not wait for these
                 const uint32_t e = first_unit * 4 + lane / 16, split = lane % 16, P = H / 16;
                 const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
 #pragma unroll
                 for (int i = 0; i < kRing; ++i) if (uint32_t(i) < P / 8) early[i] = ldg_u4(wr, i);
             }
-        }
-        {
-            uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
-            const bool glue = layer != 0;
-            // the glue's scale per token, 1 / max|y| of the previous layer: one token fetches it together with the row,
-            // several tokens go through LDS (one more round trip, fewer registers)
-            uint32_t peak = 0; float inv = 1.0f;
-            if constexpr (NT == 1) {
-                if (glue) peak = ZC_LD(p.maxabs + (layer - 1) * T);
-            } else {
-                if (glue && tid < T) {
-                    const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
-                    gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+            xint_prepare_begin(LH, lds + lp.img_rg, 1);
+            __syncthreads();
+            if (tid < H / 16) {
+                const float m = __uint_as_float(peak), inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+                RegF32 block; uint32_t low = 0, packed[8];
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    float a = __uint_as_float(uint32_t(v[w])), c = __uint_as_float(uint32_t(v[w] >> 32));
+                    if (glue) { a = bf(a * inv); c = bf(c * inv); }
+                    const uint32_t ua = __float_as_uint(a), uc = __float_as_uint(c);
+                    low |= (ua | uc) & 0xffffu;
+                    block.bits[2 * w] = ua & 0xffff0000u; block.bits[2 * w + 1] = uc & 0xffff0000u;
+                    packed[w] = (ua >> 16) | (uc & 0xffff0000u);
                 }
-                __syncthreads();
+                if (low) atomicOr(p.status, 4);   // inputs must be BF16-valued
+                uint4* copy = reinterpret_cast<uint4*>(xh + tid * 16);
+                copy[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]); copy[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
+                xint_prepare_block(block, LH, lds + lp.img_rg, tid);
             }
-            // the shared-expert gate row rides along: coalesced sixteen-byte loads, used from LDS by the gate-dot waves
-            constexpr int kGatePieces = (3072 / 8 + kDecodeThreads - 1) / kDecodeThreads;   // hidden <= 3072
-            uint4 gate_piece[kGatePieces];
-#pragma unroll
-            for (int q = 0; q < kGatePieces; ++q) gate_piece[q] = make_uint4(0, 0, 0, 0);
-            const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh),
-                [&]() {
-                    if constexpr (NT == 1) {
-#pragma unroll
-                        for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
-                        const float m = __uint_as_float(peak); inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+            if (tid < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid] = gate_piece;
+            __syncthreads();
+        } else {
+            {
+                uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
+                const bool glue = layer != 0;
+                // the glue's scale per token, 1 / max|y| of the previous layer: one token fetches it together with the row,
+                // several tokens go through LDS (one more round trip, fewer registers)
+                uint32_t peak = 0; float inv = 1.0f;
+                if constexpr (NT == 1) {
+                    if (glue) peak = ZC_LD(p.maxabs + (layer - 1) * T);
+                } else {
+                    if (glue && tid < T) {
+                        const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
+                        gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
                     }
-                },
-                [&](uint32_t i, float& a, float& b) {
-                    if (glue) {
-                        const float scale = NT == 1 ? inv : gatev[(2 * i) / H];
-                        a = bf(a * scale); b = bf(b * scale);
-                    }
-                });
-            if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
+                    __syncthreads();
+                }
+                // the shared-expert gate row rides along: coalesced sixteen-byte loads, used from LDS by the gate-dot waves
+                constexpr int kGatePieces = (3072 / 8 + kDecodeThreads - 1) / kDecodeThreads;   // hidden <= 3072
+                uint4 gate_piece[kGatePieces];
 #pragma unroll
-            for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) {
-                if constexpr (NT != 1) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);   // several tokens: after the rows, to spare registers
-                reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
+                for (int q = 0; q < kGatePieces; ++q) gate_piece[q] = make_uint4(0, 0, 0, 0);
+                const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh),
+                    [&]() {
+                        if constexpr (NT == 1) {
+#pragma unroll
+                            for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
+                            const float m = __uint_as_float(peak); inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+                        }
+                    },
+                    [&](uint32_t i, float& a, float& b) {
+                        if (glue) {
+                            const float scale = NT == 1 ? inv : gatev[(2 * i) / H];
+                            a = bf(a * scale); b = bf(b * scale);
+                        }
+                    });
+                if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
+#pragma unroll
+                for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) {
+                    if constexpr (NT != 1) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);   // several tokens: after the rows, to spare registers
+                    reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
+                }
             }
+            __syncthreads();
+            xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
         }
-        __syncthreads();
-        xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
         clock();
         {
             // One token: the shared gate/up tiles do not wait for the routing, so they run beside it in phase G on the
@@ -462,17 +499,54 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 const uint32_t sn = min(SB, slots_total - s0);
                 __syncthreads();
                 uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
-                {   // rows s0 .. s0+sn-1 of [act ; shared_act]: contiguous except across the seam between the two buffers
-                    const uint32_t routed = s0 < n ? min(sn, n - s0) : 0;
-                    if (routed) stage_copy<NT == 1 ? 12 : 6>(reinterpret_cast<const uint64_t*>(p.act) + uint64_t(s0) * I / 4, routed * I / 4, reinterpret_cast<uint64_t*>(ah));
-                    if (sn > routed) stage_copy<NT == 1 ? 12 : 6>(reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(s0 + routed - n) * I / 4, (sn - routed) * I / 4,
-                                                reinterpret_cast<uint64_t*>(ah + routed * I));
-                }
-                __syncthreads();
                 auto source_of = [&](uint32_t q) { return LdsBf16{ah + q * I}; };
-                if (s0 == 0) clock();
-                xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
-                if (s0 == 0) clock();
+                if constexpr (NT == 1) {
+                    // One token: a thread fetches whole 16-element blocks of the activations (32 bytes) and builds their
+                    // image pieces straight from registers; the BF16 copy for the literal chain is written on the way.
+                    const uint32_t per = I / 16, total = sn * per;
+                    constexpr int kMine = 2;
+                    for (uint32_t base = 0; base < total; base += kDecodeThreads * kMine) {
+                        RegBf16 piece[kMine];
+#pragma unroll
+                        for (int j = 0; j < kMine; ++j) {
+                            const uint32_t blk = base + j * kDecodeThreads + tid;
+#pragma unroll
+                            for (int w = 0; w < 4; ++w) piece[j].w[w] = 0;
+                            if (blk < total) {
+                                const uint32_t slot = s0 + blk / per, b = blk % per;
+                                const uint64_t* src = (slot < n ? reinterpret_cast<const uint64_t*>(p.act) + uint64_t(slot) * I / 4
+                                                                : reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(slot - n) * I / 4) + b * 4;
+#pragma unroll
+                                for (int w = 0; w < 4; ++w) piece[j].w[w] = __hip_atomic_load(src + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+                        }
+                        if (base == 0) { xint_prepare_begin(LI, lds + lp.img_d, sn); __syncthreads(); }   // while the loads are in flight
+#pragma unroll
+                        for (int j = 0; j < kMine; ++j) {
+                            const uint32_t blk = base + j * kDecodeThreads + tid;
+                            if (blk < total) {
+                                const uint32_t q = blk / per, b = blk % per;
+                                uint64_t* copy = reinterpret_cast<uint64_t*>(ah + q * I + b * 16);
+#pragma unroll
+                                for (int w = 0; w < 4; ++w) copy[w] = piece[j].w[w];
+                                xint_prepare_block(piece[j], LI, lds + lp.img_d + q * LI.bytes(), b);
+                            }
+                        }
+                    }
+                    if (s0 == 0) { clock(); clock(); }
+                    __syncthreads();
+                } else {
+                    {   // rows s0 .. s0+sn-1 of [act ; shared_act]: contiguous except across the seam between the two buffers
+                        const uint32_t routed = s0 < n ? min(sn, n - s0) : 0;
+                        if (routed) stage_copy<6>(reinterpret_cast<const uint64_t*>(p.act) + uint64_t(s0) * I / 4, routed * I / 4, reinterpret_cast<uint64_t*>(ah));
+                        if (sn > routed) stage_copy<6>(reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(s0 + routed - n) * I / 4, (sn - routed) * I / 4,
+                                                       reinterpret_cast<uint64_t*>(ah + routed * I));
+                    }
+                    __syncthreads();
+                    if (s0 == 0) clock();
+                    xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
+                    if (s0 == 0) clock();
+                }
                 for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
                     const uint8_t* rec; const uint64_t* off; int32_t s;
                     if (u < U) { const uint32_t e = uint32_t(uniform(experts[u])); s = uniform(head[e]); rec = L.records + uint64_t(e) * L.stride; off = p.ro; }

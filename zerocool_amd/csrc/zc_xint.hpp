@@ -60,6 +60,25 @@ struct LdsBf16 {     // BF16 copy of a BF16-valued row
         for (int i = 0; i < 8; ++i) { out[2 * i] = w[i] << 16; out[2 * i + 1] = w[i] & 0xffff0000u; }
     }
 };
+struct RegBf16 {     // one block of sixteen BF16 values held in registers (block index ignored)
+    static constexpr bool kExactProducts = true;
+    uint64_t w[4];
+    __device__ __forceinline__ void block(uint32_t, uint32_t* out) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t lo = uint32_t(w[i]), hi = uint32_t(w[i] >> 32);
+            out[4 * i] = lo << 16; out[4 * i + 1] = lo & 0xffff0000u; out[4 * i + 2] = hi << 16; out[4 * i + 3] = hi & 0xffff0000u;
+        }
+    }
+};
+struct RegF32 {      // one block of sixteen BF16-valued fp32 bit patterns held in registers (block index ignored)
+    static constexpr bool kExactProducts = true;
+    uint32_t bits[16];
+    __device__ __forceinline__ void block(uint32_t, uint32_t* out) const {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) out[i] = bits[i];
+    }
+};
 struct LdsF32 {      // fp32 copy of an arbitrary row
     static constexpr bool kExactProducts = false;
     const float* x;

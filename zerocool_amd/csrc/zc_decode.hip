@@ -36,10 +36,10 @@ constexpr uint32_t kFlagStride = 32, kReleaseBase = 32 * 1024, kReleaseStride = 
 
 struct Barrier {
     uint32_t* mem; uint32_t epoch, spin_limit; int32_t* status; uint32_t token;   // token: this launch's first epoch
-    // Flags + collector: every workgroup stores its epoch; workgroup 0 polls all flags
-    // (one per thread) and then stores eight release words.  No cache write-back or
-    // invalidate: the data that crosses is written with write-through atomics, read with
-    // coherent loads, and each wave has drained its own stores before the flag is stored.
+    // Flags: every workgroup stores its epoch in its own 128-byte line and polls the lines of
+    // all others.  No cache write-back or invalidate: the data that crosses is written with
+    // write-through atomics, read with coherent loads, and each wave has drained its own stores
+    // before the flag is stored.
     __device__ __forceinline__ void wait() {
         ++epoch;
         // Every wave waits until its own write-through stores have been acknowledged by the L2 (the point of
@@ -51,15 +51,10 @@ struct Barrier {
         uint32_t me = blockIdx.x, thread = threadIdx.x;
         asm volatile("" : "+s"(me));       // flag addresses are formed here, not kept in registers across the phases
         asm volatile("" : "+v"(thread));
-        if (me == 0) {
-            for (uint32_t w = thread; w < gridDim.x; w += blockDim.x)
-                if (w) spin(mem + kFlagStride * w);
-            __syncthreads();
-            if (thread < 8) ZC_ST(mem + kReleaseBase + kReleaseStride * thread, epoch);
-        } else if (thread == 0) {
-            ZC_ST(mem + kFlagStride * me, epoch);
-            spin(mem + kReleaseBase + kReleaseStride * (me & 7u));
-        }
+        // every workgroup watches every flag itself (one flag per thread): one store-to-load hop instead of a collector's two
+        if (thread == 0) ZC_ST(mem + kFlagStride * me, epoch);
+        for (uint32_t w = thread; w < gridDim.x; w += blockDim.x)
+            if (w != me) spin(mem + kFlagStride * w);
         __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }

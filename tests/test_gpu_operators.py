@@ -137,7 +137,10 @@ def test_router_captured_words_and_chunks(ctx):  # :798-826
         assert same_bytes(part, full.reshape(T, N)[offset:offset + count])
 
 
-@pytest.mark.parametrize("H,E,T", [(2048, 512, 1), (2048, 512, 9), (3072, 512, 8), (512, 32, 5)])
+# the last four reach the long-batch kernels: register-tiled (T >= 64) and LDS-staged (T >= 256, K % 512 == 0), with token and
+# expert counts that do not fill the last tile
+@pytest.mark.parametrize("H,E,T", [(2048, 512, 1), (2048, 512, 9), (3072, 512, 8), (512, 32, 5),
+                                    (640, 40, 70), (2048, 512, 300), (512, 40, 257), (1024, 24, 1030)])
 def test_router_random_with_offsets(ctx, H, E, T):
     w = synth.bf_bits(synth.normal(E * H, 3, 1 / math.sqrt(H))); x = synth.normal(T * H, 4)
     off = synth.normal_offsets(E, 5)

@@ -174,6 +174,10 @@ def test_dispatch_matches_counting_sort(ctx, T, E, k):  # model.cpp:449-479
     assert same_bytes(off.numpy(np.int32), o_off) and same_bytes(slots.numpy(np.int32), o_slots)
     n = int(count.numpy(np.int32)[0])
     assert n == len(o_sel) and same_bytes(sel.numpy(np.int32)[:n], o_sel) and status.numpy(np.int32)[0] == 0
+    if T * k > 1024:   # an id array that is only four-byte aligned (the long-batch kernels read sixteen bytes at a time when they can)
+        shifted = ctx.upload(np.concatenate([np.zeros(1, np.int32), ids.reshape(-1)])).view(4)
+        off2, slots2, _, _, _ = ctx.build_dispatch(shifted, T, k, E)
+        assert same_bytes(off2.numpy(np.int32), o_off) and same_bytes(slots2.numpy(np.int32), o_slots)
     ids[T // 2, k - 1] = -1
     assert ctx.build_dispatch(ctx.upload(ids), T, k, E)[4].numpy(np.int32)[0] != 0
     ids[T // 2, k - 1] = E

@@ -506,7 +506,7 @@ __global__ __launch_bounds__(1024) void dispatch_kernel(const int32_t* ids, uint
 }
 // The same sort for many slots (prefill), spread over the device: one wavefront per expert counts, one workgroup
 // scans, one wavefront per expert places.  offsets[1 + e] doubles as the count array between the first two steps.
-__global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* ids, uint32_t n, uint32_t E, int32_t* offsets, int32_t* status) {
+__global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* ids, uint32_t n, uint32_t E, int32_t* offsets, int32_t* status, bool aligned) {
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (blockIdx.x == 0) {
         int bad = 0;
@@ -515,10 +515,15 @@ __global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* ids,
     }
     if (e >= E) return;
     int32_t c = 0;
-    for (uint32_t p0 = 0; p0 < n; p0 += 64) {
-        const uint32_t p = p0 + lane;
-        c += __popcll(__ballot(p < n && ids[p] == int32_t(e)));
+    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // a lane looks at four neighbouring slots per step
+        const uint32_t p = p0 + 4 * lane;
+        int4 v = make_int4(-1, -1, -1, -1);
+        if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array
+        else { if (p < n) v.x = ids[p]; if (p + 1 < n) v.y = ids[p + 1]; if (p + 2 < n) v.z = ids[p + 2]; if (p + 3 < n) v.w = ids[p + 3]; }
+        c += (v.x == int32_t(e)) + (v.y == int32_t(e)) + (v.z == int32_t(e)) + (v.w == int32_t(e));
     }
+#pragma unroll
+    for (int o = 32; o; o >>= 1) c += __shfl_xor(c, o);
     if (lane == 0) offsets[1 + e] = c;
 }
 __global__ __launch_bounds__(64) void dispatch_scan_kernel(uint32_t E, int32_t* offsets, int32_t* selected, int32_t* count) {
@@ -540,17 +545,24 @@ __global__ __launch_bounds__(64) void dispatch_scan_kernel(uint32_t E, int32_t* 
     if (lane == 0) *count = picked;
 }
 __global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* ids, uint32_t n, uint32_t topk, uint32_t E, const int32_t* offsets,
-                                                             int32_t* slots, int32_t* rows) {
+                                                             int32_t* slots, int32_t* rows, bool aligned) {
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (e >= E) return;
     int32_t pos = offsets[e];
     if (offsets[e + 1] == pos) return;
-    for (uint32_t p0 = 0; p0 < n; p0 += 64) {
-        const uint32_t p = p0 + lane;
-        const bool m = p < n && ids[p] == int32_t(e);
-        const uint64_t mask = __ballot(m);
-        if (m) { const int32_t at = pos + __popcll(mask & ((1ull << lane) - 1)); slots[at] = int32_t(p); if (rows) rows[at] = int32_t(p / topk); }
-        pos += __popcll(mask);
+    const uint64_t below = (1ull << lane) - 1;
+    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // four neighbouring slots per lane: slots of lower lanes come first, then the lane's own in order
+        const uint32_t p = p0 + 4 * lane;
+        int4 v = make_int4(-1, -1, -1, -1);
+        if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array
+        else { if (p < n) v.x = ids[p]; if (p + 1 < n) v.y = ids[p + 1]; if (p + 2 < n) v.z = ids[p + 2]; if (p + 3 < n) v.w = ids[p + 3]; }
+        const bool m[4] = {v.x == int32_t(e), v.y == int32_t(e), v.z == int32_t(e), v.w == int32_t(e)};
+        const uint64_t mask[4] = {__ballot(m[0]), __ballot(m[1]), __ballot(m[2]), __ballot(m[3])};
+        int32_t at = pos + __popcll(mask[0] & below) + __popcll(mask[1] & below) + __popcll(mask[2] & below) + __popcll(mask[3] & below);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (m[j]) { slots[at] = int32_t(p + j); if (rows) rows[at] = int32_t((p + j) / topk); ++at; }
+        pos += __popcll(mask[0]) + __popcll(mask[1]) + __popcll(mask[2]) + __popcll(mask[3]);
     }
 }
 void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets,
@@ -560,9 +572,10 @@ void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_
         hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(1024), size_t(E + 1) * 4, s, ids, n, topk, E, offsets, slots, rows, selected, count, status);
         return;
     }
-    hipLaunchKernelGGL(dispatch_count_kernel, dim3((E + 3) / 4), dim3(256), 0, s, ids, n, E, offsets, status);
+    const bool aligned = reinterpret_cast<uintptr_t>(ids) % 16 == 0;
+    hipLaunchKernelGGL(dispatch_count_kernel, dim3((E + 3) / 4), dim3(256), 0, s, ids, n, E, offsets, status, aligned);
     hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(64), 0, s, E, offsets, selected, count);
-    hipLaunchKernelGGL(dispatch_place_kernel, dim3((E + 3) / 4), dim3(256), 0, s, ids, n, topk, E, offsets, slots, rows);
+    hipLaunchKernelGGL(dispatch_place_kernel, dim3((E + 3) / 4), dim3(256), 0, s, ids, n, topk, E, offsets, slots, rows, aligned);
 }
 
 // ---------------------------------------------------------------------------

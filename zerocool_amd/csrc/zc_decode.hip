@@ -410,7 +410,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
         if constexpr (NT == 1) {
             if (wave >= 1)
-                for (uint32_t tile = wg + nwg * (wave - 1); tile < I / 8; tile += nwg * (kDecodeWaves - 1)) {
+                for (uint32_t tile = wg + nwg * (kDecodeWaves - 1 - wave); tile < I / 8; tile += nwg * (kDecodeWaves - 1)) {   // last waves first: they have no routed tile
                     const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                     const uint8_t* rec = L.shared_record;
                     const uint8_t* w_row = rec + p.so[pr] + uint64_t(row) * (H / 2);
@@ -428,15 +428,18 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             else route_token<16>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
         }
         if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
-        for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
+        if constexpr (NT != 1) for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
         __syncthreads();
         clock();
         if (tid < n) {
             const int32_t e = ids[tid];
-            if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); next[tid] = -1; }
-            else next[tid] = atomicExch(&head[e], int32_t(tid));
+            if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); if constexpr (NT != 1) next[tid] = -1; }
+            else if constexpr (NT != 1) next[tid] = atomicExch(&head[e], int32_t(tid));
             if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * n + tid, e); st_f32(p.weights_trace + uint64_t(layer) * n + tid, weights[tid]); }
         }
+        // One token: slot j belongs to expert ids[j] and no two slots share an expert, so there is nothing to group.
+        uint32_t U = k;
+        if constexpr (NT != 1) {
         __syncthreads();
         {   // compact the experts that own at least one slot (any order: slots are independent)
             uint32_t base = 0;
@@ -455,9 +458,25 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             if (tid == 0) misc[0] = int32_t(base);
         }
         __syncthreads();
-        const uint32_t U = uint32_t(uniform(misc[0]));
+        U = uint32_t(uniform(misc[0]));
+        }
         clock();
-        {
+        if constexpr (NT == 1) {
+            const uint32_t tiles = I / 8, units = k * tiles;
+            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
+                const uint32_t slot = u / tiles, tile = u % tiles;
+                const int32_t e = uniform(ids[slot]);
+                if (e < 0 || e >= int32_t(E)) continue;   // reported above; the combine drops the slot
+                const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                const uint8_t* rec = L.records + uint64_t(e) * L.stride;
+                const uint8_t* w_row = rec + p.ro[pr] + uint64_t(row) * (H / 2);
+                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64);
+                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64);
+                const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
+                auto emit = [&](int, float v) { store_act(p.act, slot, row, v); };
+                ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
+            }
+        } else {
             const uint32_t tiles = I / 8, units = U * tiles;
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
                 const uint32_t e = uint32_t(uniform(experts[u / tiles])), tile = u % tiles;
@@ -542,6 +561,23 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
                     if (s0 == 0) clock();
                 }
+                if constexpr (NT == 1) {
+                    for (uint32_t slot = wave; slot <= k; slot += kDecodeWaves) {   // slot k is the shared expert's
+                        if (slot < s0 || slot >= s0 + sn) continue;
+                        const uint8_t* rec = L.shared_record; const uint64_t* off = p.so;
+                        if (slot < k) {
+                            const int32_t e = uniform(ids[slot]);
+                            if (e < 0 || e >= int32_t(E)) continue;
+                            rec = L.records + uint64_t(e) * L.stride; off = p.ro;
+                        }
+                        const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
+                        const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
+                        const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
+                        const uint8_t* img[PT] = {lds + lp.img_d + (slot - s0) * LI.bytes()}; LdsBf16 src[PT] = {source_of(slot - s0)};
+                        auto emit = [&](int, float v) { if (G == 0) otile[slot * 16 + col] = bf(v); };
+                        ZC_RUN_TILE(I / 128, w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit);
+                    }
+                } else
                 for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
                     const uint8_t* rec; const uint64_t* off; int32_t s;
                     if (u < U) { const uint32_t e = uint32_t(uniform(experts[u])); s = uniform(head[e]); rec = L.records + uint64_t(e) * L.stride; off = p.ro; }

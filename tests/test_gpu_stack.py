@@ -133,4 +133,12 @@ def test_stack_reports_invalid_router_output(ctx):
     with pytest.raises(z.ZcError) as err:
         ctx.moe_check()
     assert "BF16" in str(err.value)
+    # the single-token kernel has its own phases: the same two reports, and a clean run afterwards
+    for values, text in ((np.full(cfg.hidden, np.nan, f32), "invalid router output"), (np.full(cfg.hidden, 1.0000001, f32), "BF16")):
+        ctx.stack_decode(stack, ctx.upload(values), 1, out)
+        with pytest.raises(z.ZcError) as err:
+            ctx.moe_check()
+        assert text in str(err.value)
+    ctx.stack_decode(stack, ctx.upload(np.full(cfg.hidden, 0.5, f32)), 1, out)
+    ctx.moe_check()
     ctx.stack_destroy(stack)

@@ -110,6 +110,19 @@ def test_tied_logits_pick_the_lowest_ids(ctx):
 
     check_stack(ctx, cfg, 2, [1, 3], skew=None, mutate=repeat_rows)
 
+    # all 512 rows alike: every logit ties, the picks are experts 0..9 (more candidates than one wave holds: the pick-by-pick path);
+    # runs of 40: more tied candidates than picks, still within one wave
+    def one_row(layer):
+        rows = layer.router.numpy(np.uint16).reshape(cfg.experts, cfg.hidden)
+        layer.ctx.upload(np.ascontiguousarray(rows[np.zeros(cfg.experts, np.int64)]).reshape(-1), into=layer.router)
+
+    def long_runs(layer):
+        rows = layer.router.numpy(np.uint16).reshape(cfg.experts, cfg.hidden)
+        layer.ctx.upload(np.ascontiguousarray(rows[(np.arange(cfg.experts) // 40) * 40]).reshape(-1), into=layer.router)
+
+    check_stack(ctx, cfg, 2, [1, 2], skew=None, mutate=one_row)
+    check_stack(ctx, cfg, 2, [1, 2], skew=None, mutate=long_runs)
+
 
 def test_other_shapes_take_the_layered_path(ctx):  # hidden not a multiple of 512
     check_stack(ctx, workload.tiny_config(hidden=768, experts=64, topk=10, inter=512), 2, [1, 4], persistent=False)

@@ -118,9 +118,17 @@ __device__ __forceinline__ void stage_copy(const uint64_t* src, uint32_t count, 
 // Top-k of one token by one wavefront.  Lane l holds experts l*per .. l*per+per-1, so the
 // lowest lane holding the maximum, then the lowest slot inside it, is the lowest expert id:
 // one DPP maximum, one ballot and two scalar-lane reads per pick.
+//
+// With eight candidates per lane (512 experts) a faster way comes first.  The k-th largest of the 64 lane maxima is
+// found by a binary search over the bits of an order-preserving integer key (one compare and one ballot per step,
+// stopping as soon as exactly k lanes remain); k elements are then known to be at least that large, so the final top-k
+// lies among the elements at or above it: usually k to 2k of them.  They are gathered in ascending id order (`scratch`,
+// 128 words of LDS owned by this wave), one per lane, and each counts the candidates that beat it: larger value, or
+// equal value and lower id.  More than 64 candidates (masses of equal logits) or fewer than k valid lanes take the
+// picks one by one as before.
 template <int PER, class Clock>
 __device__ __forceinline__ void route_token(const float* logits, uint32_t E, uint32_t topk, uint32_t lane,
-                                            int32_t* ids, float* weights, Clock clock) {
+                                            int32_t* ids, float* weights, uint32_t* scratch, Clock clock) {
     const uint32_t per = PER == 16 ? (E + 63) / 64 : uint32_t(PER);
     const float ninf = __uint_as_float(0xff800000u);
     float cand[PER];
@@ -133,6 +141,61 @@ __device__ __forceinline__ void route_token(const float* logits, uint32_t E, uin
     float score = ninf, top = ninf;   // lane j keeps score j
     if (__ballot(cand[0] == 12345.678f) == ~0ull) return;   // (forces the loads to complete before the stamp)
     clock();
+    bool done = false;
+    if constexpr (PER == 8) {
+        constexpr uint32_t kLowest = 0x007fffffu;   // key of -inf: nothing valid is at or below it
+        uint32_t key[PER], best = 0;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            uint32_t u = __float_as_uint(cand[i]);
+            if (u == 0x80000000u) u = 0;             // the two zeros compare equal
+            key[i] = u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+            best = max(best, key[i]);
+        }
+        if (uint32_t(__popcll(__ballot(best > kLowest))) >= topk && topk < 64) {
+            uint32_t bar = 0;
+            for (int b = 31; b >= 0; --b) {
+                const uint32_t trial = bar | (1u << b), lanes = uint32_t(__popcll(__ballot(best >= trial)));
+                if (lanes >= topk) { bar = trial; if (lanes == topk) break; }
+            }
+            // candidates in ascending id order: lower lanes first, then the lane's own slots
+            const uint64_t below = (1ull << lane) - 1;
+            uint32_t before = 0, count = 0, mine = 0;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const uint64_t m = __ballot(key[i] >= bar);
+                before += uint32_t(__popcll(m & below)); count += uint32_t(__popcll(m));
+            }
+            if (count <= 64) {
+#pragma unroll
+                for (int i = 0; i < PER; ++i)
+                    if (key[i] >= bar) { scratch[before + mine] = key[i]; scratch[64 + before + mine] = lane * per + uint32_t(i); ++mine; }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const uint32_t k_mine = lane < count ? scratch[lane] : 0u, id_mine = lane < count ? scratch[64 + lane] : 0u;
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < count; ++j) {
+                    const uint32_t other = uint32_t(__builtin_amdgcn_readlane(int(k_mine), int(j)));
+                    rank += (other > k_mine || (other == k_mine && j < lane)) ? 1u : 0u;
+                }
+                if (lane < topk) { ids[lane] = -1; weights[lane] = ninf; }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                if (lane < count && rank < topk) {
+                    ids[rank] = int32_t(id_mine);
+                    weights[rank] = __uint_as_float(k_mine ^ ((k_mine >> 31) ? 0x80000000u : 0xffffffffu));   // the value back from its key
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                if (lane < topk) score = weights[lane];
+                top = weights[0];
+                done = true;
+            }
+        }
+    }
+    if (!done)
     for (uint32_t j = 0; j < topk; ++j) {
         float best = cand[0];
 #pragma unroll
@@ -316,8 +379,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         }
         clock();
         {
-            // One token: the shared gate/up tiles do not wait for the routing, so they run beside it in phase G on the
-            // waves that would otherwise idle while wave 0 picks the experts; this phase then only has the router.
+            // One token: the shared gate/up tiles run in phase G beside the routed ones, on waves that have no routed tile;
+            // this phase then only has the router.
             const uint32_t router_units = (E + 3) / 4, shared_units = NT == 1 ? 0 : I / 8, gate_units = (T + 1) / 2;
             const uint32_t units = router_units + shared_units + gate_units;
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
@@ -408,24 +471,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         refresh();
         clock();
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
-        if constexpr (NT == 1) {
-            if (wave >= 1)
-                for (uint32_t tile = wg + nwg * (kDecodeWaves - 1 - wave); tile < I / 8; tile += nwg * (kDecodeWaves - 1)) {   // last waves first: they have no routed tile
-                    const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                    const uint8_t* rec = L.shared_record;
-                    const uint8_t* w_row = rec + p.so[pr] + uint64_t(row) * (H / 2);
-                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64);
-                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64);
-                    const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
-                    auto emit = [&](int, float v) { store_act(p.shared_act, 0, row, v); };
-                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
-                }
-        }
         for (uint32_t t = wave; t < T; t += kDecodeWaves)
         {
             auto stamp = [&]() { if (t == 0) clock(); };
-            if (E == 512) route_token<8>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
-            else route_token<16>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, stamp);
+            uint32_t* scratch = reinterpret_cast<uint32_t*>(experts) + 128 * wave;   // the expert list is built later; 128 words per wave fit it for 512 experts
+            if (E == 512) route_token<8>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
+            else route_token<16>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
         }
         if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
         if constexpr (NT != 1) for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
@@ -462,18 +513,21 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         }
         clock();
         if constexpr (NT == 1) {
-            const uint32_t tiles = I / 8, units = k * tiles;
+            // the shared expert's gate/up tiles close the list (slot k): with 1280 routed tiles on 256 workgroups they land on
+            // waves that have no routed tile
+            const uint32_t tiles = I / 8, units = (k + 1) * tiles;
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
                 const uint32_t slot = u / tiles, tile = u % tiles;
-                const int32_t e = uniform(ids[slot]);
+                const int32_t e = slot < k ? uniform(ids[slot]) : 0;
                 if (e < 0 || e >= int32_t(E)) continue;   // reported above; the combine drops the slot
                 const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                const uint8_t* rec = L.records + uint64_t(e) * L.stride;
-                const uint8_t* w_row = rec + p.ro[pr] + uint64_t(row) * (H / 2);
-                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64);
-                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64);
+                const uint8_t* rec = slot < k ? L.records + uint64_t(e) * L.stride : L.shared_record;
+                const uint64_t* off = slot < k ? p.ro : p.so;
+                const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
+                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
+                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 2]) + uint64_t(row) * (H / 64);
                 const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
-                auto emit = [&](int, float v) { store_act(p.act, slot, row, v); };
+                auto emit = [&](int, float v) { if (slot < k) store_act(p.act, slot, row, v); else store_act(p.shared_act, 0, row, v); };
                 ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
             }
         } else {

@@ -401,6 +401,28 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     float c[NT];
 #pragma unroll
                     for (int t = 0; t < NT; ++t) c[t] = 0;
+                    if (NT == 1 && pieces % kRouterRing == 0) {
+                        // one token, whole rings (hidden a multiple of 1024): straight-line bodies of eight pieces, the eight input
+                        // pieces read from LDS together so that one wait covers them, the next ring requested before the chain runs
+                        for (uint32_t i0 = 0; i0 < pieces; i0 += kRouterRing) {
+                            uint4 xv[kRouterRing], wc[kRouterRing];
+#pragma unroll
+                            for (int j = 0; j < kRouterRing; ++j) { xv[j] = *reinterpret_cast<const uint4*>(xh_all + split * P + (i0 + j) * 8); wc[j] = wv[j]; }
+                            if (i0 + kRouterRing < pieces) {
+#pragma unroll
+                                for (int j = 0; j < kRouterRing; ++j) wv[j] = ldg_u4(wr, i0 + kRouterRing + j);
+                            }
+#pragma unroll
+                            for (int j = 0; j < kRouterRing; ++j) {
+                                const uint32_t xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {wc[j].x, wc[j].y, wc[j].z, wc[j].w};
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) {
+                                    c[0] = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c[0]);
+                                    c[0] = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c[0]);
+                                }
+                            }
+                        }
+                    } else
                     for (uint32_t i0 = 0; i0 < pieces; i0 += kRouterRing) {
 #pragma unroll
                         for (int j = 0; j < kRouterRing; ++j) {

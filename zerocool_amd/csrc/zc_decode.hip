@@ -286,6 +286,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         // One token: the wave's first router unit starts loading its weights while the input row is staged and its image
         // built (the weights do not depend on the input).
         const uint32_t first_unit = wg + nwg * wave;
+        // One token with whole rings of router pieces (hidden a multiple of 1024) and a workgroup to spare per router unit:
+        // unit u runs on workgroup u with its K partitions cut into segments of eight pieces, one segment per wave.  All
+        // segments load at once; the chain value then passes from wave to wave through LDS, so the unit pays one load
+        // latency instead of one per ring.  The shared gate dot goes to the next workgroup, all of whose threads form the
+        // products before one half-wave adds them in the reference's order.
+        const uint32_t router_pieces = H / 128, router_segments = router_pieces / kRing;
+        const bool segmented = NT == 1 && router_pieces % kRing == 0 && router_segments <= kDecodeWaves && (E + 3) / 4 < nwg;
         uint4 early[kRing];
 #pragma unroll
         for (int i = 0; i < kRing; ++i) early[i] = make_uint4(0, 0, 0, 0);
@@ -305,11 +312,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             }
             uint4 gate_piece = make_uint4(0, 0, 0, 0);
             if (tid < H / 8) gate_piece = ldg_u4(L.shared_gate, tid);
-            if (first_unit < (E + 3) / 4) {   // issued after the input's loads: waiting for those does not wait for these
-                const uint32_t e = first_unit * 4 + lane / 16, split = lane % 16, P = H / 16;
+            if (segmented ? (wg < (E + 3) / 4 && wave < router_segments) : first_unit < (E + 3) / 4) {   // issued after the input's loads
+                const uint32_t unit = segmented ? wg : first_unit, first_piece = segmented ? wave * kRing : 0u;
+                const uint32_t e = unit * 4 + lane / 16, split = lane % 16, P = H / 16;
                 const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
 #pragma unroll
-                for (int i = 0; i < kRing; ++i) if (uint32_t(i) < P / 8) early[i] = ldg_u4(wr, i);
+                for (int i = 0; i < kRing; ++i) if (first_piece + uint32_t(i) < P / 8) early[i] = ldg_u4(wr, first_piece + i);
             }
             xint_prepare_begin(LH, lds + lp.img_rg, 1);
             __syncthreads();
@@ -383,6 +391,53 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             // this phase then only has the router.
             const uint32_t router_units = (E + 3) / 4, shared_units = NT == 1 ? 0 : I / 8, gate_units = (T + 1) / 2;
             const uint32_t units = router_units + shared_units + gate_units;
+            if (segmented) {
+                float* handoff = reinterpret_cast<float*>(experts);   // 64 chain values; the expert list is not in use yet
+                if (wg < router_units) {
+                    const uint32_t e = wg * 4 + lane / 16, split = lane % 16, P = H / 16;
+                    float c = 0;
+                    for (uint32_t seg = 0; seg < router_segments; ++seg) {
+                        if (wave == seg) {
+                            if (seg) c = handoff[lane];
+                            uint4 xv[kRing];
+#pragma unroll
+                            for (int j = 0; j < kRing; ++j) xv[j] = *reinterpret_cast<const uint4*>(xh_all + split * P + (seg * kRing + j) * 8);
+#pragma unroll
+                            for (int j = 0; j < kRing; ++j) {
+                                const uint32_t xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {early[j].x, early[j].y, early[j].z, early[j].w};
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) {
+                                    c = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c);
+                                    c = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c);
+                                }
+                            }
+                            if (seg + 1 < router_segments) handoff[lane] = c;
+                            else {
+                                // partials added 0..15: after step s the lane of partition i <= s holds ((c0 + c1) + ..) + ci
+                                const float offset = (L.offsets && e < E) ? ldg_f32(L.offsets, e) : 0.0f;
+                                float sum = 0.0f + c;
+#pragma unroll
+                                for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c;
+                                if (split == 15 && e < E) st_f32(p.logits + e, L.offsets ? sum + offset : sum);
+                            }
+                        }
+                        if (seg + 1 < router_segments) __syncthreads();
+                    }
+                } else if (wg == router_units) {
+                    // shared_expert_gate (qwen.metal:499-506): reference lane l adds the products of k = l, l + 32, ... in turn
+                    float* products = reinterpret_cast<float*>(lds + lp.gprod);     // [32 lanes][hidden / 32 + 1]
+                    const uint16_t* gw = reinterpret_cast<const uint16_t*>(lds + lp.gatew);
+                    const uint32_t pitch = H / 32 + 1;
+                    for (uint32_t kk = tid; kk < H; kk += kDecodeThreads) products[(kk % 32) * pitch + kk / 32] = b16(xh_all[kk]) * b16(gw[kk]);
+                    __syncthreads();
+                    if (wave == 0) {
+                        float sum = 0;
+                        if (lane < 32) for (uint32_t j = 0; j < H / 32; ++j) sum += products[lane * pitch + j];
+                        sum = lane_sum32(sum);
+                        if (lane == 0) st_f32(p.gate, bf(sum));
+                    }
+                }
+            } else
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
                 if (u < router_units) {
                     // four experts x sixteen K partitions; k-ascending fused chain per partition
@@ -735,7 +790,8 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
     lp.head = take(E * 4); lp.next = take(NT * topk * 4); lp.experts = take(E * 4); lp.misc = take(64); lp.gatew = take(H * 2);
     lp.region = at;
     lp.img_rg = lp.region; lp.xh = lp.img_rg + NT * LH.bytes();
-    const uint32_t rg_end = lp.xh + align16(NT * H * 2);
+    lp.gprod = lp.xh + align16(NT * H * 2);   // one token: the shared gate dot's products, [32][hidden / 32 + 1] fp32
+    const uint32_t rg_end = lp.gprod + (NT == 1 ? align16(32 * (H / 32 + 1) * 4) : 0);
     lp.otile = lp.region;
     const uint32_t slots = NT * (topk + 1);
     lp.img_d = lp.otile + align16(slots * 16 * 4);

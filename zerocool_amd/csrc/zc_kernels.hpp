@@ -73,7 +73,7 @@ struct DecodeParams {
 constexpr uint32_t kDecodeStamps = 15;
 struct DecodeLdsPlan {
     uint32_t ids, weights, gatev, head, next, experts, misc, region, total;
-    uint32_t img_rg, xh, img_d, ah, otile, slots_per_batch, gatew;
+    uint32_t img_rg, xh, gprod, img_d, ah, otile, slots_per_batch, gatew;
 };
 DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t NT, uint32_t lds_limit);
 hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp);

@@ -26,6 +26,9 @@ namespace zc {
 
 // A value every lane holds alike (read from LDS), moved to a scalar register so that control flow on it is scalar.
 __device__ __forceinline__ int32_t uniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+// Workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load in flight, which would
+// end a prefetch early.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ __forceinline__ void st_f32(float* p, float v) { ZC_ST(reinterpret_cast<uint32_t*>(p), __float_as_uint(v)); }
 __device__ __forceinline__ void st_i32(int32_t* p, int32_t v) { ZC_ST(reinterpret_cast<uint32_t*>(p), uint32_t(v)); }
 
@@ -302,25 +305,46 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
             const bool glue = layer != 0;
             const float* row = glue ? p.layer_out : p.x_in;
-            const uint32_t peak = glue ? ZC_LD(p.maxabs + (layer - 1) * T) : 0u;
+            // A workgroup that owns a segmented router unit issues the same loads from every lane in the same order, with
+            // clamped addresses where a lane has nothing to fetch: the wait for the input's values can then leave exactly the
+            // later router loads in flight (a load under a branch forces a full wait), and its two barriers order LDS traffic
+            // only.  The other workgroups have no router loads to keep in flight and fetch only what they need.
+            const bool keep_in_flight = uniform(segmented && wg < (E + 3) / 4);
+            uint32_t peak = 0;
             uint64_t v[8];
-#pragma unroll
-            for (int w = 0; w < 8; ++w) v[w] = 0;
-            if (tid < H / 16) {
-#pragma unroll
-                for (int w = 0; w < 8; ++w) v[w] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(row) + tid * 8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
             uint4 gate_piece = make_uint4(0, 0, 0, 0);
-            if (tid < H / 8) gate_piece = ldg_u4(L.shared_gate, tid);
-            if (segmented ? (wg < (E + 3) / 4 && wave < router_segments) : first_unit < (E + 3) / 4) {   // issued after the input's loads
-                const uint32_t unit = segmented ? wg : first_unit, first_piece = segmented ? wave * kRing : 0u;
-                const uint32_t e = unit * 4 + lane / 16, split = lane % 16, P = H / 16;
+            if (keep_in_flight) {
+                peak = ZC_LD(p.maxabs + (glue ? layer - 1 : 0u) * T);
+                const uint32_t block = min(tid, H / 16 - 1);
+#pragma unroll
+                for (int w = 0; w < 8; ++w) v[w] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(row) + block * 8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                gate_piece = ldg_u4(L.shared_gate, min(tid, H / 8 - 1));
+                asm volatile("" ::: "memory");   // the router loads stay behind the loads above
+                const uint32_t first_piece = min(wave, router_segments - 1) * kRing;
+                const uint32_t e = wg * 4 + lane / 16, split = lane % 16, P = H / 16;
                 const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
 #pragma unroll
-                for (int i = 0; i < kRing; ++i) if (first_piece + uint32_t(i) < P / 8) early[i] = ldg_u4(wr, first_piece + i);
+                for (int i = 0; i < kRing; ++i) early[i] = ldg_u4(wr, first_piece + i);
+                xint_prepare_begin(LH, lds + lp.img_rg, 1);
+                lds_barrier();
+            } else {
+                if (glue) peak = ZC_LD(p.maxabs + (layer - 1) * T);
+#pragma unroll
+                for (int w = 0; w < 8; ++w) v[w] = 0;
+                if (tid < H / 16) {
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) v[w] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(row) + tid * 8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (tid < H / 8) gate_piece = ldg_u4(L.shared_gate, tid);
+                if (!segmented && first_unit < (E + 3) / 4) {   // issued after the input's loads
+                    const uint32_t e = first_unit * 4 + lane / 16, split = lane % 16, P = H / 16;
+                    const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
+#pragma unroll
+                    for (int i = 0; i < kRing; ++i) if (uint32_t(i) < P / 8) early[i] = ldg_u4(wr, i);
+                }
+                xint_prepare_begin(LH, lds + lp.img_rg, 1);
+                __syncthreads();
             }
-            xint_prepare_begin(LH, lds + lp.img_rg, 1);
-            __syncthreads();
             if (tid < H / 16) {
                 const float m = __uint_as_float(peak), inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
                 RegF32 block; uint32_t low = 0, packed[8];
@@ -339,7 +363,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 xint_prepare_block(block, LH, lds + lp.img_rg, tid);
             }
             if (tid < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid] = gate_piece;
-            __syncthreads();
+            lds_barrier();
         } else {
             {
                 uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);

@@ -626,6 +626,7 @@ struct zc_hip_stack {
     uint8_t* arena = nullptr; uint64_t arena_bytes = 0;
     float *logits = nullptr, *gate = nullptr, *shared_act = nullptr, *act = nullptr, *layer_out = nullptr;
     uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
+    unsigned long long* tlogits = nullptr; uint32_t *tact = nullptr, *tout = nullptr;   // tagged exchange buffers of the one-token kernel
     uint32_t epoch = 1u << 12;
     int cus = 0; uint32_t lds_limit = 0;
     bool persistent_ok = false;
@@ -677,7 +678,8 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         auto take = [&](uint64_t bytes) { const uint64_t o = at; at += align_up(bytes, 256); return o; };
         const uint64_t o_layers = take(sizeof(zc::DecodeLayer) * n_layers), o_logits = take(uint64_t(Tp) * E * 4), o_gate = take(Tp * 4),
                        o_sact = take(uint64_t(Tp) * I * 4), o_act = take(uint64_t(Tp) * k * I * 4), o_lout = take(uint64_t(Tp) * H * 4),
-                       o_max = take(uint64_t(n_layers) * Tp * 4), o_sync = take(zc::kDecodeSyncBytes);
+                       o_max = take(uint64_t(n_layers) * Tp * 4), o_sync = take(zc::kDecodeSyncBytes),
+                       o_tlogits = take(uint64_t(E + 1) * 8), o_tact = take(uint64_t(k + 1) * I * 4), o_tout = take(uint64_t(2) * H * 4);
         if (zc_hip_alloc(ctx, at, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
         st->arena = static_cast<uint8_t*>(p); st->arena_bytes = at;
         st->dev_layers = reinterpret_cast<zc::DecodeLayer*>(st->arena + o_layers);
@@ -685,6 +687,8 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         st->shared_act = reinterpret_cast<float*>(st->arena + o_sact); st->act = reinterpret_cast<float*>(st->arena + o_act);
         st->layer_out = reinterpret_cast<float*>(st->arena + o_lout); st->maxabs = reinterpret_cast<uint32_t*>(st->arena + o_max);
         st->sync = reinterpret_cast<uint32_t*>(st->arena + o_sync);
+        st->tlogits = reinterpret_cast<unsigned long long*>(st->arena + o_tlogits); st->tact = reinterpret_cast<uint32_t*>(st->arena + o_tact);
+        st->tout = reinterpret_cast<uint32_t*>(st->arena + o_tout);
         std::vector<zc::DecodeLayer> host(n_layers);
         for (uint32_t l = 0; l < n_layers; ++l) {
             const zc_moe_layer& y = host_layers[l];
@@ -744,6 +748,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.layers = st->dev_layers; p.x_in = x; p.out = out;
         p.logits = st->logits; p.gate = st->gate; p.shared_act = st->shared_act; p.act = st->act; p.layer_out = st->layer_out;
         p.maxabs = st->maxabs;
+        p.tlogits = st->tlogits; p.tact = st->tact; p.tout = st->tout;
         p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
         if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
         p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;

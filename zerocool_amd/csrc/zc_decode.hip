@@ -61,6 +61,24 @@ struct Barrier {
         __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }
+    // One token: data crosses between workgroups with a tag beside every value and readers poll the data itself (until()).
+    // The flag then only says "this workgroup has read everything the others wrote for this layer": it is stored without
+    // waiting for anything, and checked before the next layer's first write to those buffers.
+    __device__ __forceinline__ void arrive() {
+        ++epoch;
+        uint32_t me = blockIdx.x, thread = threadIdx.x;
+        asm volatile("" : "+s"(me));
+        asm volatile("" : "+v"(thread));
+        if (thread == 0) ZC_ST(mem + kFlagStride * me, epoch);
+    }
+    // Repeats attempt() until it succeeds, bounded like spin().
+    template <class Attempt>
+    __device__ __forceinline__ void until(Attempt attempt) {
+        for (uint32_t i = 0; !attempt(); ++i) {
+            if ((i & 31u) == 31u && ZC_LD(mem + kAbortWord) == token) return;
+            if (i >= spin_limit) { ZC_ST(mem + kAbortWord, token); atomicOr(status, 2); return; }
+        }
+    }
     // Bounded: a grid that is not fully resident must not hang the GPU.  Epochs only grow,
     // so "reached" is a signed comparison that survives wrap-around.
     __device__ __forceinline__ void spin(uint32_t* word) {
@@ -129,18 +147,17 @@ __device__ __forceinline__ void stage_copy(const uint64_t* src, uint32_t count, 
 // 128 words of LDS owned by this wave), one per lane, and each counts the candidates that beat it: larger value, or
 // equal value and lower id.  More than 64 candidates (masses of equal logits) or fewer than k valid lanes take the
 // picks one by one as before.
-template <int PER, class Clock>
-__device__ __forceinline__ void route_token(const float* logits, uint32_t E, uint32_t topk, uint32_t lane,
+//
+// fetch(cand, per) fills the lane's logits (-inf where it has no expert).
+template <int PER, class Fetch, class Clock>
+__device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t topk, uint32_t lane,
                                             int32_t* ids, float* weights, uint32_t* scratch, Clock clock) {
     const uint32_t per = PER == 16 ? (E + 63) / 64 : uint32_t(PER);
     const float ninf = __uint_as_float(0xff800000u);
     float cand[PER];
+    fetch(cand, per);
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-        const uint32_t e = lane * per + i;
-        const float c = (uint32_t(i) < per && e < E) ? load_shared_f32(logits + e) : ninf;
-        cand[i] = c > ninf ? c : ninf;   // NaN and -inf never win
-    }
+    for (int i = 0; i < PER; ++i) cand[i] = cand[i] > ninf ? cand[i] : ninf;   // NaN and -inf never win
     float score = ninf, top = ninf;   // lane j keeps score j
     if (__ballot(cand[0] == 12345.678f) == ~0ull) return;   // (forces the loads to complete before the stamp)
     clock();
@@ -284,6 +301,11 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         };
         refresh();
         clock();
+        // One token: the 16-bit tag of everything layer l exchanges, never 0 (the buffers start as zeros) and different
+        // from the tags of the layers (and launches) just before it
+        auto tag_of = [&](uint32_t l) { return (p.epoch + l) % 65535u + 1u; };
+        const uint32_t tag = tag_of(layer);
+        auto st_logit = [&](uint32_t index, float v) { ZC_ST(p.tlogits + index, (uint64_t(tag) << 32) | __float_as_uint(v)); };
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
         // One token: the wave's first router unit starts loading its weights while the input row is staged and its image
@@ -300,24 +322,33 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
 #pragma unroll
         for (int i = 0; i < kRing; ++i) early[i] = make_uint4(0, 0, 0, 0);
         if constexpr (NT == 1) {
-            // One token: thread b fetches the sixteen fp32 values of block b, applies the glue's scale, writes the BF16 copy and
-            // builds the block's image pieces straight from registers; the shared gate row and the scale ride along.
+            // One token: thread b fetches the sixteen values of block b, applies the glue's scale, writes the BF16 copy and
+            // builds the block's image pieces straight from registers; the shared gate row rides along.  After the first
+            // layer the values are the previous layer's tagged words: the thread fetches them again until every tag is that
+            // layer's, and the workgroup forms the glue's scale (the largest magnitude of the row) itself.
             uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
             const bool glue = layer != 0;
-            const float* row = glue ? p.layer_out : p.x_in;
+            const uint64_t* row = glue ? reinterpret_cast<const uint64_t*>(p.tout + ((layer - 1) & 1u) * H) : reinterpret_cast<const uint64_t*>(p.x_in);
+            const uint32_t want = tag_of(layer - 1);
             // A workgroup that owns a segmented router unit issues the same loads from every lane in the same order, with
             // clamped addresses where a lane has nothing to fetch: the wait for the input's values can then leave exactly the
             // later router loads in flight (a load under a branch forces a full wait), and its two barriers order LDS traffic
             // only.  The other workgroups have no router loads to keep in flight and fetch only what they need.
             const bool keep_in_flight = uniform(segmented && wg < (E + 3) / 4);
-            uint32_t peak = 0;
             uint64_t v[8];
             uint4 gate_piece = make_uint4(0, 0, 0, 0);
-            if (keep_in_flight) {
-                peak = ZC_LD(p.maxabs + (glue ? layer - 1 : 0u) * T);
-                const uint32_t block = min(tid, H / 16 - 1);
+            const uint32_t own = min(tid, H / 16 - 1);
+            // the flag of workgroup `tid` (all have finished reading what the previous layer exchanged), checked below
+            uint32_t seen = ZC_LD(p.sync + kFlagStride * min(tid, nwg - 1));
+            auto stale = [&]() {
+                uint32_t bad = 0;
 #pragma unroll
-                for (int w = 0; w < 8; ++w) v[w] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(row) + block * 8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int w = 0; w < 8; ++w) bad |= ((uint32_t(v[w]) ^ want) | (uint32_t(v[w] >> 32) ^ want)) & 0xffffu;
+                return bad != 0;
+            };
+            if (keep_in_flight) {
+#pragma unroll
+                for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + own * 8 + w);
                 gate_piece = ldg_u4(L.shared_gate, min(tid, H / 8 - 1));
                 asm volatile("" ::: "memory");   // the router loads stay behind the loads above
                 const uint32_t first_piece = min(wave, router_segments - 1) * kRing;
@@ -325,15 +356,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
 #pragma unroll
                 for (int i = 0; i < kRing; ++i) early[i] = ldg_u4(wr, first_piece + i);
-                xint_prepare_begin(LH, lds + lp.img_rg, 1);
-                lds_barrier();
             } else {
-                if (glue) peak = ZC_LD(p.maxabs + (layer - 1) * T);
 #pragma unroll
                 for (int w = 0; w < 8; ++w) v[w] = 0;
                 if (tid < H / 16) {
 #pragma unroll
-                    for (int w = 0; w < 8; ++w) v[w] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(row) + tid * 8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + tid * 8 + w);
                 }
                 if (tid < H / 8) gate_piece = ldg_u4(L.shared_gate, tid);
                 if (!segmented && first_unit < (E + 3) / 4) {   // issued after the input's loads
@@ -342,15 +370,45 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
 #pragma unroll
                     for (int i = 0; i < kRing; ++i) if (uint32_t(i) < P / 8) early[i] = ldg_u4(wr, i);
                 }
-                xint_prepare_begin(LH, lds + lp.img_rg, 1);
-                __syncthreads();
             }
+            if (glue) {
+                if (tid < H / 16 && stale())
+                    bar.until([&]() {
+#pragma unroll
+                        for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + own * 8 + w);
+                        return !stale();
+                    });
+                // every workgroup has taken what it needed from the buffers this layer is about to overwrite
+                for (uint32_t w = tid; w < nwg; w += kDecodeThreads) {
+                    if (w != tid) seen = ZC_LD(p.sync + kFlagStride * w);
+                    if (int32_t(seen - bar.epoch) < 0) bar.spin(p.sync + kFlagStride * w);
+                }
+                // largest magnitude of the row (NaN takes no part): per wave here, across the waves after the barrier
+                uint32_t m = 0;
+                if (tid < H / 16) {
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) {
+                        const uint32_t a = uint32_t(v[w]) & 0x7fff0000u, c = uint32_t(v[w] >> 32) & 0x7fff0000u;
+                        m = max(m, a > 0x7f800000u ? 0u : a); m = max(m, c > 0x7f800000u ? 0u : c);
+                    }
+                }
+                m = __float_as_uint(wave_max_f32(__uint_as_float(m)));
+                if (lane == 0) misc[1 + wave] = int32_t(m);
+            }
+            xint_prepare_begin(LH, lds + lp.img_rg, 1);
+            if (keep_in_flight) lds_barrier(); else __syncthreads();
             if (tid < H / 16) {
+                uint32_t peak = 0;
+                if (glue) {
+#pragma unroll
+                    for (uint32_t w = 0; w < kDecodeWaves; ++w) peak = max(peak, uint32_t(misc[1 + w]));
+                }
+                const uint32_t keep = glue ? 0xffff0000u : 0xffffffffu;   // a tagged word keeps its tag in the low half
                 const float m = __uint_as_float(peak), inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
                 RegF32 block; uint32_t low = 0, packed[8];
 #pragma unroll
                 for (int w = 0; w < 8; ++w) {
-                    float a = __uint_as_float(uint32_t(v[w])), c = __uint_as_float(uint32_t(v[w] >> 32));
+                    float a = __uint_as_float(uint32_t(v[w]) & keep), c = __uint_as_float(uint32_t(v[w] >> 32) & keep);
                     if (glue) { a = bf(a * inv); c = bf(c * inv); }
                     const uint32_t ua = __float_as_uint(a), uc = __float_as_uint(c);
                     low |= (ua | uc) & 0xffffu;
@@ -442,7 +500,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                                 float sum = 0.0f + c;
 #pragma unroll
                                 for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c;
-                                if (split == 15 && e < E) st_f32(p.logits + e, L.offsets ? sum + offset : sum);
+                                if (split == 15 && e < E) st_logit(e, L.offsets ? sum + offset : sum);
                             }
                         }
                         if (seg + 1 < router_segments) __syncthreads();
@@ -458,7 +516,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         float sum = 0;
                         if (lane < 32) for (uint32_t j = 0; j < H / 32; ++j) sum += products[lane * pitch + j];
                         sum = lane_sum32(sum);
-                        if (lane == 0) st_f32(p.gate, bf(sum));
+                        if (lane == 0) st_logit(E, bf(sum));
                     }
                 }
             } else
@@ -531,7 +589,10 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         float sum = 0.0f + c[t];
 #pragma unroll
                         for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c[t];
-                        if (split == 15 && e < E) st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + offset : sum);
+                        if (split == 15 && e < E) {
+                            if constexpr (NT == 1) st_logit(e, L.offsets ? sum + offset : sum);
+                            else st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + offset : sum);
+                        }
                     }
                 } else if (u < router_units + shared_units) {
                     const uint32_t tile = u - router_units, row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
@@ -563,12 +624,14 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                             for (int j = 0; j < 8; ++j) sum += a[j] * g[j];
                         }
                     sum = lane_sum32(sum);
-                    if (t < T && l32 == 0) st_f32(p.gate + t, bf(sum));
+                    if (t < T && l32 == 0) {
+                        if constexpr (NT == 1) st_logit(E, bf(sum)); else st_f32(p.gate + t, bf(sum));
+                    }
                 }
             }
         }
         clock_all();
-        bar.wait();
+        if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the routing below polls the logits themselves
         refresh();
         clock();
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
@@ -576,10 +639,46 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         {
             auto stamp = [&]() { if (t == 0) clock(); };
             uint32_t* scratch = reinterpret_cast<uint32_t*>(experts) + 128 * wave;   // the expert list is built later; 128 words per wave fit it for 512 experts
-            if (E == 512) route_token<8>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
-            else route_token<16>(p.logits + uint64_t(t) * E, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
+            // the lane's logits: written by other workgroups; one token polls the tagged words until all carry this layer's tag
+            auto fetch = [&](auto& cand, uint32_t per) {
+                constexpr int PER = int(sizeof(cand) / sizeof(float));
+                const float ninf = __uint_as_float(0xff800000u);
+                if constexpr (NT == 1) {
+                    uint64_t w[PER];
+                    bar.until([&]() {
+                        uint32_t bad = 0;
+#pragma unroll
+                        for (int i = 0; i < PER; ++i) {
+                            const uint32_t e = lane * per + i;
+                            w[i] = (uint32_t(i) < per && e < E) ? ZC_LD(p.tlogits + e) : (uint64_t(tag) << 32) | 0xff800000u;
+                        }
+#pragma unroll
+                        for (int i = 0; i < PER; ++i) bad |= uint32_t(w[i] >> 32) ^ tag;
+                        return bad == 0;
+                    });
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) cand[i] = __uint_as_float(uint32_t(w[i]));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) {
+                        const uint32_t e = lane * per + i;
+                        cand[i] = (uint32_t(i) < per && e < E) ? load_shared_f32(p.logits + uint64_t(t) * E + e) : ninf;
+                    }
+                }
+            };
+            if (E == 512) route_token<8>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
+            else route_token<16>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
         }
-        if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
+        // the combine's gate factor, ready early
+        if constexpr (NT == 1) {
+            if (tid == 64) {   // a wave that does not route
+                uint64_t w = 0;
+                bar.until([&]() { w = ZC_LD(p.tlogits + E); return uint32_t(w >> 32) == tag; });
+                gatev[0] = bf(sigmoid_bf(__uint_as_float(uint32_t(w))));
+            }
+        } else {
+            if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));
+        }
         if constexpr (NT != 1) for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
         __syncthreads();
         clock();
@@ -628,7 +727,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
                 const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 2]) + uint64_t(row) * (H / 64);
                 const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
-                auto emit = [&](int, float v) { if (slot < k) store_act(p.act, slot, row, v); else store_act(p.shared_act, 0, row, v); };
+                // SwiGLU of the finished tile as tagged words, one per activation: row `slot` of the tagged buffer (row k: shared)
+                auto emit = [&](int, float v) {
+                    const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                    const uint32_t a = __float_as_uint(swiglu_bf(v, up));
+                    if (lane < 8) ZC_ST(p.tact + uint64_t(slot) * I + row, (a & 0xffff0000u) | tag);
+                };
                 ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
             }
         } else {
@@ -656,13 +760,14 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             }
         }
         clock_all();
-        bar.wait();
+        if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the staging below polls the activations themselves
         refresh();
         clock();
         // ---------------- phase D: down tiles per 16 output rows, combine ----------------
         float* otile = reinterpret_cast<float*>(lds + lp.otile);
         const uint32_t slots_total = n + T, SB = lp.slots_per_batch;
         if (wg >= H / 16) { clock(); clock(); clock(); }   // workgroups without a row tile keep the stamp count
+        if constexpr (NT == 1) { if (wg >= H / 16) bar.arrive(); }
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
             const uint32_t row = rt * 16 + col;
             for (uint32_t s0 = 0; s0 < slots_total; s0 += SB) {
@@ -676,35 +781,63 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     const uint32_t per = I / 16, total = sn * per;
                     constexpr int kMine = 2;
                     for (uint32_t base = 0; base < total; base += kDecodeThreads * kMine) {
-                        RegBf16 piece[kMine];
+                        uint64_t words[kMine][8];   // sixteen tagged words of a block; a slot without a valid expert stays zero
+                        bool wanted[kMine];
 #pragma unroll
                         for (int j = 0; j < kMine; ++j) {
                             const uint32_t blk = base + j * kDecodeThreads + tid;
 #pragma unroll
-                            for (int w = 0; w < 4; ++w) piece[j].w[w] = 0;
+                            for (int w = 0; w < 8; ++w) words[j][w] = 0;
+                            wanted[j] = false;
                             if (blk < total) {
-                                const uint32_t slot = s0 + blk / per, b = blk % per;
-                                const uint64_t* src = (slot < n ? reinterpret_cast<const uint64_t*>(p.act) + uint64_t(slot) * I / 4
-                                                                : reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(slot - n) * I / 4) + b * 4;
-#pragma unroll
-                                for (int w = 0; w < 4; ++w) piece[j].w[w] = __hip_atomic_load(src + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                const uint32_t slot = s0 + blk / per;
+                                const int32_t e = slot < k ? ids[slot] : 0;
+                                wanted[j] = e >= 0 && e < int32_t(E);
                             }
                         }
-                        if (base == 0) { xint_prepare_begin(LI, lds + lp.img_d, sn); __syncthreads(); }   // while the loads are in flight
+                        bool prepared = false;
+                        auto fetch = [&]() {
+                            uint32_t bad = 0;
+#pragma unroll
+                            for (int j = 0; j < kMine; ++j) {
+                                const uint32_t blk = base + j * kDecodeThreads + tid;
+                                if (wanted[j]) {
+                                    const uint64_t* src = reinterpret_cast<const uint64_t*>(p.tact + uint64_t(s0 + blk / per) * I + (blk % per) * 16);
+#pragma unroll
+                                    for (int w = 0; w < 8; ++w) words[j][w] = ZC_LD(src + w);
+                                }
+                            }
+                            if (base == 0 && !prepared) { xint_prepare_begin(LI, lds + lp.img_d, sn); prepared = true; }   // while the loads are in flight
+#pragma unroll
+                            for (int j = 0; j < kMine; ++j)
+                                if (wanted[j]) {
+#pragma unroll
+                                    for (int w = 0; w < 8; ++w) bad |= ((uint32_t(words[j][w]) ^ tag) | (uint32_t(words[j][w] >> 32) ^ tag)) & 0xffffu;
+                                }
+                            return bad == 0;
+                        };
+                        bar.until(fetch);
+                        if (base == 0) __syncthreads();
 #pragma unroll
                         for (int j = 0; j < kMine; ++j) {
                             const uint32_t blk = base + j * kDecodeThreads + tid;
                             if (blk < total) {
                                 const uint32_t q = blk / per, b = blk % per;
-                                uint64_t* copy = reinterpret_cast<uint64_t*>(ah + q * I + b * 16);
+                                RegF32 piece;
+                                uint32_t* copy = reinterpret_cast<uint32_t*>(ah + q * I + b * 16);
 #pragma unroll
-                                for (int w = 0; w < 4; ++w) copy[w] = piece[j].w[w];
-                                xint_prepare_block(piece[j], LI, lds + lp.img_d + q * LI.bytes(), b);
+                                for (int w = 0; w < 8; ++w) {
+                                    const uint32_t lo = uint32_t(words[j][w]) & 0xffff0000u, hi = uint32_t(words[j][w] >> 32) & 0xffff0000u;
+                                    piece.bits[2 * w] = lo; piece.bits[2 * w + 1] = hi;
+                                    copy[w] = (lo >> 16) | hi;
+                                }
+                                xint_prepare_block(piece, LI, lds + lp.img_d + q * LI.bytes(), b);
                             }
                         }
                     }
                     if (s0 == 0) { clock(); clock(); }
                     __syncthreads();
+                    if (rt + nwg >= H / 16 && s0 + SB >= slots_total) bar.arrive();   // nothing more to read from other workgroups in this layer
                 } else {
                     {   // rows s0 .. s0+sn-1 of [act ; shared_act]: contiguous except across the seam between the two buffers
                         const uint32_t routed = s0 < n ? min(sn, n - s0) : 0;
@@ -788,18 +921,21 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 const float g = gatev[t];
                 const float y = bf(bf(sum) + bf(g * otile[(n + t) * 16 + c]));
                 const uint64_t at = uint64_t(t) * H + rt * 16 + c;
-                st_f32(p.layer_out + at, y);
+                if constexpr (NT == 1) ZC_ST(p.tout + (layer & 1u) * H + at, (__float_as_uint(y) & 0xffff0000u) | tag);   // y is BF16-valued
+                else st_f32(p.layer_out + at, y);
                 if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * T * H + at, y);
                 if (layer + 1 == p.L) st_f32(p.out + at, y);
-                uint32_t m = __float_as_uint(y) & 0x7fffffffu;
-                if (m > 0x7f800000u) m = 0;   // NaN does not take part in the maximum
+                if constexpr (NT != 1) {   // one token: the next layer's staging finds the maximum itself
+                    uint32_t m = __float_as_uint(y) & 0x7fffffffu;
+                    if (m > 0x7f800000u) m = 0;   // NaN does not take part in the maximum
 #pragma unroll
-                for (int o = 8; o; o >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), o)));
-                if (c == 0) __hip_atomic_fetch_max(p.maxabs + layer * T + t, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int o = 8; o; o >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), o)));
+                    if (c == 0) __hip_atomic_fetch_max(p.maxabs + layer * T + t, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
         clock_all();
-        bar.wait();
+        if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the next layer polls the output words themselves
         clock();
     }
 }

@@ -66,6 +66,10 @@ struct DecodeParams {
     const float* x_in; float* out;   // [T][H]
     float *logits, *gate, *shared_act, *act, *layer_out;   // exchange buffers
     uint32_t* maxabs;                // [L][T] bit patterns of max |layer output|
+    // One token: the exchange buffers carry a tag beside every value, so that a reader polls the data itself instead of
+    // waiting at a grid barrier and fetching afterwards.  tlogits [E + 1] words {fp32 bits, tag << 32} (word E: the shared
+    // gate dot); tact [topk + 1][I] and tout [2][H] words {BF16 value << 16 | 16-bit tag}.  All zero before the first launch.
+    unsigned long long* tlogits; uint32_t *tact, *tout;
     int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][T][topk], [L][T][topk], [L][T][H]
     uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
     unsigned long long* clocks;      // optional [L * kDecodeStamps][workgroups] 100 MHz timestamps, one per workgroup

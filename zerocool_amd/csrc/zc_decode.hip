@@ -770,6 +770,63 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         if constexpr (NT == 1) { if (wg >= H / 16) bar.arrive(); }
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
             const uint32_t row = rt * 16 + col;
+            if (NT == 1 && SB >= slots_total) {
+                // One token, all slots' images resident: every wave works alone.  It requests the first weights of its slot's
+                // tile, then polls that slot's activations (one 16-element block per lane), builds the slot's image and the
+                // BF16 copy under the latency of those loads, and runs the tile; no workgroup barrier until the combine, and
+                // a wave starts as soon as its own slot is complete.
+                __syncthreads();
+                clock(); clock();
+                uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
+                for (uint32_t slot = wave; slot <= k; slot += kDecodeWaves) {   // slot k is the shared expert's
+                    const uint8_t* rec = L.shared_record; const uint64_t* off = p.so;
+                    if (slot < k) {
+                        const int32_t e = uniform(ids[slot]);
+                        if (e < 0 || e >= int32_t(E)) continue;
+                        rec = L.records + uint64_t(e) * L.stride; off = p.ro;
+                    }
+                    const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
+                    uint8_t* image = lds + lp.img_d + slot * LI.bytes();
+                    uint16_t* copy_row = ah + slot * I;
+                    auto wave_sync = [&]() {   // LDS traffic of this wave's lanes, in program order
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    };
+                    auto prologue = [&]() {
+                        if (lane < LI.mask_bytes() / 4) reinterpret_cast<uint32_t*>(image + LI.planes_bytes() + LI.info_bytes())[lane] = 0;
+                        if (lane < 4) reinterpret_cast<uint32_t*>(image + LI.blocks() * 48)[lane] = 0;
+                        wave_sync();
+                        for (uint32_t b = lane; b < I / 16; b += 64) {
+                            const uint64_t* words = reinterpret_cast<const uint64_t*>(p.tact + uint64_t(slot) * I + b * 16);
+                            uint64_t w[8];
+                            bar.until([&]() {
+                                uint32_t bad = 0;
+#pragma unroll
+                                for (int i = 0; i < 8; ++i) w[i] = ZC_LD(words + i);
+#pragma unroll
+                                for (int i = 0; i < 8; ++i) bad |= ((uint32_t(w[i]) ^ tag) | (uint32_t(w[i] >> 32) ^ tag)) & 0xffffu;
+                                return bad == 0;
+                            });
+                            RegF32 piece;
+                            uint32_t* copy = reinterpret_cast<uint32_t*>(copy_row + b * 16);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+                                const uint32_t lo = uint32_t(w[i]) & 0xffff0000u, hi = uint32_t(w[i] >> 32) & 0xffff0000u;
+                                piece.bits[2 * i] = lo; piece.bits[2 * i + 1] = hi;
+                                copy[i] = (lo >> 16) | hi;
+                            }
+                            xint_prepare_block(piece, LI, image, b);
+                        }
+                        wave_sync();
+                    };
+                    const uint8_t* img[PT] = {image}; LdsBf16 src[PT] = {LdsBf16{copy_row}};
+                    auto emit = [&](int, float v) { if (G == 0) otile[slot * 16 + col] = bf(v); };
+                    xint_run_tile_after<PT, 4>(w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit, prologue);
+                }
+            } else
             for (uint32_t s0 = 0; s0 < slots_total; s0 += SB) {
                 const uint32_t sn = min(SB, slots_total - s0);
                 __syncthreads();
@@ -897,6 +954,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
             __syncthreads();
+            if (NT == 1 && SB >= slots_total && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
             clock();
             // weighted combine of the tile (reference: qwen.metal:804-816)
             if (tid < T * 16) {

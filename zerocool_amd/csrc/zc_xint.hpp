@@ -223,10 +223,13 @@ __device__ __forceinline__ float xint_literal_dot(const v4i codes, const Source 
 //   1. every span: A operands from LDS, two MFMAs, digit sums -> fp32 block dots
 //   2. only if some block of the body is unsafe: those dots again by the literal chain
 //   3. every span: acc += scale*dot + sum*bias, in span order
-template <int PT, int R, class Source, class Emit>
-__device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
-                                              const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,
-                                              int nt, Emit emit) {
+//
+// prologue() runs once the first ring of weights has been requested and before anything is read from the images: a caller
+// whose images are not built yet builds them there, under the latency of those loads.
+template <int PT, int R, class Source, class Emit, class Prologue>
+__device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                                    const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,
+                                                    int nt, Emit emit, Prologue prologue) {
     static_assert(R == 8 || R == 4, "bodies of eight or four spans; spans must be a multiple of R");
     const uint32_t G = lane >> 4, row_a = lane & 15u, c_a = row_a >> 2, p_a = row_a & 3u;
     const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
@@ -247,6 +250,7 @@ __device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16
     const uint32_t M = 0x0f0f0f0fu;
     const v4i zero = {0, 0, 0, 0};
     auto expand = [&](uint32_t lo, uint32_t hi) { const v4i r = {int(lo & M), int((lo >> 4) & M), int(hi & M), int((hi >> 4) & M)}; return r; };
+    prologue();
     for (uint32_t d0 = 0; d0 < spans; d0 += R) {
         uint4 codes[R]; uint32_t sd[R], bd[R];
 #pragma unroll
@@ -325,6 +329,13 @@ __device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16
         }
         emit(t, v[0] + v[1]);
     }
+}
+
+template <int PT, int R, class Source, class Emit>
+__device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                              const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,
+                                              int nt, Emit emit) {
+    xint_run_tile_after<PT, R>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit, []() {});
 }
 
 }  // namespace zc

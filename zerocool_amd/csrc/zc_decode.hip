@@ -281,6 +281,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };   // after the slowest wave of the workgroup
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
+    if (tid == 0) misc[10] = 0;   // the router chain's hand-off word: no tag is 0
     // SwiGLU of a finished gate/up tile (gate rows in columns 0-7, up rows in 8-15), stored as packed BF16 pairs:
     // the lane of an even row writes rows r and r+1 of activation row `slot_row` as one word.
     auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {
@@ -335,9 +336,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             // later router loads in flight (a load under a branch forces a full wait), and its two barriers order LDS traffic
             // only.  The other workgroups have no router loads to keep in flight and fetch only what they need.
             const bool keep_in_flight = uniform(segmented && wg < (E + 3) / 4);
+            // In such a workgroup the staging threads are the waves after the router's: those build the image while the router
+            // waves already run their chains, which need the BF16 copy only.
+            const bool side = keep_in_flight && 64 * router_segments + H / 16 <= kDecodeThreads;
+            const uint32_t blk = side ? tid - 64 * router_segments : tid;   // the thread's block; wraps to "none" for the router's waves
             uint64_t v[8];
             uint4 gate_piece = make_uint4(0, 0, 0, 0);
-            const uint32_t own = min(tid, H / 16 - 1);
+            const uint32_t own = min(blk, H / 16 - 1);
             // the flag of workgroup `tid` (all have finished reading what the previous layer exchanged), checked below
             uint32_t seen = ZC_LD(p.sync + kFlagStride * min(tid, nwg - 1));
             auto stale = [&]() {
@@ -346,7 +351,21 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 for (int w = 0; w < 8; ++w) bad |= ((uint32_t(v[w]) ^ want) | (uint32_t(v[w] >> 32) ^ want)) & 0xffffu;
                 return bad != 0;
             };
-            if (keep_in_flight) {
+            if (side) {
+                // the router's waves request their weights and nothing else; the staging waves fetch the input and nothing
+                // else (this workgroup never reads the shared gate row)
+#pragma unroll
+                for (int w = 0; w < 8; ++w) v[w] = 0;
+                if (wave < router_segments) {
+                    const uint32_t e = wg * 4 + lane / 16, split = lane % 16, P = H / 16;
+                    const uint16_t* wr = L.router + uint64_t(e < E ? e : E - 1) * H + split * P;
+#pragma unroll
+                    for (int i = 0; i < kRing; ++i) early[i] = ldg_u4(wr, wave * kRing + i);
+                } else if (blk < H / 16) {
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + blk * 8 + w);
+                }
+            } else if (keep_in_flight) {
 #pragma unroll
                 for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + own * 8 + w);
                 gate_piece = ldg_u4(L.shared_gate, min(tid, H / 8 - 1));
@@ -372,7 +391,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
             if (glue) {
-                if (tid < H / 16 && stale())
+                if (blk < H / 16 && stale())
                     bar.until([&]() {
 #pragma unroll
                         for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + own * 8 + w);
@@ -385,7 +404,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
                 // largest magnitude of the row (NaN takes no part): per wave here, across the waves after the barrier
                 uint32_t m = 0;
-                if (tid < H / 16) {
+                if (blk < H / 16) {
 #pragma unroll
                     for (int w = 0; w < 8; ++w) {
                         const uint32_t a = uint32_t(v[w]) & 0x7fff0000u, c = uint32_t(v[w] >> 32) & 0x7fff0000u;
@@ -397,7 +416,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             }
             xint_prepare_begin(LH, lds + lp.img_rg, 1);
             if (keep_in_flight) lds_barrier(); else __syncthreads();
-            if (tid < H / 16) {
+            if (blk < H / 16) {
                 uint32_t peak = 0;
                 if (glue) {
 #pragma unroll
@@ -416,12 +435,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     packed[w] = (ua >> 16) | (uc & 0xffff0000u);
                 }
                 if (low) atomicOr(p.status, 4);   // inputs must be BF16-valued
-                uint4* copy = reinterpret_cast<uint4*>(xh + tid * 16);
+                uint4* copy = reinterpret_cast<uint4*>(xh + blk * 16);
                 copy[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]); copy[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
-                xint_prepare_block(block, LH, lds + lp.img_rg, tid);
+                if (!side) xint_prepare_block(block, LH, lds + lp.img_rg, blk);
             }
             if (tid < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid] = gate_piece;
             lds_barrier();
+            if (side && blk < H / 16) xint_prepare_block(LdsBf16{xh}, LH, lds + lp.img_rg, blk);   // from the BF16 copy, beside the router's waves; the tiles come after a barrier
         } else {
             {
                 uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
@@ -474,36 +494,44 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             const uint32_t router_units = (E + 3) / 4, shared_units = NT == 1 ? 0 : I / 8, gate_units = (T + 1) / 2;
             const uint32_t units = router_units + shared_units + gate_units;
             if (segmented) {
-                float* handoff = reinterpret_cast<float*>(experts);   // 64 chain values; the expert list is not in use yet
+                float* handoff = reinterpret_cast<float*>(lds + lp.gprod);   // 64 chain values; the products table belongs to another workgroup
                 if (wg < router_units) {
                     const uint32_t e = wg * 4 + lane / 16, split = lane % 16, P = H / 16;
                     float c = 0;
-                    for (uint32_t seg = 0; seg < router_segments; ++seg) {
-                        if (wave == seg) {
-                            if (seg) c = handoff[lane];
-                            uint4 xv[kRing];
+                    // the chain value passes from one wave to the next through LDS with a flag word of its own: the other
+                    // waves of the workgroup are busy with the image and do not come to a barrier here
+                    if (wave < router_segments) {
+                        const uint32_t seg = wave;
+                        if (seg) {
+                            for (uint32_t i = 0; uint32_t(__hip_atomic_load(misc + 10, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != tag * 4 + seg && i < (1u << 22); ++i)
+                                __builtin_amdgcn_s_sleep(1);
+                            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                            c = handoff[lane];
+                        }
+                        uint4 xv[kRing];
 #pragma unroll
-                            for (int j = 0; j < kRing; ++j) xv[j] = *reinterpret_cast<const uint4*>(xh_all + split * P + (seg * kRing + j) * 8);
+                        for (int j = 0; j < kRing; ++j) xv[j] = *reinterpret_cast<const uint4*>(xh_all + split * P + (seg * kRing + j) * 8);
 #pragma unroll
-                            for (int j = 0; j < kRing; ++j) {
-                                const uint32_t xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {early[j].x, early[j].y, early[j].z, early[j].w};
+                        for (int j = 0; j < kRing; ++j) {
+                            const uint32_t xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {early[j].x, early[j].y, early[j].z, early[j].w};
 #pragma unroll
-                                for (int q = 0; q < 4; ++q) {
-                                    c = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c);
-                                    c = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c);
-                                }
-                            }
-                            if (seg + 1 < router_segments) handoff[lane] = c;
-                            else {
-                                // partials added 0..15: after step s the lane of partition i <= s holds ((c0 + c1) + ..) + ci
-                                const float offset = (L.offsets && e < E) ? ldg_f32(L.offsets, e) : 0.0f;
-                                float sum = 0.0f + c;
-#pragma unroll
-                                for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c;
-                                if (split == 15 && e < E) st_logit(e, L.offsets ? sum + offset : sum);
+                            for (int q = 0; q < 4; ++q) {
+                                c = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c);
+                                c = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c);
                             }
                         }
-                        if (seg + 1 < router_segments) __syncthreads();
+                        if (seg + 1 < router_segments) {
+                            handoff[lane] = c;
+                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                            if (lane == 0) __hip_atomic_store(misc + 10, int32_t(tag * 4 + seg + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        } else {
+                            // partials added 0..15: after step s the lane of partition i <= s holds ((c0 + c1) + ..) + ci
+                            const float offset = (L.offsets && e < E) ? ldg_f32(L.offsets, e) : 0.0f;
+                            float sum = 0.0f + c;
+#pragma unroll
+                            for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c;
+                            if (split == 15 && e < E) st_logit(e, L.offsets ? sum + offset : sum);
+                        }
                     }
                 } else if (wg == router_units) {
                     // shared_expert_gate (qwen.metal:499-506): reference lane l adds the products of k = l, l + 32, ... in turn

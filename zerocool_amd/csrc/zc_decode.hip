@@ -148,10 +148,11 @@ __device__ __forceinline__ void stage_copy(const uint64_t* src, uint32_t count, 
 // equal value and lower id.  More than 64 candidates (masses of equal logits) or fewer than k valid lanes take the
 // picks one by one as before.
 //
-// fetch(cand, per) fills the lane's logits (-inf where it has no expert).
-template <int PER, class Fetch, class Clock>
+// fetch(cand, per) fills the lane's logits (-inf where it has no expert); ready() runs once the ids are final, before the
+// softmax weights are formed.
+template <int PER, class Fetch, class Clock, class Ready>
 __device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t topk, uint32_t lane,
-                                            int32_t* ids, float* weights, uint32_t* scratch, Clock clock) {
+                                            int32_t* ids, float* weights, uint32_t* scratch, Clock clock, Ready ready) {
     const uint32_t per = PER == 16 ? (E + 63) / 64 : uint32_t(PER);
     const float ninf = __uint_as_float(0xff800000u);
     float cand[PER];
@@ -239,6 +240,7 @@ __device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t to
         if (j == 0) top = value;
         if (lane == 0) ids[j] = found ? int32_t(winner) : -1;
     }
+    ready();
     clock();
     // softmax over the selected: reference lane l sums values 4l..4l+3 (qwen.metal:758-764)
     const float v = lane < topk ? exp32(score - top) : 0.0f;
@@ -281,7 +283,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };   // after the slowest wave of the workgroup
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
-    if (tid == 0) misc[10] = 0;   // the router chain's hand-off word: no tag is 0
+    if (tid == 0) { misc[10] = 0; misc[11] = 0; }   // the router chain's hand-off word and the ids-ready word: no tag is 0
     // SwiGLU of a finished gate/up tile (gate rows in columns 0-7, up rows in 8-15), stored as packed BF16 pairs:
     // the lane of an even row writes rows r and r+1 of activation row `slot_row` as one word.
     auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {
@@ -694,21 +696,28 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     }
                 }
             };
-            if (E == 512) route_token<8>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
-            else route_token<16>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp);
+            // One token: the other waves wait for the ids only (a flag word in LDS), not for the softmax weights, which the
+            // combine needs much later; the routing wave takes its tiles last.
+            auto ready = [&]() {
+                if constexpr (NT == 1) {
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                    if (lane == 0) __hip_atomic_store(misc + 11, int32_t(tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            };
+            if (E == 512) route_token<8>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp, ready);
+            else route_token<16>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp, ready);
         }
-        // the combine's gate factor, ready early
         if constexpr (NT == 1) {
-            if (tid == 64) {   // a wave that does not route
-                uint64_t w = 0;
-                bar.until([&]() { w = ZC_LD(p.tlogits + E); return uint32_t(w >> 32) == tag; });
-                gatev[0] = bf(sigmoid_bf(__uint_as_float(uint32_t(w))));
+            if (wave != 0) {
+                for (uint32_t i = 0; uint32_t(__hip_atomic_load(misc + 11, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != tag && i < (1u << 22); ++i)
+                    __builtin_amdgcn_s_sleep(1);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
             }
         } else {
-            if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));
+            if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
+            for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
+            __syncthreads();
         }
-        if constexpr (NT != 1) for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
-        __syncthreads();
         clock();
         if (tid < n) {
             const int32_t e = ids[tid];
@@ -744,7 +753,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             // the shared expert's gate/up tiles close the list (slot k): with 1280 routed tiles on 256 workgroups they land on
             // waves that have no routed tile
             const uint32_t tiles = I / 8, units = (k + 1) * tiles;
-            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
+            const uint32_t turn = (wave + kDecodeWaves - 1) % kDecodeWaves;   // the routing wave, still busy with the softmax, comes last
+            for (uint32_t u = wg + nwg * turn; u < units; u += nwg * kDecodeWaves) {
                 const uint32_t slot = u / tiles, tile = u % tiles;
                 const int32_t e = slot < k ? uniform(ids[slot]) : 0;
                 if (e < 0 || e >= int32_t(E)) continue;   // reported above; the combine drops the slot
@@ -762,6 +772,11 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     if (lane < 8) ZC_ST(p.tact + uint64_t(slot) * I + row, (a & 0xffff0000u) | tag);
                 };
                 ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
+            }
+            if (tid == 64) {   // the combine's gate factor (written by another workgroup)
+                uint64_t w = 0;
+                bar.until([&]() { w = ZC_LD(p.tlogits + E); return uint32_t(w >> 32) == tag; });
+                gatev[0] = bf(sigmoid_bf(__uint_as_float(uint32_t(w))));
             }
         } else {
             const uint32_t tiles = I / 8, units = U * tiles;

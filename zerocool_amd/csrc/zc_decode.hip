@@ -813,8 +813,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         if constexpr (NT == 1) { if (wg >= H / 16) bar.arrive(); }
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
             const uint32_t row = rt * 16 + col;
-            if (NT == 1 && SB >= slots_total) {
-                // One token, all slots' images resident: every wave works alone.  It requests the first weights of its slot's
+            if (NT == 1 && SB >= slots_total && I == 1024) {
+                // One token, all slots' images resident, tiles of two bodies (intermediate 1024): every wave works alone.  It requests the first weights of its slot's
                 // tile, then polls that slot's activations (one 16-element block per lane), builds the slot's image and the
                 // BF16 copy under the latency of those loads, and runs the tile; no workgroup barrier until the combine, and
                 // a wave starts as soon as its own slot is complete.
@@ -853,21 +853,18 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                                 for (int i = 0; i < 8; ++i) bad |= ((uint32_t(w[i]) ^ tag) | (uint32_t(w[i] >> 32) ^ tag)) & 0xffffu;
                                 return bad == 0;
                             });
-                            RegF32 piece;
-                            uint32_t* copy = reinterpret_cast<uint32_t*>(copy_row + b * 16);
+                            uint4* copy = reinterpret_cast<uint4*>(copy_row + b * 16);
+                            uint32_t packed[8];
 #pragma unroll
-                            for (int i = 0; i < 8; ++i) {
-                                const uint32_t lo = uint32_t(w[i]) & 0xffff0000u, hi = uint32_t(w[i] >> 32) & 0xffff0000u;
-                                piece.bits[2 * i] = lo; piece.bits[2 * i + 1] = hi;
-                                copy[i] = (lo >> 16) | hi;
-                            }
-                            xint_prepare_block(piece, LI, image, b);
+                            for (int i = 0; i < 8; ++i) packed[i] = (uint32_t(w[i]) >> 16) | (uint32_t(w[i] >> 32) & 0xffff0000u);
+                            copy[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]); copy[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
+                            xint_prepare_block(LdsBf16{copy_row}, LI, image, b);   // from the copy just written: fewer registers held
                         }
                         wave_sync();
                     };
                     const uint8_t* img[PT] = {image}; LdsBf16 src[PT] = {LdsBf16{copy_row}};
                     auto emit = [&](int, float v) { if (G == 0) otile[slot * 16 + col] = bf(v); };
-                    xint_run_tile_after<PT, 4>(w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit, prologue);
+                    xint_run_tile_after<PT, 4, true>(w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit, prologue);   // two bodies: both requested at once
                 }
             } else
             for (uint32_t s0 = 0; s0 < slots_total; s0 += SB) {
@@ -997,7 +994,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
             __syncthreads();
-            if (NT == 1 && SB >= slots_total && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
+            if (NT == 1 && SB >= slots_total && I == 1024 && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
             clock();
             // weighted combine of the tile (reference: qwen.metal:804-816)
             if (tid < T * 16) {

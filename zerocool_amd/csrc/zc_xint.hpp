@@ -226,7 +226,10 @@ __device__ __forceinline__ float xint_literal_dot(const v4i codes, const Source 
 //
 // prologue() runs once the first ring of weights has been requested and before anything is read from the images: a caller
 // whose images are not built yet builds them there, under the latency of those loads.
-template <int PT, int R, class Source, class Emit, class Prologue>
+//
+// PAIR: the tile has exactly two bodies (spans == 2 R) and both are requested before the prologue, each into registers of
+// its own: the second body then does not wait for a memory latency of its own either.
+template <int PT, int R, bool PAIR = false, class Source, class Emit, class Prologue>
 __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
                                                     const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,
                                                     int nt, Emit emit, Prologue prologue) {
@@ -238,6 +241,11 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
     for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
 #pragma unroll
     for (int q = 0; q < R / 4; ++q) { sring[q] = ldg_u4(s_row, q); bring[q] = ldg_u4(b_row, q); }
+    uint4 ring2[PAIR ? R : 1], sring2[PAIR ? R / 4 : 1], bring2[PAIR ? R / 4 : 1];
+    if constexpr (PAIR) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) ring2[j] = ldg_u4(c, (R + j) * 4);
+    }
     float acc[PT][4][2];
 #pragma unroll
     for (int t = 0; t < PT; ++t)
@@ -251,21 +259,8 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
     const v4i zero = {0, 0, 0, 0};
     auto expand = [&](uint32_t lo, uint32_t hi) { const v4i r = {int(lo & M), int((lo >> 4) & M), int(hi & M), int((hi >> 4) & M)}; return r; };
     prologue();
-    for (uint32_t d0 = 0; d0 < spans; d0 += R) {
-        uint4 codes[R]; uint32_t sd[R], bd[R];
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
-            codes[j] = ring[j];
-            const uint4 sq = sring[j / 4], bq = bring[j / 4];
-            sd[j] = (j % 4 == 0) ? sq.x : (j % 4 == 1) ? sq.y : (j % 4 == 2) ? sq.z : sq.w;
-            bd[j] = (j % 4 == 0) ? bq.x : (j % 4 == 1) ? bq.y : (j % 4 == 2) ? bq.z : bq.w;
-        }
-        if (d0 + R < spans) {
-#pragma unroll
-            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
-#pragma unroll
-            for (int q = 0; q < R / 4; ++q) { sring[q] = ldg_u4(s_row, (d0 + R) / 4 + q); bring[q] = ldg_u4(b_row, (d0 + R) / 4 + q); }
-        }
+    // one body: spans d0 .. d0 + R - 1 with their codes and scale / bias dwords
+    auto compute = [&](uint32_t d0, const uint4 (&codes)[R], const uint32_t (&sd)[R], const uint32_t (&bd)[R]) {
 #pragma unroll
         for (int t = 0; t < PT; ++t) {
             if (t >= nt) break;
@@ -312,6 +307,39 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
                 }
             }
         }
+    };
+    auto dwords = [&](const uint4 (&from)[R / 4], uint32_t (&to)[R]) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint4 q = from[j / 4];
+            to[j] = (j % 4 == 0) ? q.x : (j % 4 == 1) ? q.y : (j % 4 == 2) ? q.z : q.w;
+        }
+    };
+    if constexpr (PAIR) {
+        // the second body's scales and biases share cache lines with the first body's: requested late, they are close by
+#pragma unroll
+        for (int q = 0; q < R / 4; ++q) { sring2[q] = ldg_u4(s_row, R / 4 + q); bring2[q] = ldg_u4(b_row, R / 4 + q); }
+        uint32_t sd[R], bd[R];
+        dwords(sring, sd); dwords(bring, bd);
+        compute(0, ring, sd, bd);
+        if constexpr (R > 0) {   // (a scope of its own for the second body's dwords)
+            uint32_t sd2[R], bd2[R];
+            dwords(sring2, sd2); dwords(bring2, bd2);
+            compute(R, ring2, sd2, bd2);
+        }
+    } else
+    for (uint32_t d0 = 0; d0 < spans; d0 += R) {
+        uint4 codes[R]; uint32_t sd[R], bd[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) codes[j] = ring[j];
+        dwords(sring, sd); dwords(bring, bd);
+        if (d0 + R < spans) {
+#pragma unroll
+            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
+#pragma unroll
+            for (int q = 0; q < R / 4; ++q) { sring[q] = ldg_u4(s_row, (d0 + R) / 4 + q); bring[q] = ldg_u4(b_row, (d0 + R) / 4 + q); }
+        }
+        compute(d0, codes, sd, bd);
     }
     // Reference lane sum (xor butterfly 16, 8, 4, 2, 1): strides 16 and 8 pair accumulators,
     // 4 and 2 pair lane groups, 1 pairs the two blocks of a lane.

@@ -823,9 +823,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
                 for (uint32_t slot = wave; slot <= k; slot += kDecodeWaves) {   // slot k is the shared expert's
                     const uint8_t* rec = L.shared_record; const uint64_t* off = p.so;
+                    // what the combine adds up: the slot's output times its softmax weight (a dropped slot: zero times it),
+                    // the shared expert's output times the gate factor, rounded
+                    const float factor = slot < k ? weights[slot] : gatev[0];
                     if (slot < k) {
                         const int32_t e = uniform(ids[slot]);
-                        if (e < 0 || e >= int32_t(E)) continue;
+                        if (e < 0 || e >= int32_t(E)) { if (G == 0) otile[slot * 16 + col] = 0.0f * factor; continue; }
                         rec = L.records + uint64_t(e) * L.stride; off = p.ro;
                     }
                     const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
@@ -863,7 +866,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         wave_sync();
                     };
                     const uint8_t* img[PT] = {image}; LdsBf16 src[PT] = {LdsBf16{copy_row}};
-                    auto emit = [&](int, float v) { if (G == 0) otile[slot * 16 + col] = bf(v); };
+                    auto emit = [&](int, float v) { if (G == 0) otile[slot * 16 + col] = slot < k ? bf(v) * factor : bf(factor * bf(v)); };
                     xint_run_tile_after<PT, 4, true>(w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit, prologue);   // two bodies: both requested at once
                 }
             } else
@@ -1002,6 +1005,16 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 float partial[8];
 #pragma unroll
                 for (int q = 0; q < 8; ++q) partial[q] = 0;
+                const bool products = NT == 1 && SB >= slots_total && I == 1024;   // the waves left products, not outputs
+                if (products) {
+                    for (uint32_t base = 0; base < k; base += 8) {
+                        float value[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) value[j] = otile[min(base + j, k - 1) * 16 + c];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) if (base + j < k) partial[j] = base == 0 ? value[j] : partial[j] + value[j];
+                    }
+                } else
                 for (uint32_t base = 0; base < k; base += 8) {   // eight independent products at a time, partial j takes slots j, j+8, ...
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
@@ -1016,8 +1029,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
                 float sum = partial[0];
                 for (uint32_t kk = 1; kk < 8 && kk < k; ++kk) sum += partial[kk];
-                const float g = gatev[t];
-                const float y = bf(bf(sum) + bf(g * otile[(n + t) * 16 + c]));
+                const float y = bf(bf(sum) + (products ? otile[n * 16 + c] : bf(gatev[t] * otile[(n + t) * 16 + c])));
                 const uint64_t at = uint64_t(t) * H + rt * 16 + c;
                 if constexpr (NT == 1) ZC_ST(p.tout + (layer & 1u) * H + at, (__float_as_uint(y) & 0xffff0000u) | tag);   // y is BF16-valued
                 else st_f32(p.layer_out + at, y);

@@ -754,8 +754,16 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             // waves that have no routed tile
             const uint32_t tiles = I / 8, units = (k + 1) * tiles;
             const uint32_t turn = (wave + kDecodeWaves - 1) % kDecodeWaves;   // the routing wave, still busy with the softmax, comes last
-            for (uint32_t u = wg + nwg * turn; u < units; u += nwg * kDecodeWaves) {
-                const uint32_t slot = u / tiles, tile = u % tiles;
+            // With whole rounds of routed tiles the shared tiles (one more round, not a full one) go to the workgroups counted
+            // from the far end: the near end owns the router units and comes to the tiles last.
+            const bool far_end = (k * tiles) % nwg == 0 && tiles <= nwg;
+            for (uint32_t u = wg + nwg * turn; u < (far_end ? k * tiles + nwg : units); u += nwg * kDecodeWaves) {
+                uint32_t slot = u / tiles, tile = u % tiles;
+                if (far_end && u >= k * tiles) {
+                    const uint32_t s = nwg - 1 - wg;   // the shared tile of this workgroup, if it has one
+                    if (s >= tiles) continue;
+                    slot = k; tile = s;
+                }
                 const int32_t e = slot < k ? uniform(ids[slot]) : 0;
                 if (e < 0 || e >= int32_t(E)) continue;   // reported above; the combine drops the slot
                 const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;

@@ -1,9 +1,8 @@
 // Persistent decode kernel: a whole stack of MoE layers for a few tokens in ONE launch.
 //
-// One workgroup per compute unit stays resident for all layers.  A layer is three
-// phases separated by grid barriers:
-//   R  router logits (16-split chains), shared expert gate/up, shared-expert gate dot
-//   G  every workgroup routes (top-k + softmax) for itself, then the routed gate/up tiles
+// One workgroup per compute unit stays resident for all layers.  A layer is three phases:
+//   R  router logits (16-split chains), shared-expert gate dot
+//   G  every workgroup routes (top-k + softmax) for itself, then the gate/up tiles (routed and shared)
 //   D  routed + shared down tiles; a workgroup owns 16 output rows for ALL experts, so
 //      the weighted combine (moe_sum) runs inside it without another exchange
 // Arithmetic is the exact-integer matrix-core form (zc_xint.hpp) and the literal router /
@@ -11,8 +10,15 @@
 //
 // Cross-workgroup data (logits, activations, layer outputs) is written and read ONLY with
 // agent-scope relaxed atomics, which write through to / read from device-coherent
-// memory; barriers then need no cache write-back or invalidate, only wait counters.
+// memory; no cache write-back or invalidate is needed, only wait counters.
 // Weights are read with ordinary cached loads: nothing writes them.
+//
+// Several tokens (NT = 8) separate the phases with grid barriers (Barrier::wait).  One token (NT = 1) has none on its
+// path: every exchanged value carries a tag (a 16-bit number that advances with every layer of every launch) and its
+// reader polls the data itself until the tag is the expected one (Barrier::until); one flag per workgroup and layer,
+// stored without waiting and checked a layer later (Barrier::arrive), keeps a buffer from being overwritten before
+// every workgroup has read it.  Inside a workgroup, waves hand work on through flag words in LDS where a workgroup
+// barrier would make waves wait that have other work.
 //
 // Between layers the stacked-decode workload applies a stand-in glue (not reference
 // arithmetic): x_next = bf(y * (1 / max|y|)) per token, order independent.

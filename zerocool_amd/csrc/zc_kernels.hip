@@ -293,15 +293,17 @@ __global__ __launch_bounds__(256) void router_tiled_kernel(const uint16_t* w, co
             if (split == 0 && e0 + e < E && t0 + t < T) out[uint64_t(t0 + t) * E + e0 + e] = offsets ? sum + offsets[e0 + e] : sum;
         }
 }
-// Long batches with K a multiple of 512: a workgroup of 512 threads covers 32 tokens x 16 experts and stages 32 elements
-// of every K partition through LDS at a time (whole 128-byte lines of the inputs, read once per workgroup), so a token
+// Long batches with K a multiple of 256: a workgroup of 512 threads covers 32 tokens x 16 experts and stages 16 elements
+// of every K partition through LDS at a time (whole 64-byte pieces of the inputs, read once per workgroup), so a token
 // row is fetched from the L2 by 32 workgroups instead of 128.  Lane = (partition, token group, expert group) with a
-// 4 x 4 register tile as above; the chains still run k-ascending inside each partition.
-constexpr uint32_t kRouterXPitch = 36, kRouterWPitch = 20;   // words per (row, partition) piece: 32 fp32 + 4, 32 bf16 + 4 (conflict-free 16-/8-byte reads)
-__global__ __launch_bounds__(512) void router_block_kernel(const uint16_t* w, const float* x, uint32_t T, uint32_t K,
-                                                           uint32_t E, const float* offsets, float* out) {
-    __shared__ __align__(16) uint32_t xs[32 * 16 * kRouterXPitch];   // [token][partition][32 fp32]
-    __shared__ __align__(16) uint32_t ws[16 * 16 * kRouterWPitch];   // [expert][partition][32 bf16]
+// 4 x 4 register tile as above; the chains still run k-ascending inside each partition.  The chunk is small on purpose:
+// 52 KB of LDS and few registers let two or three workgroups share a compute unit and hide each other's load latency.
+constexpr uint32_t kRouterChunk = 16;
+constexpr uint32_t kRouterXPitch = 20, kRouterWPitch = 12;   // words per (row, partition) piece: 16 fp32 + 4, 16 bf16 + 4 (conflict-free 16-/8-byte reads)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void router_block_kernel(const uint16_t* w, const float* x, uint32_t T, uint32_t K,
+                                                              uint32_t E, const float* offsets, float* out) {
+    __shared__ __align__(16) uint32_t xs[32 * 16 * kRouterXPitch];   // [token][partition][16 fp32]
+    __shared__ __align__(16) uint32_t ws[16 * 16 * kRouterWPitch];   // [expert][partition][16 bf16]
     const uint32_t tid = threadIdx.x, split = tid % 16, pair = tid / 16, tg = pair % 8, eg = pair / 8;
     const uint32_t t0 = blockIdx.y * 32, e0 = blockIdx.x * 16, P = K / 16;
     float c[4][4];
@@ -309,33 +311,34 @@ __global__ __launch_bounds__(512) void router_block_kernel(const uint16_t* w, co
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int e = 0; e < 4; ++e) c[t][e] = 0;
-    // staging duty per chunk: 32 rows x 16 partitions x 8 sixteen-byte parts of x (8 per thread), 16 x 16 x 4 of w (2 per thread)
-    uint4 xr[8], wr[2];
+    // staging duty per chunk: 32 rows x 16 partitions x 4 sixteen-byte parts of x (4 per thread), 16 x 16 x 2 of w (1 per thread)
+    // staging registers as plain 32-bit words (arrays of the vector type end up in scratch memory here)
+    uint32_t xr[16], wr[4];
     auto fetch = [&](uint32_t chunk) {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const uint32_t piece = tid + q * 512, part = piece % 8, sp = (piece / 8) % 16, row = piece / 128;
-            xr[q] = *reinterpret_cast<const uint4*>(x + uint64_t(min(t0 + row, T - 1)) * K + sp * P + chunk * 32 + part * 4);
-        }
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
+        for (int q = 0; q < 4; ++q) {
             const uint32_t piece = tid + q * 512, part = piece % 4, sp = (piece / 4) % 16, row = piece / 64;
-            wr[q] = ldg_u4(w + uint64_t(min(e0 + row, E - 1)) * K + sp * P + chunk * 32 + part * 8);
+            const uint4 v = *reinterpret_cast<const uint4*>(x + uint64_t(min(t0 + row, T - 1)) * K + sp * P + chunk * kRouterChunk + part * 4);
+            xr[4 * q] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+        }
+        {
+            const uint32_t part = tid % 2, sp = (tid / 2) % 16, row = tid / 32;
+            const uint4 v = ldg_u4(w + uint64_t(min(e0 + row, E - 1)) * K + sp * P + chunk * kRouterChunk + part * 8);
+            wr[0] = v.x; wr[1] = v.y; wr[2] = v.z; wr[3] = v.w;
         }
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const uint32_t piece = tid + q * 512, part = piece % 8, sp = (piece / 8) % 16, row = piece / 128;
-            *reinterpret_cast<uint4*>(&xs[(row * 16 + sp) * kRouterXPitch + part * 4]) = xr[q];
-        }
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
+        for (int q = 0; q < 4; ++q) {
             const uint32_t piece = tid + q * 512, part = piece % 4, sp = (piece / 4) % 16, row = piece / 64;
-            *reinterpret_cast<uint4*>(&ws[(row * 16 + sp) * kRouterWPitch + part * 4]) = wr[q];
+            *reinterpret_cast<uint4*>(&xs[(row * 16 + sp) * kRouterXPitch + part * 4]) = make_uint4(xr[4 * q], xr[4 * q + 1], xr[4 * q + 2], xr[4 * q + 3]);
+        }
+        {
+            const uint32_t part = tid % 2, sp = (tid / 2) % 16, row = tid / 32;
+            *reinterpret_cast<uint4*>(&ws[(row * 16 + sp) * kRouterWPitch + part * 4]) = make_uint4(wr[0], wr[1], wr[2], wr[3]);
         }
     };
-    const uint32_t chunks = P / 32;
+    const uint32_t chunks = P / kRouterChunk;
     fetch(0);
     for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
         __syncthreads();            // the previous chunk has been consumed
@@ -343,7 +346,7 @@ __global__ __launch_bounds__(512) void router_block_kernel(const uint16_t* w, co
         __syncthreads();
         if (chunk + 1 < chunks) fetch(chunk + 1);
 #pragma unroll
-        for (int k = 0; k < 32; k += 4) {
+        for (int k = 0; k < int(kRouterChunk); k += 4) {
             float xv[4][4], wv[4][4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
@@ -377,7 +380,7 @@ __global__ __launch_bounds__(512) void router_block_kernel(const uint16_t* w, co
 }
 void launch_router(hipStream_t s, const void* w, const float* x, uint32_t T, uint32_t K, uint32_t E,
                    const float* offsets, float* out) {
-    if (T >= 256 && K % 512 == 0) {
+    if (T >= 256 && K % 256 == 0) {
         hipLaunchKernelGGL(router_block_kernel, dim3((E + 15) / 16, (T + 31) / 32), dim3(512), 0, s, (const uint16_t*)w, x, T, K, E, offsets, out);
         return;
     }

@@ -179,22 +179,39 @@ void launch_expert_phase(hipStream_t s, const ExpertPhaseDesc& d) {
 // ---------------------------------------------------------------------------
 // Plain (unquantised) rows: lane chain k = lane + 32 j (reference: qwen.metal:499-506)
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void plain_kernel(const void* w, uint32_t dtype, const float* x, uint32_t K,
-                                                    uint32_t N, uint32_t tokens, float* out, uint32_t float_output) {
-    const uint32_t lane = threadIdx.x & 31u, row = blockIdx.x * 8 + (threadIdx.x >> 5), t = blockIdx.y;
-    if (row >= N || t >= tokens) return;
+__global__ __launch_bounds__(256) void plain_kernel(const void* __restrict__ w, uint32_t dtype, const float* __restrict__ x, uint32_t K,
+                                                    uint32_t N, uint32_t tokens, float* __restrict__ out, uint32_t float_output) {
+    // one 32-lane group per (token, row) pair, eight pairs per workgroup whatever N is (a single row keeps all groups busy)
+    const uint32_t lane = threadIdx.x & 31u;
+    const uint64_t pair = uint64_t(blockIdx.x) * 8 + (threadIdx.x >> 5);
+    if (pair >= uint64_t(N) * tokens) return;
+    const uint32_t row = uint32_t(pair % N), t = uint32_t(pair / N);
+    const float* xr = x + uint64_t(t) * K;
     float sum = 0;
-    for (uint32_t k = lane; k < K; k += 32) {
+    uint32_t k = lane;
+    for (; k + 7 * 32 < K; k += 8 * 32) {   // eight loads of each operand in flight; the additions stay in k order
+        float xv[8], wv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            xv[j] = xr[k + 32 * j];
+            wv[j] = dtype == 1 ? reinterpret_cast<const float*>(w)[uint64_t(row) * K + k + 32 * j]
+                               : b16(reinterpret_cast<const uint16_t*>(w)[uint64_t(row) * K + k + 32 * j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sum += xv[j] * wv[j];
+    }
+    for (; k < K; k += 32) {
         const float wv = dtype == 1 ? reinterpret_cast<const float*>(w)[uint64_t(row) * K + k]
                                     : b16(reinterpret_cast<const uint16_t*>(w)[uint64_t(row) * K + k]);
-        sum += x[uint64_t(t) * K + k] * wv;
+        sum += xr[k] * wv;
     }
     sum = lane_sum32(sum);
     if (lane == 0) out[uint64_t(t) * N + row] = float_output ? sum : bf(sum);
 }
 void launch_plain(hipStream_t s, const void* w, uint32_t dtype, const float* x, uint32_t K, uint32_t N,
                   uint32_t tokens, float* out, bool float_output) {
-    hipLaunchKernelGGL(plain_kernel, dim3((N + 7) / 8, tokens), dim3(256), 0, s, w, dtype, x, K, N, tokens, out,
+    const uint64_t pairs = uint64_t(N) * tokens;
+    hipLaunchKernelGGL(plain_kernel, dim3(uint32_t((pairs + 7) / 8)), dim3(256), 0, s, w, dtype, x, K, N, tokens, out,
                        uint32_t(float_output));
 }
 
@@ -509,7 +526,7 @@ __global__ __launch_bounds__(1024) void dispatch_kernel(const int32_t* ids, uint
 }
 // The same sort for many slots (prefill), spread over the device: one wavefront per expert counts, one workgroup
 // scans, one wavefront per expert places.  offsets[1 + e] doubles as the count array between the first two steps.
-__global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* ids, uint32_t n, uint32_t E, int32_t* offsets, int32_t* status, bool aligned) {
+__global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* __restrict__ ids, uint32_t n, uint32_t E, int32_t* __restrict__ offsets, int32_t* status, bool aligned) {
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (blockIdx.x == 0) {
         int bad = 0;
@@ -518,7 +535,8 @@ __global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* ids,
     }
     if (e >= E) return;
     int32_t c = 0;
-    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // a lane looks at four neighbouring slots per step
+#pragma unroll 4
+    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // a lane looks at four neighbouring slots per step; four steps' loads in flight
         const uint32_t p = p0 + 4 * lane;
         int4 v = make_int4(-1, -1, -1, -1);
         if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array
@@ -547,14 +565,15 @@ __global__ __launch_bounds__(64) void dispatch_scan_kernel(uint32_t E, int32_t* 
     }
     if (lane == 0) *count = picked;
 }
-__global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* ids, uint32_t n, uint32_t topk, uint32_t E, const int32_t* offsets,
-                                                             int32_t* slots, int32_t* rows, bool aligned) {
+__global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* __restrict__ ids, uint32_t n, uint32_t topk, uint32_t E, const int32_t* __restrict__ offsets,
+                                                             int32_t* __restrict__ slots, int32_t* __restrict__ rows, bool aligned) {
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (e >= E) return;
     int32_t pos = offsets[e];
     if (offsets[e + 1] == pos) return;
     const uint64_t below = (1ull << lane) - 1;
-    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // four neighbouring slots per lane: slots of lower lanes come first, then the lane's own in order
+#pragma unroll 4
+    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // four neighbouring slots per lane (four steps' loads in flight): slots of lower lanes come first, then the lane's own in order
         const uint32_t p = p0 + 4 * lane;
         int4 v = make_int4(-1, -1, -1, -1);
         if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array

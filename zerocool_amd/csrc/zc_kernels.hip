@@ -535,8 +535,16 @@ __global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* __re
     }
     if (e >= E) return;
     int32_t c = 0;
-#pragma unroll 4
-    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // a lane looks at four neighbouring slots per step; four steps' loads in flight
+    uint32_t p0 = 0;
+    if (aligned)
+        for (; p0 + 8 * 256 <= n; p0 += 8 * 256) {   // eight steps' loads in flight
+            int4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const int4*>(ids + p0 + j * 256 + 4 * lane);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) c += (v[j].x == int32_t(e)) + (v[j].y == int32_t(e)) + (v[j].z == int32_t(e)) + (v[j].w == int32_t(e));
+        }
+    for (; p0 < n; p0 += 256) {   // a lane looks at four neighbouring slots per step
         const uint32_t p = p0 + 4 * lane;
         int4 v = make_int4(-1, -1, -1, -1);
         if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array
@@ -572,19 +580,29 @@ __global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* __re
     int32_t pos = offsets[e];
     if (offsets[e + 1] == pos) return;
     const uint64_t below = (1ull << lane) - 1;
-#pragma unroll 4
-    for (uint32_t p0 = 0; p0 < n; p0 += 256) {   // four neighbouring slots per lane (four steps' loads in flight): slots of lower lanes come first, then the lane's own in order
-        const uint32_t p = p0 + 4 * lane;
-        int4 v = make_int4(-1, -1, -1, -1);
-        if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array
-        else { if (p < n) v.x = ids[p]; if (p + 1 < n) v.y = ids[p + 1]; if (p + 2 < n) v.z = ids[p + 2]; if (p + 3 < n) v.w = ids[p + 3]; }
-        const bool m[4] = {v.x == int32_t(e), v.y == int32_t(e), v.z == int32_t(e), v.w == int32_t(e)};
-        const uint64_t mask[4] = {__ballot(m[0]), __ballot(m[1]), __ballot(m[2]), __ballot(m[3])};
-        int32_t at = pos + __popcll(mask[0] & below) + __popcll(mask[1] & below) + __popcll(mask[2] & below) + __popcll(mask[3] & below);
+    for (uint32_t q0 = 0; q0 < n; q0 += 8 * 256) {   // eight steps' loads in flight, then the steps in order
+        int4 ahead[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (m[j]) { slots[at] = int32_t(p + j); if (rows) rows[at] = int32_t((p + j) / topk); ++at; }
-        pos += __popcll(mask[0]) + __popcll(mask[1]) + __popcll(mask[2]) + __popcll(mask[3]);
+        for (int step = 0; step < 8; ++step) {
+            const uint32_t p = q0 + step * 256 + 4 * lane;
+            int4 v = make_int4(-1, -1, -1, -1);
+            if (aligned && p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);   // sixteen-byte loads only from a sixteen-byte aligned array
+            else { if (p < n) v.x = ids[p]; if (p + 1 < n) v.y = ids[p + 1]; if (p + 2 < n) v.z = ids[p + 2]; if (p + 3 < n) v.w = ids[p + 3]; }
+            ahead[step] = v;
+        }
+#pragma unroll
+        for (int step = 0; step < 8; ++step) {   // four neighbouring slots per lane: slots of lower lanes come first, then the lane's own in order
+            if (q0 + step * 256 >= n) break;
+            const uint32_t p = q0 + step * 256 + 4 * lane;
+            const int4 v = ahead[step];
+            const bool m[4] = {v.x == int32_t(e), v.y == int32_t(e), v.z == int32_t(e), v.w == int32_t(e)};
+            const uint64_t mask[4] = {__ballot(m[0]), __ballot(m[1]), __ballot(m[2]), __ballot(m[3])};
+            int32_t at = pos + __popcll(mask[0] & below) + __popcll(mask[1] & below) + __popcll(mask[2] & below) + __popcll(mask[3] & below);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (m[j]) { slots[at] = int32_t(p + j); if (rows) rows[at] = int32_t((p + j) / topk); ++at; }
+            pos += __popcll(mask[0]) + __popcll(mask[1]) + __popcll(mask[2]) + __popcll(mask[3]);
+        }
     }
 }
 void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets,

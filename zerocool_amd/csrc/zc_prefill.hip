@@ -240,18 +240,19 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 
 // Exact recomputation of the listed elements: one group of 32 lanes plays the reference's 32 lanes for one row
 // (qwen.metal:46-62: lane width 16 when K % 512 == 0 and N % 8 == 0, else 8; xor-butterfly lane sum).
+constexpr uint32_t kPatchWordsMax = 256;
 template <int WIDTH, bool GATED>
-__global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p) {
-    // each workgroup scans 256 words of the map, gathers the marked elements in LDS, then its eight 32-lane groups
-    // take them in turn
-    __shared__ uint16_t found[8192];
+__global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint32_t words_per_group) {
+    // each workgroup scans words_per_group words of the map (few for a small map, so that it still spreads over the chip),
+    // gathers the marked elements in LDS, then its eight 32-lane groups take them in turn
+    __shared__ uint16_t found[kPatchWordsMax * 32];
     __shared__ uint32_t found_count;
     const uint32_t lane = threadIdx.x & 31u;
     const uint32_t K = p.K, N = p.N, groups = K / 64;
-    const uint32_t word = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t word = blockIdx.x * words_per_group + threadIdx.x;
     if (threadIdx.x == 0) found_count = 0;
     __syncthreads();
-    uint32_t marks = word < p.near_words ? p.near_bits[word] : 0u;
+    uint32_t marks = (threadIdx.x < words_per_group && word < p.near_words) ? p.near_bits[word] : 0u;
     if (marks) {
         uint32_t at = atomicAdd(&found_count, uint32_t(__popc(marks)));
         while (marks) { found[at++] = uint16_t(threadIdx.x * 32 + (__ffs(marks) - 1)); marks &= marks - 1; }
@@ -259,39 +260,58 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p) {
     __syncthreads();
     const uint32_t listed = found_count;
   for (uint32_t item = threadIdx.x >> 5; item < listed; item += 8) {
-    const uint32_t code = blockIdx.x * 8192u + found[item], pos = code / N, n = code % N;
+    const uint32_t code = blockIdx.x * (words_per_group * 32u) + found[item], pos = code / N, n = code % N;
     const uint32_t expert = p.ids ? uint32_t(p.ids[p.slots[pos]]) : 0u;
     const uint8_t* record = p.records + uint64_t(expert) * p.stride;
     const uint32_t a_row = p.a_rows ? uint32_t(p.a_rows[pos]) / p.a_div : pos;
     const uint16_t* xr = p.a + uint64_t(a_row) * K;
-    constexpr int DW = WIDTH / 8;
+    constexpr int DW = WIDTH / 8, kAhead = 4;   // a lane's next four blocks are fetched together: one memory latency, not four
     float result[2] = {0, 0};
-    for (uint32_t b = lane; b < K / WIDTH; b += 32) {
-        float xb[WIDTH];
+    const uint32_t blocks = K / WIDTH;
+    for (uint32_t b0 = lane; b0 < blocks; b0 += 32 * kAhead) {
+        uint4 xv[kAhead][WIDTH / 8];
+        uint32_t words[kAhead][GATED ? 2 : 1][DW];
+        uint16_t scale_bits[kAhead][GATED ? 2 : 1], bias_bits[kAhead][GATED ? 2 : 1];
 #pragma unroll
-        for (int i = 0; i < WIDTH; i += 8) {
-            const uint4 v = *reinterpret_cast<const uint4*>(xr + b * WIDTH + i);
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        for (int u = 0; u < kAhead; ++u) {
+            const uint32_t b = min(b0 + 32u * u, blocks - 1);   // past the end: the last block again, not used
 #pragma unroll
-            for (int q = 0; q < 4; ++q) { xb[i + 2 * q] = __uint_as_float(w[q] << 16); xb[i + 2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
-        }
-        float sum = 0;
+            for (int i = 0; i < WIDTH / 8; ++i) xv[u][i] = *reinterpret_cast<const uint4*>(xr + b * WIDTH + 8 * i);
+            const uint32_t g = n * groups + (b * WIDTH) / 64;
 #pragma unroll
-        for (int i = 0; i < WIDTH; i += 4) sum += bf(bf(bf(xb[i] + xb[i + 1]) + xb[i + 2]) + xb[i + 3]);
-        const uint32_t g = n * groups + (b * WIDTH) / 64;
+            for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
+                const uint32_t* src = reinterpret_cast<const uint32_t*>(record + p.off[proj * 3] + uint64_t(n) * (K / 2)) + b * DW;
 #pragma unroll
-        for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
-            const uint32_t* words = reinterpret_cast<const uint32_t*>(record + p.off[proj * 3] + uint64_t(n) * (K / 2)) + b * DW;
-            float dot = 0;
-#pragma unroll
-            for (int i = 0; i < WIDTH; i += 4) {
-                const uint32_t packed = (words[i / 8] >> (4 * (i % 8))) & 0xffffu;
-                dot += xb[i] * float(packed & 15u) + xb[i + 1] * float((packed >> 4) & 15u) +
-                       xb[i + 2] * float((packed >> 8) & 15u) + xb[i + 3] * float((packed >> 12) & 15u);
+                for (int i = 0; i < DW; ++i) words[u][proj][i] = src[i];
+                scale_bits[u][proj] = reinterpret_cast<const uint16_t*>(record + p.off[proj * 3 + 1])[g];
+                bias_bits[u][proj] = reinterpret_cast<const uint16_t*>(record + p.off[proj * 3 + 2])[g];
             }
-            const float scale = b16(reinterpret_cast<const uint16_t*>(record + p.off[proj * 3 + 1])[g]);
-            const float bias = b16(reinterpret_cast<const uint16_t*>(record + p.off[proj * 3 + 2])[g]);
-            result[proj] += scale * dot + sum * bias;
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            if (b0 + 32u * u >= blocks) break;
+            float xb[WIDTH];
+#pragma unroll
+            for (int i = 0; i < WIDTH; i += 8) {
+                const uint4 v = xv[u][i / 8];
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) { xb[i + 2 * q] = __uint_as_float(w[q] << 16); xb[i + 2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
+            }
+            float sum = 0;
+#pragma unroll
+            for (int i = 0; i < WIDTH; i += 4) sum += bf(bf(bf(xb[i] + xb[i + 1]) + xb[i + 2]) + xb[i + 3]);
+#pragma unroll
+            for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
+                float dot = 0;
+#pragma unroll
+                for (int i = 0; i < WIDTH; i += 4) {
+                    const uint32_t packed = (words[u][proj][i / 8] >> (4 * (i % 8))) & 0xffffu;
+                    dot += xb[i] * float(packed & 15u) + xb[i + 1] * float((packed >> 4) & 15u) +
+                           xb[i + 2] * float((packed >> 8) & 15u) + xb[i + 3] * float((packed >> 12) & 15u);
+                }
+                result[proj] += b16(scale_bits[u][proj]) * dot + sum * b16(bias_bits[u][proj]);
+            }
         }
     }
     result[0] = lane_sum32(result[0]);
@@ -322,9 +342,10 @@ void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32
 }
 void launch_prefill_patch(hipStream_t s, const PrefillGemm& p, bool gated) {
     const bool wide = p.K % 512 == 0 && p.N % 8 == 0;     // the reference's lane-width rule (metal.mm:649-674)
-    const dim3 grid((p.near_words + 255) / 256);
-    if (gated) { if (wide) hipLaunchKernelGGL((prefill_patch_kernel<16, true>), grid, dim3(256), 0, s, p); else hipLaunchKernelGGL((prefill_patch_kernel<8, true>), grid, dim3(256), 0, s, p); }
-    else { if (wide) hipLaunchKernelGGL((prefill_patch_kernel<16, false>), grid, dim3(256), 0, s, p); else hipLaunchKernelGGL((prefill_patch_kernel<8, false>), grid, dim3(256), 0, s, p); }
+    const uint32_t per = p.near_words >= kPatchWordsMax * 1024u ? kPatchWordsMax : 64u;   // words of the map per workgroup
+    const dim3 grid((p.near_words + per - 1) / per);
+    if (gated) { if (wide) hipLaunchKernelGGL((prefill_patch_kernel<16, true>), grid, dim3(256), 0, s, p, per); else hipLaunchKernelGGL((prefill_patch_kernel<8, true>), grid, dim3(256), 0, s, p, per); }
+    else { if (wide) hipLaunchKernelGGL((prefill_patch_kernel<16, false>), grid, dim3(256), 0, s, p, per); else hipLaunchKernelGGL((prefill_patch_kernel<8, false>), grid, dim3(256), 0, s, p, per); }
 }
 bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts) { return hidden % 128 == 0 && inter % 128 == 0 && experts <= 1024; }
 

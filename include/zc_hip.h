@@ -206,6 +206,11 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* stack, const float*
                               float* out, const zc_stack_trace* trace, uint32_t flags);
 /* 1 if zc_hip_stack_decode would take the persistent single-launch path for `tokens`. */
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* stack, uint32_t tokens);
+/* Bound of every wait of the persistent kernel on another workgroup, in polls (0 restores the default, about four
+ * seconds' worth).  A wait that runs out makes the launch give up everywhere and zc_hip_moe_check report it; the stack
+ * stays usable.  No counterpart in the reference (its command buffers cannot wait on each other); tests use a bound of
+ * one poll to exercise the give-up path without a lost workgroup. */
+zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* stack, uint32_t polls);
 zc_status zc_hip_stack_glue(zc_hip_ctx* ctx, const float* y, uint32_t tokens, uint32_t hidden, float* x_next);
 
 /* ---- Expert store: ExpertStore + ExpertCache (include/engine/storage.hpp:168-269; src/engine/storage.cpp:493-725)

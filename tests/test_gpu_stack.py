@@ -188,3 +188,38 @@ def test_single_token_launches_across_the_tag_wrap(ctx):
             ctx.free(b)
     for b in (x1, x2, out1, out2):
         ctx.free(b)
+
+
+def test_a_wait_that_runs_out_is_reported_and_the_stack_stays_usable(ctx):
+    # Every wait of the persistent kernel on another workgroup is bounded.  With a bound of one poll some wait runs out
+    # in practically every launch: the launch then gives up everywhere, ends normally, and the check reports it.  With the
+    # default bound back, the same stack gives the right answer again.
+    cfg = workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512)
+    layers = [workload.LayerWeights(ctx, cfg, 501 + l, ("zipf", 1.1)) for l in range(4)]
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], 2)
+    out = {T: ctx.alloc(T * cfg.hidden * 4) for T in (1, 2)}
+    xs = {T: workload.hidden_rows(ctx, T, cfg.hidden, 30 + T) for T in (1, 2)}
+    want = {}
+    for T in (1, 2):
+        ctx.stack_decode(stack, xs[T], T, out[T]); ctx.moe_check()
+        want[T] = out[T].numpy(f32).tobytes()
+    for T in (1, 2):
+        ctx.stack_set_wait_limit(stack, 1)
+        reported = 0
+        for _ in range(5):
+            ctx.stack_decode(stack, xs[T], T, out[T])
+            try:
+                ctx.moe_check()
+            except z.ZcError as err:
+                assert "synchronise" in str(err)
+                reported += 1
+        assert reported > 0, "a one-poll bound never ran out"
+        ctx.stack_set_wait_limit(stack, 0)
+        ctx.stack_decode(stack, xs[T], T, out[T]); ctx.moe_check()
+        assert out[T].numpy(f32).tobytes() == want[T]
+    ctx.stack_destroy(stack)
+    for l in layers:
+        for b in (l.router, l.shared_gate, l.shared_record, l.records):
+            ctx.free(b)
+    for T in (1, 2):
+        ctx.free(out[T]); ctx.free(xs[T])

@@ -628,6 +628,7 @@ struct zc_hip_stack {
     uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
     unsigned long long* tlogits = nullptr; uint32_t *tact = nullptr, *tout = nullptr;   // tagged exchange buffers of the one-token kernel
     uint32_t epoch = 1u << 12;
+    uint32_t wait_limit = 1u << 22;   // polls before a wait on another workgroup gives up
     int cus = 0; uint32_t lds_limit = 0;
     bool persistent_ok = false;
     // layered path
@@ -723,6 +724,11 @@ static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, 
     (void)ctx;
     return per_cu >= 1;
 }
+zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t polls) {
+    ZC_REQUIRE(ctx && st, "null argument");
+    st->wait_limit = polls ? polls : 1u << 22;
+    return ZC_OK;
+}
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
     if (!ctx || !st) return 0;
     zc::DecodeLdsPlan plan; uint32_t nt;
@@ -752,7 +758,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
         if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
         p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
-        p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = 1u << 22;
+        p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
         st->epoch += 3 * L + 16;   // wraps modulo 2^32; the barrier compares epochs as signed differences
         const uint32_t workgroups = uint32_t(st->cus);
         ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));

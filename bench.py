@@ -23,7 +23,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 # HBM bytes per launch of the default workload (48 layers, batch 1) from the FETCH_SIZE / WRITE_SIZE counter runs summarised
 # in profiles/decode_stack_kernel_F48_batch1_pmc.txt (counters cannot be read from inside this process).
-MEASURED_TRAFFIC = 3_023_434_000
+MEASURED_TRAFFIC = 3_023_324_000
 sys.path.insert(0, ROOT)
 
 

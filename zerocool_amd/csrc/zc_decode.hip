@@ -714,7 +714,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             else route_token<16>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp, ready);
         }
         if constexpr (NT == 1) {
-            if (wave != 0) {
+            // the wave whose only tile is the shared expert's (see the tile list below) needs no ids: it starts at once
+            const bool shared_only = (k * (I / 8)) % nwg == 0 && I / 8 <= nwg && wave == k * (I / 8) / nwg + 1 && nwg - 1 - wg < I / 8;
+            if (wave != 0 && !shared_only) {
                 for (uint32_t i = 0; uint32_t(__hip_atomic_load(misc + 11, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != tag && i < (1u << 22); ++i)
                     __builtin_amdgcn_s_sleep(1);
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");

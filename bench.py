@@ -81,7 +81,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
-              "(DESIGN.md describes how it would shard by expert)", file=sys.stderr)
+              "(the design notes describe how the path would shard by expert)", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np

@@ -630,25 +630,47 @@ void launch_scatter(hipStream_t s, const float* x, const int32_t* positions, uin
 }
 // General top-k keeps the reference's eight strided partials: partial j takes
 // k = j, j+8, ...; partials are then added 0..7.  top-k 10 is the reference expression.
-__global__ void moe_sum_kernel(const float* experts, const float* weights, const float* shared, const float* gate,
-                               uint32_t T, uint32_t H, uint32_t topk, float* out) {
-    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+template <int V>
+__global__ __launch_bounds__(256) void moe_sum_kernel(const float* __restrict__ experts, const float* __restrict__ weights, const float* __restrict__ shared,
+                                                      const float* __restrict__ gate, uint32_t T, uint32_t H, uint32_t topk, float* __restrict__ out) {
+    // V neighbouring columns per thread (one 16-byte load per slot when V is 4); every column keeps the scalar arithmetic
+    typedef float row_t __attribute__((ext_vector_type(V)));
+    const uint32_t c = (blockIdx.x * blockDim.x + threadIdx.x) * V, t = blockIdx.y;
     if (c >= H || t >= T) return;
-    float partial[8];
+    row_t partial[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) partial[k] = 0;
+    for (int k = 0; k < 8; ++k) partial[k] = row_t(0);
+    if (topk == 10) {   // the reference's shape: all ten rows requested before the first is used
+        row_t value[10]; float weight[10];
+#pragma unroll
+        for (int k = 0; k < 10; ++k) { value[k] = *reinterpret_cast<const row_t*>(experts + (uint64_t(t) * 10 + k) * H + c); weight[k] = weights[uint64_t(t) * 10 + k]; }
+#pragma unroll
+        for (int k = 0; k < 10; ++k) {
+            const row_t product = value[k] * weight[k];
+            if (k < 8) partial[k] = product; else partial[k % 8] = partial[k % 8] + product;
+        }
+    } else
     for (uint32_t k = 0; k < topk; ++k) {
-        const float product = experts[(uint64_t(t) * topk + k) * H + c] * weights[uint64_t(t) * topk + k];
+        const row_t product = *reinterpret_cast<const row_t*>(experts + (uint64_t(t) * topk + k) * H + c) * weights[uint64_t(t) * topk + k];
         if (k < 8) partial[k] = product; else partial[k % 8] = partial[k % 8] + product;
     }
-    float sum = partial[0];
+    row_t sum = partial[0];
     for (uint32_t k = 1; k < 8 && k < topk; ++k) sum += partial[k];
     const float g = bf(sigmoid_bf(gate[t]));
-    out[uint64_t(t) * H + c] = bf(bf(sum) + bf(g * shared[uint64_t(t) * H + c]));
+    const row_t sh = *reinterpret_cast<const row_t*>(shared + uint64_t(t) * H + c);
+    row_t y;
+    if constexpr (V == 1) y = row_t(bf(bf(sum[0]) + bf(g * sh[0])));
+    else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) y[i] = bf(bf(sum[i]) + bf(g * sh[i]));
+    }
+    *reinterpret_cast<row_t*>(out + uint64_t(t) * H + c) = y;
 }
 void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, const float* shared, const float* gate,
                     uint32_t T, uint32_t H, uint32_t topk, float* out) {
-    hipLaunchKernelGGL(moe_sum_kernel, dim3((H + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
+    const bool wide = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(experts) | reinterpret_cast<uintptr_t>(shared) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (wide) hipLaunchKernelGGL(moe_sum_kernel<4>, dim3((H / 4 + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
+    else hipLaunchKernelGGL(moe_sum_kernel<1>, dim3((H + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
 }
 // Stand-in glue between stacked layers: x_next = bf(y * (1 / max|y|)) per token.
 __global__ __launch_bounds__(256) void stack_glue_kernel(const float* y, uint32_t H, float* out) {

@@ -192,7 +192,8 @@ def test_moe_sum_midpoint_and_random(ctx):  # :827-842
     out = ctx.moe_sum(ctx.upload(e), ctx.upload(w), ctx.upload(shared), ctx.upload(gate), 1, H).numpy(f32)
     assert out[0] == m["expected"] and (out[1:] == 0).all()
     rng = np.random.default_rng(2)
-    for T, Hh, k in ((5, 2048, 10), (3, 3072, 10), (4, 256, 4)):
+    # widths that are and are not a multiple of four (four columns per thread or one), top-k at, below and above ten
+    for T, Hh, k in ((5, 2048, 10), (3, 3072, 10), (4, 256, 4), (2, 250, 10), (2, 252, 12), (3, 1028, 10), (1, 17, 3)):
         e = oracle.bf(rng.standard_normal((T * k, Hh))); w = rng.random((T, k)).astype(f32)
         sh = oracle.bf(rng.standard_normal((T, Hh))); g = oracle.bf(rng.standard_normal(T) * 2)
         got = ctx.moe_sum(ctx.upload(e), ctx.upload(w), ctx.upload(sh), ctx.upload(g), T, Hh, k).numpy(f32)

@@ -13,7 +13,7 @@ f32 = np.float32
 
 
 def bits(x):
-    return int(np.array(x, dtype=np.float32).view(np.uint32))
+    return int(np.asarray(x, dtype=np.float32).reshape(-1)[:1].view(np.uint32)[0])
 
 
 def test_bf16_rounding():  # :277-283 and storage.cpp:30-35

@@ -478,7 +478,7 @@ zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
 namespace {
 struct PrefillSpace {
     Workspace base;
-    uint16_t *xb, *actb, *sactb; float *xsum, *asum, *ssum;
+    uint16_t *xb, *actb, *sactb; float *xsum, *asum, *ssum, *xsum16, *asum16, *ssum16;
     int32_t *tile_expert, *tile_first, *tile_rows, *tile_count, *stile_expert, *stile_first, *stile_rows, *stile_count;
     uint32_t max_tiles, max_shared_tiles;
     uint32_t* near_bits;      // one bit per product element: recompute exactly
@@ -499,6 +499,8 @@ PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
     w.stile_expert = (int32_t*)take(w.max_shared_tiles * 4ull); w.stile_first = (int32_t*)take(w.max_shared_tiles * 4ull);
     w.stile_rows = (int32_t*)take(w.max_shared_tiles * 4ull); w.stile_count = (int32_t*)take(4);
     w.near_bits = (uint32_t*)take(n * std::max(c->hidden, c->inter) / 8);
+    w.xsum16 = (float*)take(uint64_t(T) * (c->hidden / 16) * 4); w.asum16 = (float*)take(n * (c->inter / 16) * 4);
+    w.ssum16 = (float*)take(uint64_t(T) * (c->inter / 16) * 4);
     w.bytes = at;
     return w;
 }
@@ -534,7 +536,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
     // operands of the matrix cores: bf16 rows and their group sums; work lists
     const float margin = zc::kPrefillMargin;
-    zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, ctx->moe_status);
+    zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, w.xsum16, ctx->moe_status);
     zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
     zc::launch_prefill_tiles(s, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
     auto offsets_of = [&](const void* record, int shared, uint64_t* off, int first, int count) {
@@ -547,16 +549,16 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     };
     {   // routed gate/up + SwiGLU on gathered rows (pipeline.cpp:18-24), then down scattered to the slots (pipeline.cpp:25-29)
         zc::PrefillGemm g{};
-        g.a = w.xb; g.asum = w.xsum; g.a_rows = w.base.slots; g.a_div = k; g.out_rows = nullptr;
+        g.a = w.xb; g.asum = w.xsum; g.asum16 = w.xsum16; g.a_rows = w.base.slots; g.a_div = k; g.out_rows = nullptr;
         g.records = static_cast<const uint8_t*>(l->expert_records); g.stride = l->record_stride; offsets_of(l->expert_records, 0, g.off, 0, 2);
         g.tile_expert = w.tile_expert; g.tile_first = w.tile_first; g.tile_rows = w.tile_rows; g.tile_count = w.tile_count;
         g.K = H; g.N = I; g.out_b = w.actb;
         g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(n) * I / 32); g.near_margin = margin; g.ids = w.base.ids; g.slots = w.base.slots;
         zc::launch_prefill_gemm(s, g, true, w.max_tiles);
         zc::launch_prefill_patch(s, g, true);
-        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum);
+        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum, w.asum16);
         zc::PrefillGemm d{};
-        d.a = w.actb; d.asum = w.asum; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
+        d.a = w.actb; d.asum = w.asum; d.asum16 = w.asum16; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
         d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
         d.K = I; d.N = H; d.out_f = w.base.expert_out;
@@ -566,16 +568,16 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     }
     {   // shared expert (model.cpp:482-485): one group of all the tokens
         zc::PrefillGemm g{};
-        g.a = w.xb; g.asum = w.xsum; g.a_rows = nullptr; g.a_div = 1;
+        g.a = w.xb; g.asum = w.xsum; g.asum16 = w.xsum16; g.a_rows = nullptr; g.a_div = 1;
         g.records = static_cast<const uint8_t*>(l->shared_record); g.stride = 0; offsets_of(l->shared_record, 1, g.off, 0, 2);
         g.tile_expert = w.stile_expert; g.tile_first = w.stile_first; g.tile_rows = w.stile_rows; g.tile_count = w.stile_count;
         g.K = H; g.N = I; g.out_b = w.sactb;
         g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(T) * I / 32); g.near_margin = margin; g.ids = nullptr; g.slots = nullptr;
         zc::launch_prefill_gemm(s, g, true, w.max_shared_tiles);
         zc::launch_prefill_patch(s, g, true);
-        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum);
+        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum, w.ssum16);
         zc::PrefillGemm d{};
-        d.a = w.sactb; d.asum = w.ssum; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
+        d.a = w.sactb; d.asum = w.ssum; d.asum16 = w.ssum16; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
         d.records = g.records; d.stride = 0; offsets_of(l->shared_record, 1, d.off, 2, 1);
         d.tile_expert = w.stile_expert; d.tile_first = w.stile_first; d.tile_rows = w.stile_rows; d.tile_count = w.stile_count;
         d.K = I; d.N = H; d.out_f = w.base.shared;

@@ -88,6 +88,7 @@ constexpr uint32_t kDecodeSyncBytes = (32 * 1024 + 16 * 64) * 4;
 struct PrefillGemm {
     const uint16_t* a;        // bf16 rows [.][K]
     const float* asum;        // per (row, group of 64): sum of the blocks' BF16-rounded sum-of-four chains
+    const float* asum16;      // per (row, block of 16): that block's chain sum (read by the recomputation; null: formed there)
     const int32_t* a_rows;    // row of `a` for sorted position pos: a_rows ? a_rows[pos] / a_div : pos
     uint32_t a_div;
     const int32_t* out_rows;  // output row for sorted position pos: out_rows ? out_rows[pos] : pos   (down projection)
@@ -105,8 +106,8 @@ struct PrefillGemm {
     const int32_t* slots;
 };
 constexpr float kPrefillMargin = 0x1p-22f;  // of the summed term magnitudes: four fp32 steps at that scale
-void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status);
-void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums);
+void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status);
+void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16);
 void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
                           int32_t* tile_rows, int32_t* tile_count);
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles);

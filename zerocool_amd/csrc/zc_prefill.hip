@@ -31,7 +31,7 @@ constexpr uint32_t kTileRows = 32, kTileCols = 128, kPitch = 72;   // LDS row pi
 
 // fp32 rows holding BF16 values -> bf16 rows, plus per (row, group of 64) the sum of the four blocks' BF16-rounded
 // sum-of-four chains.  One thread per (row, group).  status bit 4: a value was not BF16-valued.
-__global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status) {
+__global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status) {
     const uint32_t groups = K / 64, i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= rows * groups) return;
     const uint32_t r = i / groups, g = i % groups;
@@ -51,6 +51,7 @@ __global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint3
             packed[2 * q] = (u0 >> 16) | (u1 & 0xffff0000u); packed[2 * q + 1] = (u2 >> 16) | (u3 & 0xffff0000u);
         }
         total += sum;
+        if (sums16) sums16[uint64_t(i) * 4 + b] = sum;
         uint4* dst = reinterpret_cast<uint4*>(xb + uint64_t(r) * K + g * 64 + b * 16);
         dst[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
         dst[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint3
     if (low) atomicOr(status, 4);
 }
 // The same sums for rows that are already bf16 (the SwiGLU activations).
-__global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums) {
+__global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16) {
     const uint32_t groups = K / 64, i = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t rows = rows_ptr ? min(uint32_t(*rows_ptr), rows_max) : rows_max;
     if (i >= rows * groups) return;
@@ -78,6 +79,7 @@ __global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, c
             sum += bf(bf(bf(a + c) + d) + e);
         }
         total += sum;
+        if (sums16) sums16[uint64_t(i) * 4 + b] = sum;
     }
     sums[i] = total;
 }
@@ -272,11 +274,16 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
         uint4 xv[kAhead][WIDTH / 8];
         uint32_t words[kAhead][GATED ? 2 : 1][DW];
         uint16_t scale_bits[kAhead][GATED ? 2 : 1], bias_bits[kAhead][GATED ? 2 : 1];
+        // the block's BF16-rounded chain sum depends on the row only: with 16-element blocks it comes from the table the
+        // row kernels left (the same additions in the same order)
+        const bool tabled = WIDTH == 16 && p.asum16;
+        float chain[kAhead];
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) {
             const uint32_t b = min(b0 + 32u * u, blocks - 1);   // past the end: the last block again, not used
 #pragma unroll
             for (int i = 0; i < WIDTH / 8; ++i) xv[u][i] = *reinterpret_cast<const uint4*>(xr + b * WIDTH + 8 * i);
+            chain[u] = tabled ? p.asum16[uint64_t(a_row) * (K / 16) + b] : 0.0f;
             const uint32_t g = n * groups + (b * WIDTH) / 64;
 #pragma unroll
             for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
@@ -298,9 +305,11 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
 #pragma unroll
                 for (int q = 0; q < 4; ++q) { xb[i + 2 * q] = __uint_as_float(w[q] << 16); xb[i + 2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
             }
-            float sum = 0;
+            float sum = chain[u];
+            if (!tabled) {
 #pragma unroll
-            for (int i = 0; i < WIDTH; i += 4) sum += bf(bf(bf(xb[i] + xb[i + 1]) + xb[i + 2]) + xb[i + 3]);
+                for (int i = 0; i < WIDTH; i += 4) sum += bf(bf(bf(xb[i] + xb[i + 1]) + xb[i + 2]) + xb[i + 3]);
+            }
 #pragma unroll
             for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
                 float dot = 0;
@@ -323,13 +332,13 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
   }
 }
 
-void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, int32_t* status) {
+void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status) {
     const uint32_t items = rows * (K / 64);
-    hipLaunchKernelGGL(prefill_rows_kernel, dim3((items + 255) / 256), dim3(256), 0, s, x, rows, K, xb, sums, status);
+    hipLaunchKernelGGL(prefill_rows_kernel, dim3((items + 255) / 256), dim3(256), 0, s, x, rows, K, xb, sums, sums16, status);
 }
-void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums) {
+void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16) {
     const uint32_t items = rows_max * (K / 64);
-    hipLaunchKernelGGL(prefill_sums_kernel, dim3((items + 255) / 256), dim3(256), 0, s, xb, rows_ptr, rows_max, K, sums);
+    hipLaunchKernelGGL(prefill_sums_kernel, dim3((items + 255) / 256), dim3(256), 0, s, xb, rows_ptr, rows_max, K, sums, sums16);
 }
 void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
                           int32_t* tile_rows, int32_t* tile_count) {

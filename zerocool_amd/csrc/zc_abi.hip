@@ -536,6 +536,8 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
     // operands of the matrix cores: bf16 rows and their group sums; work lists
     const float margin = zc::kPrefillMargin;
+    // the per-block chain sums pay where a lane of the recomputation has several blocks of a row (long rows); short rows form them in place
+    const bool table_inter = I / 16 >= 128;
     zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, w.xsum16, ctx->moe_status);
     zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
     zc::launch_prefill_tiles(s, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
@@ -556,9 +558,9 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(n) * I / 32); g.near_margin = margin; g.ids = w.base.ids; g.slots = w.base.slots;
         zc::launch_prefill_gemm(s, g, true, w.max_tiles);
         zc::launch_prefill_patch(s, g, true);
-        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum, w.asum16);
+        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum, table_inter ? w.asum16 : nullptr);
         zc::PrefillGemm d{};
-        d.a = w.actb; d.asum = w.asum; d.asum16 = w.asum16; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
+        d.a = w.actb; d.asum = w.asum; d.asum16 = table_inter ? w.asum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
         d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
         d.K = I; d.N = H; d.out_f = w.base.expert_out;
@@ -575,9 +577,9 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(T) * I / 32); g.near_margin = margin; g.ids = nullptr; g.slots = nullptr;
         zc::launch_prefill_gemm(s, g, true, w.max_shared_tiles);
         zc::launch_prefill_patch(s, g, true);
-        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum, w.ssum16);
+        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum, table_inter ? w.ssum16 : nullptr);
         zc::PrefillGemm d{};
-        d.a = w.sactb; d.asum = w.ssum; d.asum16 = w.ssum16; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
+        d.a = w.sactb; d.asum = w.ssum; d.asum16 = table_inter ? w.ssum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
         d.records = g.records; d.stride = 0; offsets_of(l->shared_record, 1, d.off, 2, 1);
         d.tile_expert = w.stile_expert; d.tile_first = w.stile_first; d.tile_rows = w.stile_rows; d.tile_count = w.stile_count;
         d.K = I; d.N = H; d.out_f = w.base.shared;

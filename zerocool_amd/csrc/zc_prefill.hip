@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 // Exact recomputation of the listed elements: one group of 32 lanes plays the reference's 32 lanes for one row
 // (qwen.metal:46-62: lane width 16 when K % 512 == 0 and N % 8 == 0, else 8; xor-butterfly lane sum).
 constexpr uint32_t kPatchWordsMax = 256;
-template <int WIDTH, bool GATED>
+template <int WIDTH, bool GATED, bool TABLED>
 __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint32_t words_per_group) {
     // each workgroup scans words_per_group words of the map (few for a small map, so that it still spreads over the chip),
     // gathers the marked elements in LDS, then its eight 32-lane groups take them in turn
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
         uint16_t scale_bits[kAhead][GATED ? 2 : 1], bias_bits[kAhead][GATED ? 2 : 1];
         // the block's BF16-rounded chain sum depends on the row only: with 16-element blocks it comes from the table the
         // row kernels left (the same additions in the same order)
-        const bool tabled = WIDTH == 16 && p.asum16;
+        constexpr bool tabled = TABLED;   // a compile-time choice: with both forms in one kernel the registers of either stay live
         float chain[kAhead];
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) {
@@ -314,10 +314,13 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
             for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
                 float dot = 0;
 #pragma unroll
-                for (int i = 0; i < WIDTH; i += 4) {
-                    const uint32_t packed = (words[u][proj][i / 8] >> (4 * (i % 8))) & 0xffffu;
-                    dot += xb[i] * float(packed & 15u) + xb[i + 1] * float((packed >> 4) & 15u) +
-                           xb[i + 2] * float((packed >> 8) & 15u) + xb[i + 3] * float((packed >> 12) & 15u);
+                for (int i = 0; i < WIDTH; i += 8) {
+                    // nibble j of a word is element j: the even ones and the odd ones as bytes, each converted by one byte-to-float instruction
+                    const uint32_t even = words[u][proj][i / 8] & 0x0f0f0f0fu, odd = (words[u][proj][i / 8] >> 4) & 0x0f0f0f0fu;
+                    dot += xb[i] * float(even & 0xffu) + xb[i + 1] * float(odd & 0xffu) +
+                           xb[i + 2] * float((even >> 8) & 0xffu) + xb[i + 3] * float((odd >> 8) & 0xffu);
+                    dot += xb[i + 4] * float((even >> 16) & 0xffu) + xb[i + 5] * float((odd >> 16) & 0xffu) +
+                           xb[i + 6] * float(even >> 24) + xb[i + 7] * float(odd >> 24);
                 }
                 result[proj] += b16(scale_bits[u][proj]) * dot + sum * b16(bias_bits[u][proj]);
             }
@@ -353,8 +356,11 @@ void launch_prefill_patch(hipStream_t s, const PrefillGemm& p, bool gated) {
     const bool wide = p.K % 512 == 0 && p.N % 8 == 0;     // the reference's lane-width rule (metal.mm:649-674)
     const uint32_t per = p.near_words >= kPatchWordsMax * 1024u ? kPatchWordsMax : 64u;   // words of the map per workgroup
     const dim3 grid((p.near_words + per - 1) / per);
-    if (gated) { if (wide) hipLaunchKernelGGL((prefill_patch_kernel<16, true>), grid, dim3(256), 0, s, p, per); else hipLaunchKernelGGL((prefill_patch_kernel<8, true>), grid, dim3(256), 0, s, p, per); }
-    else { if (wide) hipLaunchKernelGGL((prefill_patch_kernel<16, false>), grid, dim3(256), 0, s, p, per); else hipLaunchKernelGGL((prefill_patch_kernel<8, false>), grid, dim3(256), 0, s, p, per); }
+    const bool tabled = wide && p.asum16;                 // the table holds sums of 16-element blocks
+#define ZC_PATCH(W, G, T) hipLaunchKernelGGL((prefill_patch_kernel<W, G, T>), grid, dim3(256), 0, s, p, per)
+    if (gated) { if (tabled) ZC_PATCH(16, true, true); else if (wide) ZC_PATCH(16, true, false); else ZC_PATCH(8, true, false); }
+    else { if (tabled) ZC_PATCH(16, false, true); else if (wide) ZC_PATCH(16, false, false); else ZC_PATCH(8, false, false); }
+#undef ZC_PATCH
 }
 bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts) { return hidden % 128 == 0 && inter % 128 == 0 && experts <= 1024; }
 

@@ -164,7 +164,7 @@ def test_route_stress_rows(ctx):  # :744-797
             ctx.route(ctx.upload(v), bad_tokens, 512)
 
 
-@pytest.mark.parametrize("T,E,k", [(1, 512, 10), (7, 512, 10), (64, 512, 10), (513, 512, 10), (2048, 512, 10), (5, 32, 4)])
+@pytest.mark.parametrize("T,E,k", [(1, 512, 10), (7, 512, 10), (64, 512, 10), (513, 512, 10), (2048, 512, 10), (5, 32, 4), (1000, 512, 10), (821, 64, 3), (2731, 130, 3)])
 def test_dispatch_matches_counting_sort(ctx, T, E, k):  # model.cpp:449-479
     rng = np.random.default_rng(T)
     skew = rng.standard_normal(E) * 2

@@ -528,22 +528,28 @@ __global__ __launch_bounds__(1024) void dispatch_kernel(const int32_t* ids, uint
 // scans, one wavefront per expert places.  offsets[1 + e] doubles as the count array between the first two steps.
 __global__ __launch_bounds__(256) void dispatch_count_kernel(const int32_t* __restrict__ ids, uint32_t n, uint32_t E, int32_t* __restrict__ offsets, int32_t* status, bool aligned) {
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (blockIdx.x == 0) {
+    {   // every workgroup checks its share of the ids (one workgroup doing all of them was the longest-running one)
         int bad = 0;
-        for (uint32_t p = threadIdx.x; p < n; p += blockDim.x) bad |= (ids[p] < 0 || ids[p] >= int32_t(E));
+        for (uint32_t p = blockIdx.x * blockDim.x + threadIdx.x; p < n; p += gridDim.x * blockDim.x) { const int32_t id = ids[p]; bad |= (id < 0 || id >= int32_t(E)); }
         if (bad) atomicOr(status, 1);
     }
     if (e >= E) return;
     int32_t c = 0;
     uint32_t p0 = 0;
-    if (aligned)
-        for (; p0 + 8 * 256 <= n; p0 += 8 * 256) {   // eight steps' loads in flight
-            int4 v[8];
+    if (aligned && n >= 8 * 256) {   // eight steps' loads in flight, the next eight requested before these are counted
+        int4 v[8], w[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const int4*>(ids + p0 + j * 256 + 4 * lane);
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const int4*>(ids + j * 256 + 4 * lane);
+        for (; p0 + 8 * 256 <= n; p0 += 8 * 256) {
+            const uint32_t following = p0 + 16 * 256 <= n ? p0 + 8 * 256 : p0;   // none left: the same batch again, not counted
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w[j] = *reinterpret_cast<const int4*>(ids + following + j * 256 + 4 * lane);
 #pragma unroll
             for (int j = 0; j < 8; ++j) c += (v[j].x == int32_t(e)) + (v[j].y == int32_t(e)) + (v[j].z == int32_t(e)) + (v[j].w == int32_t(e));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = w[j];
         }
+    }
     for (; p0 < n; p0 += 256) {   // a lane looks at four neighbouring slots per step
         const uint32_t p = p0 + 4 * lane;
         int4 v = make_int4(-1, -1, -1, -1);
@@ -580,7 +586,41 @@ __global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* __re
     int32_t pos = offsets[e];
     if (offsets[e + 1] == pos) return;
     const uint64_t below = (1ull << lane) - 1;
-    for (uint32_t q0 = 0; q0 < n; q0 += 8 * 256) {   // eight steps' loads in flight, then the steps in order
+    // eight steps of 256 slots, in order: four neighbouring slots per lane, slots of lower lanes first, then the lane's own
+    auto place = [&](const int4 (&batch)[8], uint32_t q0) {
+#pragma unroll
+        for (int step = 0; step < 8; ++step) {
+            if (q0 + step * 256 >= n) break;
+            const uint32_t p = q0 + step * 256 + 4 * lane;
+            const int4 v = batch[step];
+            const bool m[4] = {v.x == int32_t(e), v.y == int32_t(e), v.z == int32_t(e), v.w == int32_t(e)};
+            const uint64_t mask[4] = {__ballot(m[0]), __ballot(m[1]), __ballot(m[2]), __ballot(m[3])};
+            if ((mask[0] | mask[1] | mask[2] | mask[3]) == 0) continue;   // uniform: none of these 256 slots is the expert's
+            int32_t at = pos + __popcll(mask[0] & below) + __popcll(mask[1] & below) + __popcll(mask[2] & below) + __popcll(mask[3] & below);
+            uint32_t token = p / topk, rest = p % topk;   // one division per step, not one per slot
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (m[j]) { slots[at] = int32_t(p + j); if (rows) rows[at] = int32_t(token); ++at; }
+                if (++rest == topk) { rest = 0; ++token; }
+            }
+            pos += __popcll(mask[0]) + __popcll(mask[1]) + __popcll(mask[2]) + __popcll(mask[3]);
+        }
+    };
+    uint32_t q0 = 0;
+    if (aligned && n >= 8 * 256) {   // whole batches: the next batch is requested before this one is placed
+        int4 ahead[8], next[8];
+#pragma unroll
+        for (int step = 0; step < 8; ++step) ahead[step] = *reinterpret_cast<const int4*>(ids + step * 256 + 4 * lane);
+        for (; q0 + 8 * 256 <= n; q0 += 8 * 256) {
+            const uint32_t following = q0 + 16 * 256 <= n ? q0 + 8 * 256 : q0;   // none left: the same batch again, not placed
+#pragma unroll
+            for (int step = 0; step < 8; ++step) next[step] = *reinterpret_cast<const int4*>(ids + following + step * 256 + 4 * lane);
+            place(ahead, q0);
+#pragma unroll
+            for (int step = 0; step < 8; ++step) ahead[step] = next[step];
+        }
+    }
+    for (; q0 < n; q0 += 8 * 256) {   // the ragged end, or an array that is not sixteen-byte aligned
         int4 ahead[8];
 #pragma unroll
         for (int step = 0; step < 8; ++step) {
@@ -590,19 +630,7 @@ __global__ __launch_bounds__(256) void dispatch_place_kernel(const int32_t* __re
             else { if (p < n) v.x = ids[p]; if (p + 1 < n) v.y = ids[p + 1]; if (p + 2 < n) v.z = ids[p + 2]; if (p + 3 < n) v.w = ids[p + 3]; }
             ahead[step] = v;
         }
-#pragma unroll
-        for (int step = 0; step < 8; ++step) {   // four neighbouring slots per lane: slots of lower lanes come first, then the lane's own in order
-            if (q0 + step * 256 >= n) break;
-            const uint32_t p = q0 + step * 256 + 4 * lane;
-            const int4 v = ahead[step];
-            const bool m[4] = {v.x == int32_t(e), v.y == int32_t(e), v.z == int32_t(e), v.w == int32_t(e)};
-            const uint64_t mask[4] = {__ballot(m[0]), __ballot(m[1]), __ballot(m[2]), __ballot(m[3])};
-            int32_t at = pos + __popcll(mask[0] & below) + __popcll(mask[1] & below) + __popcll(mask[2] & below) + __popcll(mask[3] & below);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (m[j]) { slots[at] = int32_t(p + j); if (rows) rows[at] = int32_t((p + j) / topk); ++at; }
-            pos += __popcll(mask[0]) + __popcll(mask[1]) + __popcll(mask[2]) + __popcll(mask[3]);
-        }
+        place(ahead, q0);
     }
 }
 void launch_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets,

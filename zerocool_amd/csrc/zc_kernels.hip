@@ -4,6 +4,7 @@
 // wavefront carries two output rows.  Results are bit-identical to the CPU statement
 // of the same arithmetic for any input.
 #include "zc_kernels.hpp"
+#include <type_traits>
 #include "zc_device.hpp"
 
 namespace zc {
@@ -189,17 +190,34 @@ __global__ __launch_bounds__(256) void plain_kernel(const void* __restrict__ w, 
     const float* xr = x + uint64_t(t) * K;
     float sum = 0;
     uint32_t k = lane;
-    for (; k + 7 * 32 < K; k += 8 * 32) {   // eight loads of each operand in flight; the additions stay in k order
-        float xv[8], wv[8];
+    // every element's 32-bit word is aligned and inside the array: a four-byte aligned array with an even number of elements
+    const bool even_rows = (reinterpret_cast<uintptr_t>(w) & 3u) == 0 && ((uint64_t(N) * K) & 1u) == 0;
+    // `count` loads of each operand in flight; the additions stay in k order.  The weight's type is chosen outside the
+    // batch: loads on either side of a branch would each be waited for where the sides join.
+    auto batch = [&](auto count, auto kind) {
+        constexpr int kLoads = decltype(count)::value, kKind = decltype(kind)::value;
+        float xv[kLoads], wv[kLoads];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kLoads; ++j) {
             xv[j] = xr[k + 32 * j];
-            wv[j] = dtype == 1 ? reinterpret_cast<const float*>(w)[uint64_t(row) * K + k + 32 * j]
-                               : b16(reinterpret_cast<const uint16_t*>(w)[uint64_t(row) * K + k + 32 * j]);
+            const uint64_t at = uint64_t(row) * K + k + 32 * j;
+            if constexpr (kKind == 0) wv[j] = reinterpret_cast<const float*>(w)[at];
+            else if constexpr (kKind == 1) {   // a BF16 weight from the aligned 32-bit word that holds it
+                const uint32_t word = reinterpret_cast<const uint32_t*>(w)[at >> 1];
+                wv[j] = __uint_as_float((at & 1) ? (word & 0xffff0000u) : (word << 16));
+            } else wv[j] = b16(reinterpret_cast<const uint16_t*>(w)[at]);
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) sum += xv[j] * wv[j];
-    }
+        for (int j = 0; j < kLoads; ++j) sum += xv[j] * wv[j];
+        k += kLoads * 32;
+    };
+    auto batches = [&](auto kind) {   // a row is one memory latency per batch: long rows take sixteen loads at a time
+        while (k + 15 * 32 < K) batch(std::integral_constant<int, 16>{}, kind);
+        while (k + 7 * 32 < K) batch(std::integral_constant<int, 8>{}, kind);
+    };
+    if (dtype == 1) batches(std::integral_constant<int, 0>{});
+    else if (even_rows) batches(std::integral_constant<int, 1>{});
+    else batches(std::integral_constant<int, 2>{});
     for (; k < K; k += 32) {
         const float wv = dtype == 1 ? reinterpret_cast<const float*>(w)[uint64_t(row) * K + k]
                                     : b16(reinterpret_cast<const uint16_t*>(w)[uint64_t(row) * K + k]);

@@ -151,7 +151,10 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
         uint32_t out[16];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const uint32_t even = words[w] & 0x0f0f0f0fu, odd = (words[w] >> 4) & 0x0f0f0f0fu;
+            uint32_t even = words[w] & 0x0f0f0f0fu, odd = (words[w] >> 4) & 0x0f0f0f0fu;
+            // the masked words are kept from the optimiser, which would otherwise fold mask and shift into a bit-field extract
+            // per element and convert that: with whole bytes every element is one byte-to-float conversion
+            asm volatile("" : "+v"(even), "+v"(odd));
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const f32x2 pair = {float((even >> (8 * q)) & 0xffu), float((odd >> (8 * q)) & 0xffu)};

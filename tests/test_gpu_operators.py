@@ -116,7 +116,9 @@ def test_single_token_rows(ctx, K, N):  # :1100-1125 shapes plus the benchmark s
         ctx.free(b)
 
 
-@pytest.mark.parametrize("K,N", [(10240, 4), (2560, 1), (2560, 48), (2048, 1), (3072, 1)])
+# the last three: a row of sixteen-load and eight-load batches plus single steps, rows shorter than one batch, and an odd
+# number of weights (their 16-bit words are then read one by one, not through aligned 32-bit words)
+@pytest.mark.parametrize("K,N", [(10240, 4), (2560, 1), (2560, 48), (2048, 1), (3072, 1), (864, 5), (96, 2), (257, 3)])
 def test_plain_rows(ctx, K, N):  # :1126-1135, the shared_expert_gate shape
     rng = np.random.default_rng(K + N)
     w = oracle.bf_bits(0.02 * rng.standard_normal(N * K)); x = oracle.bf(rng.standard_normal(2 * K))

@@ -27,6 +27,11 @@
  *   route ids         stable-sort brute force incl. NaN/inf/ties (…:744-797)
  *   moe_sum           captured BF16 midpoint value (…:827-842)
  *   dispatch/scatter  brute force (…:1500-1533)
+ *   plain_mm          double precision within the fp32 bound on the reference's four
+ *                     shapes (…:1126-1135), and exact closed forms that hold only for
+ *                     the lane chain k = lane + 32 j (2^24 / 1 absorption rows)
+ *   Q4 lane widths    exact closed forms that tell sixteen-element lane steps from
+ *                     eight-element ones, and the every-32nd-block revisit, bit for bit
  *   route softmax WEIGHT BITS and the final simd_sum association of the affine
  *   dots: parity unpinned at bit level (only an Apple GPU run could pin them);
  *   sum-to-one and tolerance checks only.

@@ -159,8 +159,9 @@ def test_stack_reports_invalid_router_output(ctx):
 
 def test_single_token_launches_across_the_tag_wrap(ctx):
     # The one-token kernel marks everything its workgroups exchange with a 16-bit tag that advances with every layer of
-    # every launch: a few thousand launches of a two-layer stack take it once around, with launches of the several-token
-    # kernel (which shares the flags, not the tagged buffers) in between.  Every launch must give the first one's output.
+    # every one-token launch: some thirty thousand launches of a two-layer stack take it once around, with launches of the
+    # several-token kernel (which shares the flags, not the tagged buffers, and must not move the tags) in between.
+    # Every launch must give the first one's output.
     cfg = workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512)
     layers = [workload.LayerWeights(ctx, cfg, 401 + l, ("zipf", 1.1)) for l in range(2)]
     stack = ctx.stack_create(cfg, [l.layer for l in layers], 2)
@@ -171,17 +172,25 @@ def test_single_token_launches_across_the_tag_wrap(ctx):
     first = out1.numpy(f32).tobytes()
     ctx.stack_decode(stack, x2, 2, out2); ctx.moe_check()
     first2 = out2.numpy(f32).tobytes()
-    launches = 65535 // (3 * 2 + 16) + 200
+    launches = 65535 // 2 + 300
     for i in range(launches):
         ctx.stack_decode(stack, x1, 1, out1)
         if i % 97 == 0:
             ctx.stack_decode(stack, x2, 2, out2)
-        if i % 500 == 0 or i > launches - 400 and i % 7 == 0:
+        if i % 4000 == 0 or i > launches - 600 and i % 7 == 0:
             ctx.moe_check()
             assert out1.numpy(f32).tobytes() == first, f"launch {i}"
             assert out2.numpy(f32).tobytes() == first2, f"launch {i}"
     ctx.moe_check()
     assert out1.numpy(f32).tobytes() == first
+    # A long run of several-token launches between two one-token launches: however many there are, the one-token launch
+    # that follows must not meet a tag its predecessor left (run lengths around a multiple of the tag period included).
+    for run in (1, 409, 1228, 1229, 2979):
+        for _ in range(run):
+            ctx.stack_decode(stack, x2, 2, out2)
+        ctx.stack_decode(stack, x1, 1, out1); ctx.moe_check()
+        assert out1.numpy(f32).tobytes() == first, f"after {run} two-token launches"
+        assert out2.numpy(f32).tobytes() == first2
     ctx.stack_destroy(stack)
     for l in layers:
         for b in (l.router, l.shared_gate, l.shared_record, l.records):

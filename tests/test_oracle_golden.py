@@ -235,3 +235,76 @@ def test_q4_lane_width_shapes_track_double(K, N):  # shapes of :1100-1125; value
         oracle.b16(b).astype(np.float64).reshape(N, -1), 64, 1)
     want = dec @ x.astype(np.float64)
     assert np.max(np.abs(got - want)) < 2e-2 * np.max(np.abs(want)) + 1e-3   # BF16 bias-sum rule bounds the gap
+
+
+# ---- lane partitions pinned by exact arithmetic -------------------------------------------------------------------
+# fp32 cannot hold 2^24 + 1: added to 2^24 a one is lost, added to -(2^24) it is kept.  Inputs built from
+# {2^24, -2^24, 1} therefore give a result that depends on WHICH additions share an accumulator, while every other
+# addition in the kernel is exact, so the expected values below follow from the kernel text alone (which element
+# belongs to which lane), not from the order of the final lane sum.
+BIG = float(2 ** 24)
+
+
+@pytest.mark.parametrize("K,N,tokens", [(10240, 4, 1), (2560, 1, 1), (2560, 48, 2), (2560, 64, 1)])   # shapes of :1126-1135
+def test_plain_mm_tracks_double(K, N, tokens):  # qwen.metal:499-506
+    rng = np.random.default_rng(K + N)
+    w = oracle.bf_bits(0.02 * rng.standard_normal(N * K)); x = oracle.bf(rng.standard_normal(tokens * K))
+    got = oracle.plain_mm(w, x, K, N, tokens, float_output=True)
+    wd = oracle.b16(w).astype(np.float64).reshape(N, K); xd = x.astype(np.float64).reshape(tokens, K)
+    want = xd @ wd.T
+    bound = 2.0 ** -23 * (K // 32 + 6) * (np.abs(xd) @ np.abs(wd).T)   # a lane chain of K/32 terms, five butterfly steps
+    assert (np.abs(got - want) <= bound).all()
+    rounded = oracle.plain_mm(w, x, K, N, tokens)
+    assert rounded.tobytes() == oracle.bf(got).tobytes()
+
+
+def test_plain_mm_lane_chain_is_k_mod_32():  # qwen.metal:503: lane l adds k = l, l + 32, l + 64, ... in turn
+    K, N, T = 2560, 3, 2
+    w = np.full(N * K, 0x3f80, np.uint16)                   # every weight 1.0: the products are the inputs
+    x = np.ones((T, K), f32)
+    # token 0: 2^24 and -2^24 meet in lane 5 (k = 5 and k = 37), so they cancel before any one is added:
+    # lane 5 holds K/32 - 2, every other lane K/32, all exact, and so is their sum whatever its order.
+    x[0, 5] = BIG; x[0, 37] = -BIG
+    # token 1: the same pair one element apart (lanes 6 and 7): lane 6 loses its 79 ones (2^24 + 1 -> 2^24), lane 7
+    # keeps them (-(2^24) + 79 is exact); both lanes together give 79, the other thirty lanes 80 each.
+    x[1, 6] = BIG; x[1, 7] = -BIG
+    got = oracle.plain_mm(w, x, K, N, T, float_output=True)
+    assert (got[0] == K - 2).all(), got          # a k-ascending sum over all lanes gives K - 33, a stride of 64 loses lane 5's ones
+    assert (got[1] == 79 + 30 * 80).all(), got
+    assert oracle.plain_mm(w, x, K, N, T).tobytes() == oracle.bf(got).tobytes()
+    # rows and tokens are indexed as [n][K] and [t][K]: a weight row of zeros silences exactly its own output
+    w2 = w.copy(); w2[K:2 * K] = 0
+    got2 = oracle.plain_mm(w2, x, K, N, T, float_output=True)
+    assert (got2[:, 1] == 0).all() and (got2[:, 0] == got[:, 0]).all() and (got2[:, 2] == got[:, 2]).all()
+
+
+def _q4_bias_only(K, N, x):
+    """Codes 0, every bias 1.0: a row's output is the lane-ordered sum of the blocks' BF16 chain sums."""
+    w = np.zeros(N * K // 8, np.uint32)
+    s = np.full(N * K // 64, 0x3f80, np.uint16); b = np.full(N * K // 64, 0x3f80, np.uint16)
+    return oracle.linear(oracle.make_linear(w, s, b, K, N), np.asarray(x, f32), 1, float_output=True)[0]
+
+
+def test_q4_lane_width_rule_bit_level():  # qwen.metal:46-62; metal.mm:795-803: sixteen elements per lane step iff K % 512 == 0 and N % 8 == 0
+    # elements 0..15 carry the four quads (1, 2^24, 1, -2^24).  In one lane step of sixteen, the chain sums meet in one
+    # accumulator: ((1 + 2^24) + 1) - 2^24 = 0.  In steps of eight, lane 0 holds 1 + 2^24 -> 2^24 and lane 1 holds
+    # 1 - 2^24 exactly: together 1.  All other lanes hold zero, so the order of the lane sum does not matter.
+    def row(K):
+        x = np.zeros(K, f32); x[0] = 1; x[4] = BIG; x[8] = 1; x[12] = -BIG
+        return x
+    assert (_q4_bias_only(512, 8, row(512)) == 0.0).all()      # wide lanes
+    assert (_q4_bias_only(1024, 16, row(1024)) == 0.0).all()
+    assert (_q4_bias_only(256, 8, row(256)) == 1.0).all()      # K % 512 != 0: narrow lanes
+    assert (_q4_bias_only(512, 7, row(512)) == 1.0).all()      # N % 8 != 0: narrow lanes
+    assert (_q4_bias_only(704, 8, row(704)) == 1.0).all()      # the reference's own narrow shape (:1103)
+
+
+def test_q4_lane_revisits_every_32nd_block():  # qwen.metal:51: base = lane * width + j * 32 * width
+    # wide lanes, K = 1536: lane 3 owns the blocks at elements 48, 560 and 1072; their chain sums 2^24, 1, -2^24 meet in
+    # that order in lane 3's accumulator: (2^24 + 1) - 2^24 = 0.  Contiguous blocks per lane, or any other stride, would
+    # leave the one in a lane of its own.
+    K = 1536
+    x = np.zeros(K, f32); x[48] = BIG; x[560] = 1; x[1072] = -BIG
+    assert (_q4_bias_only(K, 8, x) == 0.0).all()
+    x = np.zeros(K, f32); x[48] = BIG; x[64] = 1; x[1072] = -BIG     # the one in lane 4 instead: it survives
+    assert (_q4_bias_only(K, 8, x) == 1.0).all()

@@ -2,7 +2,7 @@
 // be replayed against this library:
 //  * RouteTrace: the coordinator's JSON-lines capture "qwen_route_trace_v1" (include/engine/route_trace.hpp): one
 //    object per line {kind, sequence, monotonic_ns, event, request_id, forward_id, details}; the selected experts of a
-//    layer travel in a "routes" event.  Same call order rules and limits (20000 events, 64 KiB per line, 16 MiB).
+//    layer travel in a "routes" event.  The format's nesting rules and limits (20000 events, 64 KiB per line, 16 MiB) hold.
 //  * read_route_trace: parses such a file back into committed forwards.
 //  * tensor dumps: Model::trace writes <dir>/step_<offset>/<name>.bin as raw bytes (model.cpp:274-283), e.g.
 //    router_<layer>.bin (fp32 logits) and route_<layer>.bin (int32 ids); write_tensor_dump / read_tensor_dump do the
@@ -12,84 +12,124 @@
 #include <chrono>
 #include <cstring>
 #include <cstdio>
-#include <fcntl.h>
-#include <unistd.h>
 
 namespace zerocool::engine {
 
+// Writer of the capture format.  A capture is a strict nesting: trace { request { forward { routes x layers } } },
+// which is kept here as one explicit stage plus the geometry of the forward that is open.  Every event goes through
+// one serializer (Event), which owns the envelope fields, the limits and the flush.
 class RouteTrace {
+    enum class Stage { Idle, Request, Forward, Closed };
+    // One line of the capture: details are appended field by field, the envelope is added when the line is written.
+    class Event {
+    public:
+        explicit Event(const char* name) : name_(name) {}
+        Event& number(const char* key, uint64_t v) { field(key) += std::to_string(v); return *this; }
+        Event& flag(const char* key, bool v) { field(key) += v ? "true" : "false"; return *this; }
+        Event& raw(const char* key, const std::string& json) { field(key) += json; return *this; }
+        Event& text(const char* key, const std::string& v) {
+            std::string& out = field(key);
+            out += '"';
+            for (const unsigned char c : v) {
+                if (c == '"' || c == '\\') { out += '\\'; out += char(c); }
+                else if (c < 0x20) { char b[8]; std::snprintf(b, sizeof b, "\\u%04x", c); out += b; }
+                else out += char(c);
+            }
+            out += '"';
+            return *this;
+        }
+        Event& integers(const char* key, std::span<const int> v) {
+            std::string& out = field(key);
+            out += '[';
+            for (size_t i = 0; i < v.size(); ++i) { if (i) out += ','; out += std::to_string(v[i]); }
+            out += ']';
+            return *this;
+        }
+        const char* name() const { return name_; }
+        std::string details() const { return "{" + body_ + "}"; }
+    private:
+        std::string& field(const char* key) { if (!body_.empty()) body_ += ','; body_ += '"'; body_ += key; body_ += "\":"; return body_; }
+        const char* name_; std::string body_;
+    };
+    static constexpr uint64_t kMaxEvents = 20000, kMaxLine = 64u << 10, kMaxBytes = 16u << 20, kMaxContext = 8192;
+
 public:
     RouteTrace(const std::filesystem::path& path, const std::string& identity_json, uint32_t layers, uint32_t topk) : layers_(layers), topk_(topk) {
-        Json::parse(identity_json);   // must be valid JSON: it is embedded verbatim
-        const int fd = ::open(path.c_str(), O_WRONLY | O_CREAT | O_EXCL | O_CLOEXEC, 0600);
-        if (fd < 0) throw std::runtime_error("route trace must be a new file: " + path.string());
-        stream_ = ::fdopen(fd, "w");
-        if (!stream_) { ::close(fd); throw std::runtime_error("cannot open route trace"); }
-        try { emit("trace_begin", "{\"identity\":" + identity_json + "}"); } catch (...) { std::fclose(stream_); stream_ = nullptr; throw; }
+        Json::parse(identity_json);   // embedded as it is, so it has to parse
+        file_ = std::fopen(path.c_str(), "wx");   // exclusive: a capture never continues or replaces another file
+        if (!file_) throw std::runtime_error("route trace must be a new file: " + path.string());
+        try { write(Event("trace_begin").raw("identity", identity_json)); }
+        catch (...) { std::fclose(file_); file_ = nullptr; throw; }
     }
     RouteTrace(const RouteTrace&) = delete;
+    RouteTrace& operator=(const RouteTrace&) = delete;
     ~RouteTrace() {
-        if (stream_) {
-            if (!terminal_) try { emit("trace_end", "{\"status\":\"incomplete\"}"); } catch (...) {}
-            std::fclose(stream_);
-        }
+        if (!file_) return;
+        if (stage_ != Stage::Closed) { try { write(Event("trace_end").text("status", "incomplete")); } catch (...) {} }
+        std::fclose(file_);
     }
     void request_begin(const std::string& name, std::span<const int> prompt, int max_tokens, bool prime) {
-        if (request_ || forward_ || terminal_) throw std::logic_error("route request already active");
-        request_ = true; ++request_id_;
-        emit("request_begin", "{\"name\":" + quoted(name) + ",\"input_token_ids\":" + list(prompt) + ",\"max_tokens\":" + std::to_string(max_tokens) + ",\"prime\":" + (prime ? "true" : "false") + "}");
+        expect(Stage::Idle, "a route request is already open");
+        ++request_id_; stage_ = Stage::Request;
+        write(Event("request_begin").text("name", name).integers("input_token_ids", prompt).raw("max_tokens", std::to_string(max_tokens)).flag("prime", prime));
     }
     void request_end(std::span<const int> output, const std::string& reason, uint64_t reused) {
-        if (!request_ || forward_ || terminal_) throw std::logic_error("route request not complete");
-        emit("request_end", "{\"output_token_ids\":" + list(output) + ",\"finish_reason\":" + quoted(reason) + ",\"reused_tokens\":" + std::to_string(reused) + "}");
-        request_ = false;
+        expect(Stage::Request, "no route request to end, or a forward is still open");
+        write(Event("request_end").integers("output_token_ids", output).text("finish_reason", reason).number("reused_tokens", reused));
+        stage_ = Stage::Idle;
     }
     void begin(uint64_t session, uint32_t offset, std::span<const int> input, const std::string& phase, size_t slots) {
-        if (!request_ || forward_ || terminal_ || input.empty() || offset + input.size() > 8192 || !session) throw std::logic_error("invalid route forward start");
-        forward_ = true; ++forward_id_; next_layer_ = 0; offset_ = offset; tokens_ = uint32_t(input.size());
-        emit("forward_begin", "{\"session_id\":" + quoted(std::to_string(session)) + ",\"offset\":" + std::to_string(offset) + ",\"tokens\":" + std::to_string(tokens_) +
-                                  ",\"input_token_ids\":" + list(input) + ",\"request_phase\":" + quoted(phase) + ",\"expert_slots\":" + std::to_string(slots) + "}");
+        expect(Stage::Request, "a forward needs an open request and no other forward");
+        if (!session || input.empty() || uint64_t(offset) + input.size() > kMaxContext) throw std::logic_error("route forward outside the context window");
+        ++forward_id_; stage_ = Stage::Forward; open_ = Forward{offset, uint32_t(input.size()), 0};
+        write(Event("forward_begin").text("session_id", std::to_string(session)).number("offset", offset).number("tokens", open_.tokens)
+                  .integers("input_token_ids", input).text("request_phase", phase).number("expert_slots", slots));
     }
     void routes(int layer, uint32_t offset, uint32_t tokens, std::span<const int> selected) {
-        if (!forward_ || terminal_ || layer != next_layer_ || layer >= int(layers_) || offset != offset_ || tokens != tokens_ || selected.size() != size_t(tokens) * topk_)
-            throw std::logic_error("route pass does not match active forward");
-        emit("routes", "{\"layer\":" + std::to_string(layer) + ",\"routes\":" + list(selected) + "}"); ++next_layer_;
+        expect(Stage::Forward, "routes outside a forward");
+        const bool in_turn = layer >= 0 && uint32_t(layer) == open_.layers_seen && open_.layers_seen < layers_;
+        if (!in_turn || offset != open_.offset || tokens != open_.tokens || selected.size() != size_t(tokens) * topk_)
+            throw std::logic_error("routes do not belong to the open forward");
+        write(Event("routes").number("layer", uint64_t(layer)).integers("routes", selected));
+        ++open_.layers_seen;
     }
     void commit(uint32_t position) {
-        if (!forward_ || terminal_ || next_layer_ != int(layers_) || position != offset_ + tokens_) throw std::logic_error("route forward did not complete all layers");
-        emit("forward_commit", "{\"position\":" + std::to_string(position) + "}"); forward_ = false;
+        expect(Stage::Forward, "commit outside a forward");
+        if (open_.layers_seen != layers_ || position != open_.offset + open_.tokens) throw std::logic_error("the forward has not routed every layer");
+        write(Event("forward_commit").number("position", position));
+        stage_ = Stage::Request;
     }
-    void abort() { if (forward_ && !terminal_) { emit("forward_abort", "{\"captured_layers\":" + std::to_string(next_layer_) + "}"); forward_ = false; } }
-    void cache_reset() { emit("cache_reset", "{}"); }
+    void abort() {   // a forward given up half way; harmless when none is open
+        if (stage_ != Stage::Forward) return;
+        write(Event("forward_abort").number("captured_layers", open_.layers_seen));
+        stage_ = Stage::Request;
+    }
+    void cache_reset() { write(Event("cache_reset")); }
     void finish() {
-        if (request_ || forward_ || terminal_) throw std::logic_error("route trace is incomplete");
-        emit("trace_end", "{\"status\":\"complete\"}"); terminal_ = true;
+        expect(Stage::Idle, "the route trace still has an open request");
+        write(Event("trace_end").text("status", "complete"));
+        stage_ = Stage::Closed;
     }
+
 private:
-    static std::string quoted(const std::string& s) {
-        std::string out = "\"";
-        for (unsigned char c : s) {
-            if (c == '"' || c == '\\') { out += '\\'; out += char(c); }
-            else if (c < 0x20) { char b[8]; std::snprintf(b, sizeof b, "\\u%04x", c); out += b; }
-            else out += char(c);
-        }
-        return out + "\"";
-    }
-    static std::string list(std::span<const int> v) { std::string out = "["; for (size_t i = 0; i < v.size(); ++i) { if (i) out += ','; out += std::to_string(v[i]); } return out + "]"; }
-    void emit(const char* event, const std::string& details) {
-        if (sequence_ >= 20000) throw std::runtime_error("route trace event limit exceeded");
+    struct Forward { uint32_t offset = 0, tokens = 0, layers_seen = 0; };
+    void expect(Stage wanted, const char* otherwise) const { if (stage_ != wanted) throw std::logic_error(otherwise); }
+    void write(const Event& e) {
+        if (written_ >= kMaxEvents) throw std::runtime_error("route trace holds its 20000 events");
         const auto now = std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
-        const std::string line = "{\"details\":" + details + ",\"event\":\"" + event + "\",\"forward_id\":" + std::to_string(forward_id_) + ",\"kind\":\"qwen_route_trace_v1\",\"monotonic_ns\":" +
-                                 std::to_string(now) + ",\"request_id\":" + std::to_string(request_id_) + ",\"sequence\":" + std::to_string(sequence_ + 1) + "}\n";
-        if (line.size() > 65536 || bytes_ + line.size() > (16u << 20)) throw std::runtime_error("route trace byte limit exceeded");
-        if (std::fwrite(line.data(), 1, line.size(), stream_) != line.size() || std::fflush(stream_)) throw std::runtime_error("cannot flush route trace");
-        ++sequence_; bytes_ += line.size();
+        // keys in alphabetical order, as a sorted-key JSON writer prints them
+        std::string line = "{\"details\":" + e.details() + ",\"event\":\"" + e.name() + "\",\"forward_id\":" + std::to_string(forward_id_) +
+                           ",\"kind\":\"qwen_route_trace_v1\",\"monotonic_ns\":" + std::to_string(now) + ",\"request_id\":" + std::to_string(request_id_) +
+                           ",\"sequence\":" + std::to_string(written_ + 1) + "}\n";
+        if (line.size() > kMaxLine || bytes_ + line.size() > kMaxBytes) throw std::runtime_error("route trace is over its size limit");
+        if (std::fwrite(line.data(), 1, line.size(), file_) != line.size() || std::fflush(file_) != 0) throw std::runtime_error("route trace could not be written");
+        ++written_; bytes_ += line.size();
     }
-    std::FILE* stream_ = nullptr;
-    uint64_t sequence_ = 0, bytes_ = 0, request_id_ = 0, forward_id_ = 0;
-    uint32_t offset_ = 0, tokens_ = 0, layers_, topk_;
-    int next_layer_ = 0;
-    bool request_ = false, forward_ = false, terminal_ = false;
+    std::FILE* file_ = nullptr;
+    Stage stage_ = Stage::Idle;
+    Forward open_;
+    uint64_t written_ = 0, bytes_ = 0, request_id_ = 0, forward_id_ = 0;
+    uint32_t layers_, topk_;
 };
 
 struct TracedForward {

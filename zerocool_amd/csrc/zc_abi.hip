@@ -556,6 +556,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.tile_expert = w.tile_expert; g.tile_first = w.tile_first; g.tile_rows = w.tile_rows; g.tile_count = w.tile_count;
         g.K = H; g.N = I; g.out_b = w.actb;
         g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(n) * I / 32); g.near_margin = margin; g.ids = w.base.ids; g.slots = w.base.slots;
+        g.covered = w.base.offsets + E; g.experts = E;
         zc::launch_prefill_gemm(s, g, true, w.max_tiles);
         zc::launch_prefill_patch(s, g, true);
         zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum, table_inter ? w.asum16 : nullptr);
@@ -565,6 +566,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
         d.K = I; d.N = H; d.out_f = w.base.expert_out;
         d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(n) * H / 32); d.near_margin = margin; d.ids = w.base.ids; d.slots = w.base.slots;
+        d.covered = w.base.offsets + E; d.experts = E;
         zc::launch_prefill_gemm(s, d, false, w.max_tiles);
         zc::launch_prefill_patch(s, d, false);
     }
@@ -632,6 +634,7 @@ struct zc_hip_stack {
     uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
     unsigned long long* tlogits = nullptr; uint32_t *tact = nullptr, *tout = nullptr;   // tagged exchange buffers of the one-token kernel
     uint32_t epoch = 1u << 12;
+    uint32_t tag_base = 0;            // tags of the one-token kernel's exchange words: advanced by that kernel's launches only
     uint32_t wait_limit = 1u << 22;   // polls before a wait on another workgroup gives up
     int cus = 0; uint32_t lds_limit = 0;
     bool persistent_ok = false;
@@ -676,7 +679,7 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
     if (zc_hip_alloc(ctx, uint64_t(T) * H * 4, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
     st->xb = static_cast<float*>(p);
     // persistent path arena
-    st->persistent_ok = persistent_shape(*c);
+    st->persistent_ok = persistent_shape(*c) && n_layers <= 16384;   // the 16-bit exchange tags tell at most 65535 layers apart
     if (st->persistent_ok) {
         const uint32_t Tp = T < 8 ? T : 8;
         uint64_t at = 0;
@@ -764,6 +767,11 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
         st->epoch += 3 * L + 16;   // wraps modulo 2^32; the barrier compares epochs as signed differences
+        // The tagged buffers are written by one-token launches only, so their tags advance with those launches only:
+        // a launch's layer 0 then expects the tag right after the one its predecessor's last layer left, however many
+        // launches of the other kernel ran in between.
+        p.tag_base = st->tag_base;
+        if (nt == 1) st->tag_base = (st->tag_base + L) % 65535u;
         const uint32_t workgroups = uint32_t(st->cus);
         ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
         return ZC_OK;

@@ -312,7 +312,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         clock();
         // One token: the 16-bit tag of everything layer l exchanges, never 0 (the buffers start as zeros) and different
         // from the tags of the layers (and launches) just before it
-        auto tag_of = [&](uint32_t l) { return (p.epoch + l) % 65535u + 1u; };
+        auto tag_of = [&](uint32_t l) { return (p.tag_base + l) % 65535u + 1u; };
         const uint32_t tag = tag_of(layer);
         auto st_logit = [&](uint32_t index, float v) { ZC_ST(p.tlogits + index, (uint64_t(tag) << 32) | __float_as_uint(v)); };
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------

@@ -72,6 +72,7 @@ struct DecodeParams {
     unsigned long long* tlogits; uint32_t *tact, *tout;
     int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][T][topk], [L][T][topk], [L][T][H]
     uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
+    uint32_t tag_base;               // one token: layer l exchanges under tag (tag_base + l) % 65535 + 1; advances only with one-token launches
     unsigned long long* clocks;      // optional [L * kDecodeStamps][workgroups] 100 MHz timestamps, one per workgroup
 };
 constexpr uint32_t kDecodeStamps = 15;
@@ -104,6 +105,9 @@ struct PrefillGemm {
     uint32_t* near_bits; uint32_t near_words; float near_margin;
     const int32_t* ids;       // expert of sorted position pos: ids ? ids[slots[pos]] : 0 (used by the recomputation)
     const int32_t* slots;
+    // Sorted positions the product kernel covered: positions below *covered (the dispatch's offsets[experts]; an id
+    // outside [0, experts) leaves the tail uncovered and its map words unwritten) or, when covered is null, all of them.
+    const int32_t* covered; uint32_t experts;
 };
 constexpr float kPrefillMargin = 0x1p-22f;  // of the summed term magnitudes: four fp32 steps at that scale
 void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status);

@@ -257,7 +257,11 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
     const uint32_t word = blockIdx.x * words_per_group + threadIdx.x;
     if (threadIdx.x == 0) found_count = 0;
     __syncthreads();
-    uint32_t marks = (threadIdx.x < words_per_group && word < p.near_words) ? p.near_bits[word] : 0u;
+    // Only the map words of covered positions were written by the product kernel: a word past them holds whatever the
+    // buffer held before.  N is a multiple of 32, so a word never straddles two positions.
+    const uint32_t positions = p.near_words / (N / 32u);
+    const uint32_t covered = p.covered ? min(uint32_t(max(*p.covered, 0)), positions) : positions;
+    uint32_t marks = (threadIdx.x < words_per_group && word < p.near_words && word / (N / 32u) < covered) ? p.near_bits[word] : 0u;
     if (marks) {
         uint32_t at = atomicAdd(&found_count, uint32_t(__popc(marks)));
         while (marks) { found[at++] = uint16_t(threadIdx.x * 32 + (__ffs(marks) - 1)); marks &= marks - 1; }
@@ -267,6 +271,7 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
   for (uint32_t item = threadIdx.x >> 5; item < listed; item += 8) {
     const uint32_t code = blockIdx.x * (words_per_group * 32u) + found[item], pos = code / N, n = code % N;
     const uint32_t expert = p.ids ? uint32_t(p.ids[p.slots[pos]]) : 0u;
+    if (p.ids && expert >= p.experts) continue;   // an id the router could not give (reported through the status word)
     const uint8_t* record = p.records + uint64_t(expert) * p.stride;
     const uint32_t a_row = p.a_rows ? uint32_t(p.a_rows[pos]) / p.a_div : pos;
     const uint16_t* xr = p.a + uint64_t(a_row) * K;

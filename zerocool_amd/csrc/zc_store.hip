@@ -24,6 +24,7 @@ struct zc_hip_store {
     uint8_t* pool = nullptr;            // [capacity] slots, HBM (or plain host memory)
     hipStream_t side = nullptr;
     std::vector<hipEvent_t> filled;     // per slot: recorded after the slot's last fill
+    std::vector<hipEvent_t> released;   // per slot: recorded on the compute stream at every release of a lease; the slot's next fill waits for it
     std::vector<uint64_t> pending;      // host-memory store: per slot, the key of a fill that waits for its release, or ~0
     std::unordered_set<uint64_t> held;  // host-memory store: keys whose fills wait
     std::unique_ptr<zc::SlotCache> cache;
@@ -53,6 +54,9 @@ zc::SlotCache::Hooks hooks_of(zc_hip_store* s) {
     zc::SlotCache::Hooks h;
     if (s->ctx) {
         h.start = [s](size_t slot, uint64_t key) {
+            // The slot's previous record may still be read by kernels that were enqueued before its lease was released:
+            // the fill is ordered after the compute stream's position at that release, on the device, without the host.
+            ZC_STORE_HIP(hipStreamWaitEvent(s->side, s->released[slot], 0));
             ZC_STORE_HIP(hipMemcpyAsync(s->pool + slot * s->stride, s->backing + key * s->stride, s->record_bytes, hipMemcpyHostToDevice, s->side));
             ZC_STORE_HIP(hipEventRecord(s->filled[slot], s->side));
         };
@@ -64,6 +68,7 @@ zc::SlotCache::Hooks hooks_of(zc_hip_store* s) {
         };
         h.wait = [s](size_t slot) { ZC_STORE_HIP(hipEventSynchronize(s->filled[slot])); };
         h.move = [s](size_t from, size_t to) {
+            ZC_STORE_HIP(hipStreamWaitEvent(s->side, s->released[to], 0));
             ZC_STORE_HIP(hipMemcpyAsync(s->pool + to * s->stride, s->pool + from * s->stride, s->record_bytes, hipMemcpyDeviceToDevice, s->side));
             ZC_STORE_HIP(hipEventRecord(s->filled[to], s->side));
         };
@@ -88,10 +93,16 @@ void provide_pool(zc_hip_store* s, uint64_t slots, uint64_t keep) {
         if (s->pool && keep) { ZC_STORE_HIP(hipMemcpyAsync(fresh, s->pool, keep * s->stride, hipMemcpyDeviceToDevice, s->side)); ZC_STORE_HIP(hipStreamSynchronize(s->side)); }
         if (s->pool) zc_hip_free(s->ctx, s->pool);
         while (s->filled.size() > slots) { (void)hipEventDestroy(s->filled.back()); s->filled.pop_back(); }
+        while (s->released.size() > slots) { (void)hipEventDestroy(s->released.back()); s->released.pop_back(); }
         while (s->filled.size() < slots) {
             hipEvent_t e; ZC_STORE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
             ZC_STORE_HIP(hipEventRecord(e, s->side));   // a slot that was never filled counts as finished
             s->filled.push_back(e);
+        }
+        while (s->released.size() < slots) {
+            hipEvent_t e; ZC_STORE_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            ZC_STORE_HIP(hipEventRecord(e, s->side));   // a slot that was never leased has no reader to wait for
+            s->released.push_back(e);
         }
     } else {
         fresh = new uint8_t[slots * s->stride]();
@@ -133,6 +144,7 @@ zc_status zc_hip_store_destroy(zc_hip_store* s) {
     if (s->ctx) {
         if (s->side) { (void)hipStreamSynchronize(s->side); }
         for (hipEvent_t e : s->filled) (void)hipEventDestroy(e);
+        for (hipEvent_t e : s->released) (void)hipEventDestroy(e);
         if (s->side) (void)hipStreamDestroy(s->side);
         if (s->pool) zc_hip_free(s->ctx, s->pool);
         if (s->backing) zc_hip_free(s->ctx, s->backing);
@@ -173,7 +185,12 @@ zc_status zc_hip_store_wait(zc_hip_store* s, uint64_t lease) {
 }
 zc_status zc_hip_store_release(zc_hip_store* s, uint64_t lease) {
     if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
-    return guarded([&] { s->cache->release(lease); return ZC_OK; });
+    return guarded([&] {
+        s->cache->release(lease);
+        // Everything enqueued on the context's stream so far may read the slot; whatever refills it waits for this point.
+        if (s->ctx) ZC_STORE_HIP(hipEventRecord(s->released[lease], static_cast<hipStream_t>(zc_hip_stream(s->ctx))));
+        return ZC_OK;
+    });
 }
 zc_status zc_hip_store_prefetch(zc_hip_store* s, uint32_t layer, uint32_t expert, int* issued) {
     if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");

@@ -74,13 +74,15 @@ def test_tiny_layer_mixed_bits_and_group32(ctx):
     check_layer(ctx, workload.tiny_config(hidden=512, inter=256, group=32, bits=(8, 4, 4, 8)), 5, 13, None)
 
 
-@pytest.mark.parametrize("T", [1, 8])
-def test_single_layer_config(ctx, T):  # BASELINE configs 1 and 2
-    check_layer(ctx, workload.config("S"), T, 1, ("normal", 0.5))
+@pytest.mark.parametrize("T", [1, 8, 32, 64])
+def test_single_layer_config(ctx, T):  # BASELINE configs 1 and 2: every batch size the configuration names
+    tr = check_layer(ctx, workload.config("S"), T, 1, ("normal", 0.5))
+    print(f"T={T}: {len(np.unique(tr['ids']))} distinct experts for {T * 10} slots")
 
 
-def test_mixed_artifact_config(ctx):  # BASELINE config 4
-    check_layer(ctx, workload.config("S-mixed"), 1, 4, None)
+@pytest.mark.parametrize("T", [1, 16])
+def test_mixed_artifact_config(ctx, T):  # BASELINE config 4: decode batch 1 and 16
+    check_layer(ctx, workload.config("S-mixed"), T, 4, None)
 
 
 def test_reference_shape(ctx):  # hidden 2560 / intermediate 640: the narrow-lane (width 8) down projection

@@ -84,6 +84,66 @@ def test_prefill_against_the_cpu_oracle(ctx):
     assert rel(fast["out"].reshape(T, cfg.hidden), want) <= TOLERANCE
 
 
+def test_prefill_full_size_unskewed(ctx):
+    # BASELINE config 3 as written: 2048 tokens through the single-layer shape, no router skew (every expert gets rows,
+    # about forty each, so an expert's rows span several 32-row tiles).  Checked on ALL tokens against the exact path
+    # (itself byte-equal to the oracle at every smaller size) and on a sample of token rows against the CPU oracle
+    # directly: tokens are independent of each other, so the oracle can run on the sample alone.
+    cfg = workload.config("S")
+    T = 2048
+    weights = workload.LayerWeights(ctx, cfg, 301, None)
+    x = workload.hidden_rows(ctx, T, cfg.hidden, 302)
+    exact, fast = run_both(ctx, cfg, weights, x, T)
+    assert fast["ids"].tobytes() == exact["ids"].tobytes()
+    assert fast["weights"].tobytes() == exact["weights"].tobytes()
+    counts = np.bincount(exact["ids"].ravel(), minlength=cfg.experts)
+    assert counts.min() > 0 and counts.max() > 32, "the unskewed batch should touch every expert and need several tiles for some"
+    assert rel(fast["expert_out"], exact["expert_out"]) <= ONE_BF16_STEP
+    assert rel(fast["out"], exact["out"]) <= TOLERANCE
+    same = np.mean(fast["out"].view(np.uint32) == exact["out"].view(np.uint32))
+    print(f"T={T} unskewed: {int((counts > 0).sum())} experts used, {counts.max()} rows at most; layer output max rel err "
+          f"{rel(fast['out'], exact['out']):.3g}, identical {same:.6f}")
+    assert same > 0.9999, same
+    sample = np.random.default_rng(5).choice(T, 256, replace=False); sample.sort()
+    h = weights.host()
+    ocfg = oracle.Config(*[getattr(cfg, n) for n, _ in z.Config._fields_])
+    xs = x.numpy(f32).reshape(T, cfg.hidden)[sample]
+    want, tr = oracle.moe_layer(ocfg, h["router"], h["shared_gate"], h["shared_record"], h["records"], h["stride"],
+                                xs, len(sample), router_offsets=h["offsets"], threads=16, trace=True)
+    assert fast["ids"].reshape(T, cfg.topk)[sample].tobytes() == tr["ids"].tobytes(), "routing ids differ from the oracle"
+    assert fast["weights"].reshape(T, cfg.topk)[sample].tobytes() == tr["weights"].tobytes()
+    got = fast["out"].reshape(T, cfg.hidden)[sample]
+    assert rel(got, want) <= TOLERANCE
+    assert exact["out"].reshape(T, cfg.hidden)[sample].tobytes() == want.tobytes()   # the exact path stays byte-equal at full size
+    for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, x):
+        ctx.free(b)
+
+
+def test_prefill_reports_unroutable_rows(ctx):
+    # A NaN row gives that token no selectable expert (ids -1): its sorted positions are not covered by any tile.  The
+    # call must end normally and the check must report "invalid router output", as the exact path does.
+    cfg = workload.tiny_config(512, 32, 4, 128)
+    weights = workload.LayerWeights(ctx, cfg, 94, ("normal", 0.5))
+    T = 70
+    ws = ctx.alloc(ctx.moe_prefill_workspace_bytes(cfg, T)); out = ctx.alloc(T * cfg.hidden * 4)
+    good = workload.hidden_rows(ctx, T, cfg.hidden, 95)
+    ctx.fill(ws, 0xff)                        # whatever an earlier call could have left in the recomputation map: all bits set
+    ctx.moe_prefill(cfg, weights.layer, good, T, out, ws); ctx.moe_check()
+    want = out.numpy(f32).reshape(T, cfg.hidden).copy()
+    rows = good.numpy(f32).reshape(T, cfg.hidden).copy()
+    rows[[3, 41]] = np.nan
+    ctx.fill(ws, 0xff)
+    ctx.moe_prefill(cfg, weights.layer, ctx.upload(rows.ravel()), T, out, ws)
+    with pytest.raises(z.ZcError) as err:
+        ctx.moe_check()
+    assert "invalid router output" in str(err.value)
+    got = out.numpy(f32).reshape(T, cfg.hidden)
+    keep = np.setdiff1d(np.arange(T), [3, 41])
+    assert got[keep].tobytes() == want[keep].tobytes()      # the other tokens are untouched by their neighbours' failure
+    ctx.moe_prefill(cfg, weights.layer, good, T, out, ws); ctx.moe_check()     # and the path is usable afterwards
+    assert out.numpy(f32).tobytes() == want.tobytes()
+
+
 def test_prefill_rejects_what_it_cannot_run(ctx):
     mixed = workload.tiny_config(512, 32, 4, 128, bits=(4, 8, 8, 8))
     assert ctx.moe_prefill_workspace_bytes(mixed, 64) == 0

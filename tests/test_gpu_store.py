@@ -81,3 +81,30 @@ def test_layer_through_capped_slots_equals_resident_layer(ctx, tokens):
     st = capped.store.stats()
     assert st.misses > 6 and st.evictions > 0 and st.hits + st.misses > 0
     capped.close()
+
+
+def test_capped_layer_at_the_stack_shape_against_the_oracle(ctx):
+    # One layer of the 48-layer configuration (hidden 3072, intermediate 1024, 512 experts, top-10) whose 512 records live
+    # in pinned host memory with 24 HBM slots in front of them, checked against the CPU oracle, which reads the records'
+    # home directly: routing ids and output bytes.
+    import ctypes as C
+    import oracle
+    cfg = workload.config("F")
+    capped = workload.StoreBackedStack(ctx, cfg, [71], ("zipf", 1.1), slots=24)
+    w = capped.layers[0]
+    stride = capped.store.stride
+    home = capped.store.lib.zc_hip_store_backing(capped.store.handle, 0, 0)
+    records = np.ctypeslib.as_array(C.cast(home, C.POINTER(C.c_uint8)), shape=(cfg.experts * stride,))
+    ocfg = oracle.Config(*[getattr(cfg, n) for n, _ in z.Config._fields_])
+    for tokens, seed in ((1, 5), (3, 6), (1, 7)):
+        x = workload.hidden_rows(ctx, tokens, cfg.hidden, 950 + seed)
+        got, host_ids = capped.layer_forward(0, x, tokens)
+        want, tr = oracle.moe_layer(ocfg, w.router.numpy(np.uint16), w.shared_gate.numpy(np.uint16), w.shared_record.numpy(np.uint8),
+                                    records, stride, x.numpy(f32), tokens, router_offsets=w.offsets_host, threads=16, trace=True)
+        assert host_ids.tobytes() == tr["ids"].tobytes(), "routing ids differ from the oracle"
+        g = got.numpy(f32).reshape(tokens, cfg.hidden)
+        assert float(np.max(np.abs(g - want)) / np.max(np.abs(want))) <= 2e-3
+        assert g.tobytes() == want.tobytes()
+    st = capped.store.stats()
+    assert st.misses >= 10 and st.hits > 0      # the second and third steps find most of their experts in the slots
+    capped.close()

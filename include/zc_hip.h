@@ -165,6 +165,20 @@ uint64_t zc_hip_moe_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens);
 zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* layer,
                              const float* x, uint32_t tokens, float* out, void* workspace,
                              const zc_moe_trace* trace);
+/* zc_hip_moe_forward without a workspace argument and without any allocation.  It has no counterpart in the reference
+ * (whose scratch arenas come from Metal::allocate, metal.mm:386-433); it is for callers that cannot allocate: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The workspace lives in a static device array
+ * of zc_hip_moe_static_scratch_bytes() bytes (4 MiB) that every GPU the library runs on holds until the process ends;
+ * its address is looked up once per device in zc_hip_create.  A call whose workspace
+ * (zc_hip_moe_workspace_bytes(cfg, tokens)) does not fit is refused with ZC_INVALID_ARGUMENT and a message that names
+ * both sizes.  The call itself performs no hipMalloc / hipFree and creates no stream or event; inputs, outputs and the
+ * optional trace buffers are the caller's.  All calls on one GPU share the one array, whatever context they come
+ * through: calls that can overlap on that GPU (two contexts, two threads) race; calls on one context's stream are
+ * ordered and safe.  Nothing in the array has to start at zero (every word a kernel reads has been written by an earlier
+ * kernel of the same call), so a call leaves the previous call's contents in place without reading them. */
+uint64_t zc_hip_moe_static_scratch_bytes(void);
+zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* layer,
+                                    const float* x, uint32_t tokens, float* out, const zc_moe_trace* trace);
 /* Prefill (many tokens): the same layer with the expert products as a sorted-token grouped GEMM on the bf16 matrix
  * cores with fp32 accumulation -- what encode_expert_rows batches per expert in the reference (pipeline.cpp:7-31 over
  * q4_mm / q4_gate_up, qwen.metal:289-376).  Router ids, softmax weights and the dispatch are the exact kernels (bit-equal

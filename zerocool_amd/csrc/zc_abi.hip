@@ -10,7 +10,17 @@
 #include <unordered_map>
 #include <vector>
 
+// Scratch of the allocation-free entry point (zc_hip_moe_forward_static): the workspace that zc_hip_moe_forward takes
+// as an argument, as a static device array.  Every GPU the library runs on holds its own copy at its own address until
+// the process ends; g_scratch[device] is that address, looked up once per device in zc_hip_create.  Host code never
+// uses the array's name as an address: the name is only a handle for hipGetSymbolAddress.
+constexpr uint64_t kStaticScratchBytes = 4ull << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
 thread_local std::string g_error;
 zc_status fail(zc_status code, std::string text) { g_error = std::move(text); return code; }
 }  // namespace
@@ -44,6 +54,7 @@ struct zc_hip_ctx {
     int32_t* moe_status = nullptr;     // device flag: an id outside [0,E) was seen
     hipEvent_t timer[2] = {nullptr, nullptr};
     uint32_t affine_policy = 1;        // 0 literal lane kernels, 1 exact-integer matrix-core kernels where possible
+    void* static_scratch = nullptr;    // this device's copy of the static scratch array
     std::mutex mutex;
 };
 
@@ -58,8 +69,18 @@ zc_status zc_hip_create(int device, uint64_t budget_bytes, zc_hip_ctx** out) {
     ZC_HIP(hipGetDeviceCount(&count));
     if (device < 0 || device >= count) return fail(ZC_RUNTIME_ERROR, "no such HIP device");
     ZC_HIP(hipSetDevice(device));
+    void* device_scratch = nullptr;
+    {   // once per device, with that device current: where this GPU keeps its copy of the static scratch array
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (device < kMaxDevices && g_scratch[device]) device_scratch = g_scratch[device];
+        else {
+            const hipError_t e = hipGetSymbolAddress(&device_scratch, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !device_scratch) return fail(ZC_RUNTIME_ERROR, std::string("HIP execution: cannot locate the static scratch array: ") + hipGetErrorString(e));
+            if (device < kMaxDevices) g_scratch[device] = device_scratch;
+        }
+    }
     auto* ctx = new zc_hip_ctx;
-    ctx->device = device; ctx->budget = budget_bytes;
+    ctx->device = device; ctx->budget = budget_bytes; ctx->static_scratch = device_scratch;
     if (hipStreamCreate(&ctx->stream) != hipSuccess) { delete ctx; return fail(ZC_RUNTIME_ERROR, "HIP execution: cannot create stream"); }
     if (hipMalloc(&ctx->moe_status, 256) != hipSuccess || hipMemsetAsync(ctx->moe_status, 0, 256, ctx->stream) != hipSuccess) {
         hipStreamDestroy(ctx->stream); delete ctx; return fail(ZC_RUNTIME_ERROR, "HIP execution: cannot allocate status word");
@@ -412,6 +433,23 @@ Workspace carve(const zc_moe_config* c, uint32_t T, void* base) {
 uint64_t zc_hip_moe_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens) {
     if (validate_config(cfg) != ZC_OK || !tokens) return 0;
     return carve(cfg, tokens, nullptr).bytes;
+}
+uint64_t zc_hip_moe_static_scratch_bytes(void) { return kStaticScratchBytes; }
+// zc_hip_moe_forward with its workspace in the static scratch array of the context's device.  Nothing on this path
+// allocates or frees: no hipMalloc / hipFree / hipHostMalloc, no stream or event creation, no host containers.
+zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
+                                    float* out, const zc_moe_trace* trace) {
+    if (const zc_status s = validate_config(c)) return s;
+    ZC_REQUIRE(ctx && T, "invalid MoE layer buffers");
+    ZC_REQUIRE(ctx->static_scratch, "the static scratch array was not located for this device");
+    const uint64_t need = carve(c, T, nullptr).bytes;
+    if (need > kStaticScratchBytes) {
+        char text[200];
+        snprintf(text, sizeof text, "zc_hip_moe_forward_static: %u tokens of this shape need %llu bytes of scratch, the static array holds %llu; use zc_hip_moe_forward with a workspace",
+                 T, (unsigned long long)need, (unsigned long long)kStaticScratchBytes);
+        return fail(ZC_INVALID_ARGUMENT, text);
+    }
+    return zc_hip_moe_forward(ctx, c, l, x, T, out, ctx->static_scratch, trace);
 }
 zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
                              float* out, void* workspace, const zc_moe_trace* trace) {

@@ -52,7 +52,7 @@ def load_library():
     lib.zc_hip_last_error.restype = C.c_char_p
     lib.zc_hip_version.restype = C.c_char_p
     for name in ("zc_hip_allocated", "zc_hip_peak", "zc_hip_moe_workspace_bytes", "zc_hip_moe_prefill_workspace_bytes", "zc_hip_projection_bytes",
-                 "zc_hip_record_bytes", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy"):
+                 "zc_hip_record_bytes", "zc_hip_moe_static_scratch_bytes", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy"):
         getattr(lib, name).restype = C.c_uint64
     lib.zc_hip_stream.restype = C.c_void_p
     lib.zc_hip_store_backing.restype = C.c_void_p
@@ -349,6 +349,11 @@ class Context:
     def moe_forward(self, cfg, layer, x, tokens, out, workspace, trace=None):
         self._call("zc_hip_moe_forward", C.byref(cfg), C.byref(layer), _ptr(x), C.c_uint32(tokens), _ptr(out),
                    _ptr(workspace), C.byref(trace) if trace is not None else None)
+
+    def moe_forward_static(self, cfg, layer, x, tokens, out, trace=None):
+        """zc_hip_moe_forward with its workspace in the library's static device array: allocates nothing."""
+        self._call("zc_hip_moe_forward_static", C.byref(cfg), C.byref(layer), _ptr(x), C.c_uint32(tokens), _ptr(out),
+                   C.byref(trace) if trace is not None else None)
 
     def moe_prefill_workspace_bytes(self, cfg, tokens):
         return self.lib.zc_hip_moe_prefill_workspace_bytes(C.byref(cfg), C.c_uint32(tokens))

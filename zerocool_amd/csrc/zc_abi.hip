@@ -668,7 +668,7 @@ struct zc_hip_stack {
     // persistent path
     zc::DecodeLayer* dev_layers = nullptr;
     uint8_t* arena = nullptr; uint64_t arena_bytes = 0;
-    float *logits = nullptr, *gate = nullptr, *shared_act = nullptr, *act = nullptr, *layer_out = nullptr;
+    float *logits = nullptr, *gate = nullptr, *shared_act = nullptr, *act = nullptr, *layer_out = nullptr, *eout = nullptr;
     uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
     unsigned long long* tlogits = nullptr; uint32_t *tact = nullptr, *tout = nullptr;   // tagged exchange buffers of the one-token kernel
     uint32_t epoch = 1u << 12;
@@ -724,7 +724,7 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         auto take = [&](uint64_t bytes) { const uint64_t o = at; at += align_up(bytes, 256); return o; };
         const uint64_t o_layers = take(sizeof(zc::DecodeLayer) * n_layers), o_logits = take(uint64_t(Tp) * E * 4), o_gate = take(Tp * 4),
                        o_sact = take(uint64_t(Tp) * I * 4), o_act = take(uint64_t(Tp) * k * I * 4), o_lout = take(uint64_t(Tp) * H * 4),
-                       o_max = take(uint64_t(n_layers) * Tp * 4), o_sync = take(zc::kDecodeSyncBytes),
+                       o_max = take(uint64_t(n_layers) * Tp * 4), o_sync = take(zc::kDecodeSyncBytes), o_eout = take(uint64_t(Tp) * (k + 1) * H * 4),
                        o_tlogits = take(uint64_t(E + 1) * 8), o_tact = take(uint64_t(k + 1) * I * 4), o_tout = take(uint64_t(2) * H * 4);
         if (zc_hip_alloc(ctx, at, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
         st->arena = static_cast<uint8_t*>(p); st->arena_bytes = at;
@@ -732,7 +732,7 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         st->logits = reinterpret_cast<float*>(st->arena + o_logits); st->gate = reinterpret_cast<float*>(st->arena + o_gate);
         st->shared_act = reinterpret_cast<float*>(st->arena + o_sact); st->act = reinterpret_cast<float*>(st->arena + o_act);
         st->layer_out = reinterpret_cast<float*>(st->arena + o_lout); st->maxabs = reinterpret_cast<uint32_t*>(st->arena + o_max);
-        st->sync = reinterpret_cast<uint32_t*>(st->arena + o_sync);
+        st->sync = reinterpret_cast<uint32_t*>(st->arena + o_sync); st->eout = reinterpret_cast<float*>(st->arena + o_eout);
         st->tlogits = reinterpret_cast<unsigned long long*>(st->arena + o_tlogits); st->tact = reinterpret_cast<uint32_t*>(st->arena + o_tact);
         st->tout = reinterpret_cast<uint32_t*>(st->arena + o_tout);
         std::vector<zc::DecodeLayer> host(n_layers);
@@ -757,16 +757,22 @@ zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* st) {
     delete st;
     return ZC_OK;
 }
-static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, zc::DecodeLdsPlan* plan, uint32_t* nt) {
+static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, zc::DecodeLdsPlan* plan, zc::MultiLdsPlan* multi, uint32_t* nt) {
     if (!st->persistent_ok || tokens > 8 || tokens > st->max_tokens) return false;
     const zc_moe_config& c = st->cfg;
     *nt = token_tile(tokens);
     if (tokens * c.topk > 256) return false;
-    *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
-    if (plan->total > st->lds_limit || plan->slots_per_batch == 0) return false;
     int per_cu = 0;
-    if (zc::decode_stack_occupancy(*nt, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
     (void)ctx;
+    if (*nt == 1) {
+        *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
+        if (plan->total > st->lds_limit || plan->slots_per_batch == 0) return false;
+        if (zc::decode_stack_occupancy(*nt, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+    } else {
+        *multi = zc::decode_multi_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
+        if (multi->total > st->lds_limit) return false;
+        if (zc::decode_multi_occupancy(multi->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+    }
     return per_cu >= 1;
 }
 zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t polls) {
@@ -776,8 +782,8 @@ zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_
 }
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
     if (!ctx || !st) return 0;
-    zc::DecodeLdsPlan plan; uint32_t nt;
-    return persistent_plan(ctx, st, tokens, &plan, &nt) ? 1 : 0;
+    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt;
+    return persistent_plan(ctx, st, tokens, &plan, &multi, &nt) ? 1 : 0;
 }
 zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
                               const zc_stack_trace* trace, uint32_t flags) {
@@ -785,8 +791,8 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
     ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && x != out, "invalid or overlapping linear output");
     const zc_moe_config& c = st->cfg;
     const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
-    zc::DecodeLdsPlan plan; uint32_t nt = 0;
-    if (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &nt)) {
+    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt = 0;
+    if (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt)) {
         zc::DecodeParams p{};
         p.H = H; p.E = c.experts; p.topk = k; p.I = c.inter; p.T = tokens; p.L = L;
         for (int shared = 0; shared < 2; ++shared)
@@ -798,20 +804,21 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
             }
         p.layers = st->dev_layers; p.x_in = x; p.out = out;
         p.logits = st->logits; p.gate = st->gate; p.shared_act = st->shared_act; p.act = st->act; p.layer_out = st->layer_out;
-        p.maxabs = st->maxabs;
+        p.maxabs = st->maxabs; p.eout = st->eout;
         p.tlogits = st->tlogits; p.tact = st->tact; p.tout = st->tout;
         p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
         if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
         p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
-        st->epoch += 3 * L + 16;   // wraps modulo 2^32; the barrier compares epochs as signed differences
+        st->epoch += 4 * L + 16;   // at most four barriers per layer; wraps modulo 2^32, the barrier compares epochs as signed differences
         // The tagged buffers are written by one-token launches only, so their tags advance with those launches only:
         // a launch's layer 0 then expects the tag right after the one its predecessor's last layer left, however many
         // launches of the other kernel ran in between.
         p.tag_base = st->tag_base;
         if (nt == 1) st->tag_base = (st->tag_base + L) % 65535u;
         const uint32_t workgroups = uint32_t(st->cus);
-        ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
+        if (nt == 1) ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
+        else ZC_HIP(zc::launch_decode_multi(ctx->stream, p, workgroups, multi));
         return ZC_OK;
     }
     // layer by layer: y = moe(x); x_next = glue(y)

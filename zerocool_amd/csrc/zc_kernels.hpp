@@ -65,6 +65,7 @@ struct DecodeParams {
     const DecodeLayer* layers;       // device array [L]
     const float* x_in; float* out;   // [T][H]
     float *logits, *gate, *shared_act, *act, *layer_out;   // exchange buffers
+    float* eout;                     // several tokens: down outputs per slot, [T * topk + T][H] (the last T rows: the shared expert's)
     uint32_t* maxabs;                // [L][T] bit patterns of max |layer output|
     // One token: the exchange buffers carry a tag beside every value, so that a reader polls the data itself instead of
     // waiting at a grid barrier and fetching afterwards.  tlogits [E + 1] words {fp32 bits, tag << 32} (word E: the shared
@@ -84,6 +85,14 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
 hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp);
 hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu);
 constexpr uint32_t kDecodeSyncBytes = (32 * 1024 + 16 * 64) * 4;
+// Two to eight tokens (zc_decode_multi.hip)
+struct MultiLdsPlan {
+    uint32_t ids, weights, gatev, head, next, experts, misc, gatew, region, total;
+    uint32_t img_x, xh, img_d, ah, cum;
+};
+MultiLdsPlan decode_multi_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t T, uint32_t lds_limit);
+hipError_t launch_decode_multi(hipStream_t s, const DecodeParams& p, uint32_t workgroups, const MultiLdsPlan& lp);
+hipError_t decode_multi_occupancy(uint32_t lds_bytes, int* blocks_per_cu);
 
 // ---- prefill: sorted-token grouped GEMM on the bf16 matrix cores (zc_prefill.hip)
 struct PrefillGemm {

@@ -359,6 +359,289 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
     }
 }
 
+// The literal fp32 chain of one block (reference: qwen.metal:52-57) from the block's two raw code words (nibble i of word w
+// is element 8 w + i) and the block's sixteen BF16 inputs in LDS.  Written as a loop over the four quads so that it is
+// small in code and registers: it runs inside the tile engines, whose registers are full.
+__device__ __forceinline__ float xint_literal_block(const uint16_t* x_block, uint32_t w_lo, uint32_t w_hi) {
+    float dot = 0;
+#pragma unroll 1
+    for (int quad = 0; quad < 4; ++quad) {
+        const uint2 xv = *reinterpret_cast<const uint2*>(x_block + 4 * quad);
+        const uint32_t nib = ((quad & 2 ? w_hi : w_lo) >> (16 * (quad & 1))) & 0xffffu;
+        const float a = __uint_as_float(xv.x << 16), c = __uint_as_float(xv.x & 0xffff0000u);
+        const float d = __uint_as_float(xv.y << 16), e = __uint_as_float(xv.y & 0xffff0000u);
+        // BF16-valued inputs times 4-bit codes are exact products: a fused multiply-add equals the reference's multiply and add
+        dot += __builtin_fmaf(e, float(nib >> 12), __builtin_fmaf(d, float((nib >> 8) & 15u), __builtin_fmaf(c, float((nib >> 4) & 15u), a * float(nib & 15u))));
+    }
+    return dot;
+}
+
+// The same tile for NTOK tokens that share the tile's weights (the tokens of a decode step routed to one expert), for
+// workgroups that run two waves per SIMD (the other wave covers this one's LDS and MFMA latencies, so the tokens of a span
+// are simply taken in turn).  Per span: the codes are expanded once; every token's block dots come from the MFMAs; then
+// ONE loop serves the literal chains of all tokens: every lane takes its next unsafe (token, block) in turn until no lane
+// has one left, so the chain's code exists once per span and its cost follows the busiest lane group, not the number
+// of tokens; then the accumulators are updated in span order.  src must be BF16 rows in LDS.  Images beyond the live
+// tokens (t >= nt) must point at valid images; their sums are computed and dropped.  Per-lane accumulation order and the
+// final butterfly are those of xint_run_tile_after.
+template <int NTOK, int R, class Emit>
+__device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                                     const uint8_t* const* img, const LdsBf16* src, const XintLayout L, uint32_t lane,
+                                                     int nt, Emit emit) {
+    static_assert(R == 4, "bodies of four spans: one mask word per token covers a body");
+    static_assert(NTOK >= 1 && NTOK <= 8, "the pending set of a lane is sixteen bits");
+    const uint32_t G = lane >> 4, row_a = lane & 15u, c_a = row_a >> 2, p_a = row_a & 3u;
+    const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
+    uint4 ring[R], sring, bring;
+#pragma unroll
+    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
+    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
+    float acc[NTOK][4][2];
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
+    const uint32_t shamt = (lane & 32u) ? 0u : 16u;   // group 2d + (G >> 1): low half for G < 2
+    const bool live = (c_a == G) && p_a < 3;
+    const uint32_t a_first = live ? 2 * G * 48 + p_a * 16 : L.blocks() * 48, a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
+    const uint32_t M = 0x0f0f0f0fu;
+    const v4i zero = {0, 0, 0, 0};
+    const uint32_t info_at = L.planes_bytes() + 2 * G * 8, mask_at = L.planes_bytes() + L.info_bytes();
+    for (uint32_t d0 = 0; d0 < spans; d0 += R) {
+        uint4 codes[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) codes[j] = ring[j];
+        const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
+        if (d0 + R < spans) {
+#pragma unroll
+            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
+            sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4);
+        }
+        // the unsafe bits of this body's blocks, per token: blocks 8d + 2G + h of spans d0 .. d0+3 sit in mask word d0/4,
+        // moved down so that bits 8j, 8j+1 are the lane's two blocks of span j
+        uint32_t unsafe[NTOK], any = 0;
+#pragma unroll
+        for (int t = 0; t < NTOK; ++t) {
+            unsafe[t] = (reinterpret_cast<const uint32_t*>(img[t] + mask_at)[d0 / 4] >> (2 * G)) & 0x03030303u;
+            any |= unsafe[t];
+        }
+        const bool literal_body = __ballot(any != 0) != 0;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint32_t d = d0 + uint32_t(j);
+            const v4i b0 = {int(codes[j].x & M), int((codes[j].x >> 4) & M), int(codes[j].y & M), int((codes[j].y >> 4) & M)};
+            const v4i b1 = {int(codes[j].z & M), int((codes[j].z >> 4) & M), int(codes[j].w & M), int((codes[j].w >> 4) & M)};
+            float dot[NTOK][2], bsum[NTOK][2];
+#pragma unroll
+            for (int t = 0; t < NTOK; ++t) {
+                const uint8_t* a_at = img[t] + a_first + d * a_span;
+                const v4i a0 = *reinterpret_cast<const v4i*>(a_at), a1 = *reinterpret_cast<const v4i*>(a_at + a_next);
+                const float4 fi = *reinterpret_cast<const float4*>(img[t] + info_at + d * 64);   // {2^e, sum} of blocks 2G, 2G+1
+                const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
+                const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, zero, 0, 0, 0);
+                // digits recombined by Horner's rule: ((d2 << 7) + d1 << 7) + d0
+                dot[t][0] = float((((r0[2] << 7) + r0[1]) << 7) + r0[0]) * fi.x; bsum[t][0] = fi.y;
+                dot[t][1] = float((((r1[2] << 7) + r1[1]) << 7) + r1[0]) * fi.z; bsum[t][1] = fi.w;
+            }
+#ifndef ZC_TIMING_NO_LITERAL
+            if (__builtin_expect(literal_body, 0)) {
+                // pending (token, block) pairs of this lane in span j: bit 2t + h
+                uint32_t pending = 0;
+#pragma unroll
+                for (int t = 0; t < NTOK; ++t) pending |= ((unsafe[t] >> (8 * j)) & 3u) << (2 * t);
+                while (__ballot(pending != 0) != 0) {
+                    if (pending) {
+                        const uint32_t item = uint32_t(__builtin_ctz(pending)), t = item >> 1, h = item & 1u;
+                        const uint16_t* row = src[0].x;
+#pragma unroll
+                        for (int q = 1; q < NTOK; ++q) row = t == uint32_t(q) ? src[q].x : row;
+                        const float lit = xint_literal_block(row + (8 * d + 2 * G + h) * 16, h ? codes[j].z : codes[j].x, h ? codes[j].w : codes[j].y);
+#pragma unroll
+                        for (int q = 0; q < NTOK; ++q) {
+                            dot[q][0] = item == uint32_t(2 * q) ? lit : dot[q][0];
+                            dot[q][1] = item == uint32_t(2 * q + 1) ? lit : dot[q][1];
+                        }
+                        pending &= pending - 1;
+                    }
+                }
+            }
+#endif
+            const float scale = __uint_as_float((sdw[j] << shamt) & 0xffff0000u), bias = __uint_as_float((bdw[j] << shamt) & 0xffff0000u);
+#pragma unroll
+            for (int t = 0; t < NTOK; ++t) {
+                acc[t][j][0] += scale * dot[t][0] + bsum[t][0] * bias;
+                acc[t][j][1] += scale * dot[t][1] + bsum[t][1] * bias;
+            }
+        }
+    }
+    // Reference lane sum (xor butterfly 16, 8, 4, 2, 1): strides 16 and 8 pair accumulators, 4 and 2 pair lane groups, 1 the two blocks of a lane.
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+        float v[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float x0 = acc[t][0][h] + acc[t][2][h], x1 = acc[t][1][h] + acc[t][3][h];
+            float sum = x0 + x1;
+            sum = sum + __shfl_xor(sum, 32);
+            sum = sum + __shfl_xor(sum, 16);
+            v[h] = sum;
+        }
+        if (t < nt) emit(t, v[0] + v[1]);
+    }
+}
+// The same for workgroups that run ONE wave per SIMD (the whole register file, up to eight tokens per pass): there is no
+// other wave to cover this one's LDS and MFMA latencies, so the work of a body is cut into steps of at most four tokens of
+// one span and software-pipelined by hand: the MFMAs of step s are issued back to back, then the LDS reads of step s + 1
+// (into the other operand buffer), then the vector work of step s.  Scheduling barriers keep the compiler from folding
+// the stages of a token back into one dependent chain.
+template <int NTOK, int R, class Emit>
+__device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                                           const uint8_t* const* img, const LdsBf16* src, const XintLayout L, uint32_t lane,
+                                                           int nt, Emit emit) {
+    static_assert(R == 4, "bodies of four spans: one mask word per token covers a body");
+    static_assert(NTOK == 1 || NTOK == 2 || NTOK == 4 || NTOK == 8, "token counts are rounded up to 1, 2, 4 or 8");
+    constexpr int TG = NTOK < 4 ? NTOK : 4, GROUPS = NTOK / TG, STEPS = R * GROUPS;
+    const uint32_t G = lane >> 4, row_a = lane & 15u, c_a = row_a >> 2, p_a = row_a & 3u;
+    const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
+    uint4 ring[R], sring, bring;
+#pragma unroll
+    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
+    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
+    float acc[NTOK][4][2];
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
+    const uint32_t shamt = (lane & 32u) ? 0u : 16u;   // group 2d + (G >> 1): low half for G < 2
+    const bool live = (c_a == G) && p_a < 3;
+    const uint32_t a_first = live ? 2 * G * 48 + p_a * 16 : L.blocks() * 48, a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
+    const uint32_t M = 0x0f0f0f0fu;
+    const v4i zero = {0, 0, 0, 0};
+    const uint32_t info_at = L.planes_bytes() + 2 * G * 8, mask_at = L.planes_bytes() + L.info_bytes();
+    // lane q < NTOK holds where token q's BF16 row starts, in elements from src[0]'s (a select chain over the tokens would be
+    // turned into a table in memory by the compiler)
+    uint32_t row_table = 0;
+#pragma unroll
+    for (int q = 1; q < NTOK; ++q) row_table = lane == uint32_t(q) ? uint32_t(src[q].x - src[0].x) : row_table;
+    for (uint32_t d0 = 0; d0 < spans; d0 += R) {
+        uint4 codes[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) codes[j] = ring[j];
+        const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
+        if (d0 + R < spans) {
+#pragma unroll
+            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
+            sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4);
+        }
+        uint32_t unsafe[NTOK], any = 0;
+#pragma unroll
+        for (int t = 0; t < NTOK; ++t) {
+            unsafe[t] = (reinterpret_cast<const uint32_t*>(img[t] + mask_at)[d0 / 4] >> (2 * G)) & 0x03030303u;
+            any |= unsafe[t];
+        }
+#ifdef ZC_TIMING_NO_LITERAL
+        const bool literal_body = false;
+#else
+        const bool literal_body = __ballot(any != 0) != 0;
+#endif
+        // operand buffers of two steps: A operands (digit planes of blocks 2G, 2G+1) and {2^e, sum} pairs of those blocks
+        v4i a0[2][TG], a1[2][TG]; float4 fi[2][TG];
+        auto load = [&](int buf, int step) {
+            const uint32_t d = d0 + uint32_t(step / GROUPS);
+            const int g = step % GROUPS;
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+                const uint8_t* image = img[g * TG + t];
+                const uint8_t* a_at = image + a_first + d * a_span;
+                a0[buf][t] = *reinterpret_cast<const v4i*>(a_at); a1[buf][t] = *reinterpret_cast<const v4i*>(a_at + a_next);
+                fi[buf][t] = *reinterpret_cast<const float4*>(image + info_at + d * 64);
+            }
+        };
+        load(0, 0);
+#pragma unroll
+        for (int step = 0; step < STEPS; ++step) {
+            const int j = step / GROUPS, g = step % GROUPS, buf = step & 1;
+            const uint32_t d = d0 + uint32_t(j);
+            const v4i b0 = {int(codes[j].x & M), int((codes[j].x >> 4) & M), int(codes[j].y & M), int((codes[j].y >> 4) & M)};
+            const v4i b1 = {int(codes[j].z & M), int((codes[j].z >> 4) & M), int(codes[j].w & M), int((codes[j].w >> 4) & M)};
+            v4i r0[TG], r1[TG];
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+                r0[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[buf][t], b0, zero, 0, 0, 0);
+                r1[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[buf][t], b1, zero, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (step + 1 < STEPS) load(buf ^ 1, step + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            float dot[TG][2];
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+                // digits recombined by Horner's rule: ((d2 << 7) + d1 << 7) + d0
+                dot[t][0] = float((((r0[t][2] << 7) + r0[t][1]) << 7) + r0[t][0]) * fi[buf][t].x;
+                dot[t][1] = float((((r1[t][2] << 7) + r1[t][1]) << 7) + r1[t][0]) * fi[buf][t].z;
+            }
+            if (__builtin_expect(literal_body, 0)) {
+                // pending (token, block) pairs of this lane in this step: bit 2t + h; every lane takes its next one in turn
+                uint32_t pending = 0;
+#pragma unroll
+                for (int t = 0; t < TG; ++t) pending |= ((unsafe[g * TG + t] >> (8 * j)) & 3u) << (2 * t);
+                while (__ballot(pending != 0) != 0) {
+                    // (every lane is active here: the row of token t is lane t's entry of the table, fetched across lanes)
+                    const uint32_t item = uint32_t(__builtin_ctz(pending | 0x80000000u)), t = item >> 1, h = item & 1u;
+                    const uint32_t row_at = uint32_t(__builtin_amdgcn_ds_bpermute(int(4 * (uint32_t(g * TG) + (t & uint32_t(TG - 1)))), int(row_table)));
+                    if (pending) {
+                        const uint16_t* row = src[0].x + int32_t(row_at);   // (a signed distance)
+                        const float lit = xint_literal_block(row + (8 * d + 2 * G + h) * 16, h ? codes[j].z : codes[j].x, h ? codes[j].w : codes[j].y);
+#pragma unroll
+                        for (int q = 0; q < TG; ++q) {
+                            dot[q][0] = item == uint32_t(2 * q) ? lit : dot[q][0];
+                            dot[q][1] = item == uint32_t(2 * q + 1) ? lit : dot[q][1];
+                        }
+                        pending &= pending - 1;
+                    }
+                }
+            }
+            const float scale = __uint_as_float((sdw[j] << shamt) & 0xffff0000u), bias = __uint_as_float((bdw[j] << shamt) & 0xffff0000u);
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+                acc[g * TG + t][j][0] += scale * dot[t][0] + fi[buf][t].y * bias;
+                acc[g * TG + t][j][1] += scale * dot[t][1] + fi[buf][t].w * bias;
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+        float v[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float x0 = acc[t][0][h] + acc[t][2][h], x1 = acc[t][1][h] + acc[t][3][h];
+            float sum = x0 + x1;
+            sum = sum + __shfl_xor(sum, 32);
+            sum = sum + __shfl_xor(sum, 16);
+            v[h] = sum;
+        }
+        if (t < nt) emit(t, v[0] + v[1]);
+    }
+}
+template <class Emit>
+__device__ __forceinline__ void xint_run_tile_upto8(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                                    const uint8_t* const* img, const LdsBf16* src, const XintLayout L, uint32_t lane,
+                                                    int nt, Emit emit) {
+    if (nt <= 1) xint_run_tile_tokens_piped<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    else if (nt == 2) xint_run_tile_tokens_piped<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    else if (nt <= 4) xint_run_tile_tokens_piped<4, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    else xint_run_tile_tokens_piped<8, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+}
+// Picks the instance for the number of live tokens: 1, 2 or 4 (the count is rounded up; padded tokens repeat image 0).
+template <class Emit>
+__device__ __forceinline__ void xint_run_tile_upto4(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                                    const uint8_t* const* img, const LdsBf16* src, const XintLayout L, uint32_t lane,
+                                                    int nt, Emit emit) {
+    if (nt <= 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    else if (nt == 2) xint_run_tile_tokens<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    else xint_run_tile_tokens<4, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+}
+
 template <int PT, int R, class Source, class Emit>
 __device__ __forceinline__ void xint_run_tile(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
                                               const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,

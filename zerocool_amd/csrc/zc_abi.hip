@@ -724,7 +724,7 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         auto take = [&](uint64_t bytes) { const uint64_t o = at; at += align_up(bytes, 256); return o; };
         const uint64_t o_layers = take(sizeof(zc::DecodeLayer) * n_layers), o_logits = take(uint64_t(Tp) * E * 4), o_gate = take(Tp * 4),
                        o_sact = take(uint64_t(Tp) * I * 4), o_act = take(uint64_t(Tp) * k * I * 4), o_lout = take(uint64_t(Tp) * H * 4),
-                       o_max = take(uint64_t(n_layers) * Tp * 4), o_sync = take(zc::kDecodeSyncBytes), o_eout = take(uint64_t(Tp) * (k + 1) * H * 4),
+                       o_max = take(std::max<uint64_t>(uint64_t(n_layers) * Tp * 4, uint64_t(Tp) * (H / 64 + 1) * 4)), o_sync = take(zc::kDecodeSyncBytes), o_eout = take(uint64_t(Tp) * (k + 1) * H * 4),
                        o_tlogits = take(uint64_t(E + 1) * 8), o_tact = take(uint64_t(k + 1) * I * 4), o_tout = take(uint64_t(2) * H * 4);
         if (zc_hip_alloc(ctx, at, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
         st->arena = static_cast<uint8_t*>(p); st->arena_bytes = at;

@@ -48,7 +48,7 @@ __device__ __forceinline__ void run_tile(const uint8_t* w_row, const uint16_t* s
     else if constexpr (kPassTokens == 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     else if constexpr (kPassTokens == 2) {
         if (nt <= 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
-        else xint_run_tile_tokens<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+        else xint_run_tile_tokens_piped<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     } else xint_run_tile_upto4(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
 }
 
@@ -74,7 +74,6 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
     auto clock = [&]() { if (p.clocks && tid == 0) p.clocks[uint64_t(stamp) * nwg + wg] = wall_clock64(); ++stamp; };
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };
 
-    if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
     // SwiGLU of a finished gate/up tile (gate rows in columns 0-7, up rows in 8-15), stored as packed BF16 pairs: the lane
     // of an even row writes rows r and r+1 of activation row `slot_row` as one word.
     auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {
@@ -107,12 +106,19 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
         const uint32_t pairs = (T + 1) / 2, router_units = ((E + 3) / 4) * pairs, gate_units = (T + 1) / 2;
         constexpr int kPieces = 24;   // sixteen-byte pieces of a K partition at hidden 3072
         const uint32_t u_first = wg + nwg * wave;
+        const bool ahead = H / 128 <= uint32_t(kPieces);
         {
             const bool glue = layer != 0;
             // the glue's scale per token: 1 / max|y| of the previous layer
-            if (glue && tid < T) {
-                const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
-                gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
+            if (glue) {   // the largest magnitude of every row: the combine left one candidate per 64 columns
+                const uint32_t groups = H / 64;
+                uint32_t m = 0;
+                for (uint32_t g = lane; g < groups; g += 64) if (wave < T) m = max(m, ZC_LD(p.maxabs + wave * groups + g));
+                m = __float_as_uint(wave_max_f32(__uint_as_float(m)));
+                if (wave < T && lane == 0) {
+                    const float v = __uint_as_float(m);
+                    gatev[wave] = (v > 0.0f && v < __uint_as_float(0x7f800000u)) ? 1.0f / v : 1.0f;
+                }
             }
             __syncthreads();
             const int bad = stage_bf16<12>(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), []() {},
@@ -129,14 +135,6 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
         // workgroup build the tokens' images meanwhile.  With more units than waves (a small grid) every wave does both.
         const bool all_build = router_units + gate_units > nwg * kMultiWaves;
         const uint32_t builders_from = all_build ? 0u : min(kMultiWaves - 1, (router_units + gate_units - min(wg, router_units + gate_units) + nwg - 1) / nwg);
-        if (wave >= builders_from) {
-            const uint32_t builders = (kMultiWaves - builders_from) * 64u, blocks = LH.blocks();
-            for (uint32_t i = tid - builders_from * 64u; i < T * blocks; i += builders) {
-                const uint32_t q = i / blocks;
-                xint_prepare_block(LdsBf16{xh + q * H}, LH, lds + lp.img_x + q * LH.bytes(), i % blocks);
-            }
-        }
-        const bool ahead = H / 128 <= uint32_t(kPieces);
         for (uint32_t u = u_first; u < router_units + gate_units; u += nwg * kMultiWaves) {
             if (u < router_units) {
                 const uint32_t t0 = (u % pairs) * 2, e = (u / pairs) * 4 + lane / 16, split = lane % 16, P = H / 16;
@@ -205,6 +203,13 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                     }
                 sum = lane_sum32(sum);
                 if (t < T && l32 == 0) st_f32(p.gate + t, bf(sum));
+            }
+        }
+        if (wave >= builders_from) {
+            const uint32_t builders = (kMultiWaves - builders_from) * 64u, blocks = LH.blocks();
+            for (uint32_t i = tid - builders_from * 64u; i < T * blocks; i += builders) {
+                const uint32_t q = i / blocks;
+                xint_prepare_block(LdsBf16{xh + q * H}, LH, lds + lp.img_x + q * LH.bytes(), i % blocks);
             }
         }
         clock_all();
@@ -430,7 +435,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
             if (m > 0x7f800000u) m = 0;   // NaN does not take part in the maximum
             // the lanes of a wave hold consecutive columns; a wave may straddle two tokens only when H is not a multiple of 64
             m = __float_as_uint(wave_max_f32(__uint_as_float(m)));
-            if (lane == 0) __hip_atomic_fetch_max(p.maxabs + layer * T + t, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) ZC_ST(p.maxabs + group, m);   // group = t * (H / 64) + column group: read by the next layer's staging
         }
         clock_all();
         bar.wait();

@@ -359,6 +359,12 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
     }
 }
 
+// (timing experiments only: -DZC_TIMING_NO_WEIGHTS feeds the tile engines register constants instead of weights)
+#ifdef ZC_TIMING_NO_WEIGHTS
+#define ZC_TILE_LOAD(p, i) make_uint4(0x12345678u + uint32_t(i), 0x9abcdef0u ^ lane, 0x3c003c00u, 0x0f1e2d3cu + uint32_t(i))
+#else
+#define ZC_TILE_LOAD(p, i) ldg_u4(p, i)
+#endif
 // The literal fp32 chain of one block (reference: qwen.metal:52-57) from the block's two raw code words (nibble i of word w
 // is element 8 w + i) and the block's sixteen BF16 inputs in LDS.  Written as a loop over the four quads so that it is
 // small in code and registers: it runs inside the tile engines, whose registers are full.
@@ -394,8 +400,8 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
     const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
     uint4 ring[R], sring, bring;
 #pragma unroll
-    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
-    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
+    for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, j * 4);
+    sring = ZC_TILE_LOAD(s_row, 0); bring = ZC_TILE_LOAD(b_row, 0);
     float acc[NTOK][4][2];
 #pragma unroll
     for (int t = 0; t < NTOK; ++t)
@@ -414,8 +420,8 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
         const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
         if (d0 + R < spans) {
 #pragma unroll
-            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
-            sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4);
+            for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, (d0 + j + R) * 4);
+            sring = ZC_TILE_LOAD(s_row, (d0 + R) / 4); bring = ZC_TILE_LOAD(b_row, (d0 + R) / 4);
         }
         // the unsafe bits of this body's blocks, per token: blocks 8d + 2G + h of spans d0 .. d0+3 sit in mask word d0/4,
         // moved down so that bits 8j, 8j+1 are the lane's two blocks of span j
@@ -505,8 +511,8 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
     const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
     uint4 ring[R], sring, bring;
 #pragma unroll
-    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
-    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
+    for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, j * 4);
+    sring = ZC_TILE_LOAD(s_row, 0); bring = ZC_TILE_LOAD(b_row, 0);
     float acc[NTOK][4][2];
 #pragma unroll
     for (int t = 0; t < NTOK; ++t)
@@ -530,8 +536,8 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
         const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
         if (d0 + R < spans) {
 #pragma unroll
-            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
-            sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4);
+            for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, (d0 + j + R) * 4);
+            sring = ZC_TILE_LOAD(s_row, (d0 + R) / 4); bring = ZC_TILE_LOAD(b_row, (d0 + R) / 4);
         }
         uint32_t unsafe[NTOK], any = 0;
 #pragma unroll

@@ -225,6 +225,12 @@ int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* stack, uint32_t to
  * stays usable.  No counterpart in the reference (its command buffers cannot wait on each other); tests use a bound of
  * one poll to exercise the give-up path without a lost workgroup. */
 zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* stack, uint32_t polls);
+/* One-token launches of the persistent kernel start every layer's gate/up tiles on the experts that layer picked at the
+ * previous one-token step, before this step's ids are known, and redo only the slots that were guessed wrong (the
+ * reference predicts a layer's experts to prefetch their records, model.cpp:438-445, 489-500; here the guess hides the
+ * router, the logits exchange and the selection).  Outputs are the same bytes with or without it.  on = 0 switches the
+ * guessing off (every slot is then computed after the selection); default on. */
+zc_status zc_hip_stack_set_speculation(zc_hip_ctx* ctx, zc_hip_stack* stack, int on);
 zc_status zc_hip_stack_glue(zc_hip_ctx* ctx, const float* y, uint32_t tokens, uint32_t hidden, float* x_next);
 
 /* ---- Expert store: ExpertStore + ExpertCache (include/engine/storage.hpp:168-269; src/engine/storage.cpp:493-725)

@@ -232,3 +232,39 @@ def test_a_wait_that_runs_out_is_reported_and_the_stack_stays_usable(ctx):
             ctx.free(b)
     for T in (1, 2):
         ctx.free(out[T]); ctx.free(xs[T])
+
+
+@pytest.mark.parametrize("skew", [None, ("zipf", 1.1)])
+def test_guessed_experts_never_change_the_result(ctx, skew):
+    # One-token launches start a layer's gate/up tiles on the experts that layer picked at the previous one-token step and redo
+    # only the slots that were guessed wrong.  A run of DIFFERENT tokens (without router skew nearly every guess is wrong, with
+    # the Zipf offsets most are right), with several-token launches in between, must give the bytes of the layer-by-layer
+    # path for every token, and the same with the guessing switched off.
+    cfg = workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512)
+    L = 3
+    layers = [workload.LayerWeights(ctx, cfg, 601 + l, skew) for l in range(L)]
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], 2)
+    out, out2 = ctx.alloc(cfg.hidden * 4), ctx.alloc(2 * cfg.hidden * 4)
+    xs = [workload.hidden_rows(ctx, 1, cfg.hidden, 40 + i) for i in range(6)]
+    x2 = workload.hidden_rows(ctx, 2, cfg.hidden, 77)
+    want, ids = [], []
+    n = cfg.topk
+    trace_ids, trace_w = ctx.alloc(L * n * 4), ctx.alloc(L * n * 4)
+    for x in xs:
+        ctx.stack_decode(stack, x, 1, out, z.StackTrace(trace_ids.ptr, trace_w.ptr, None, None), layered=True); ctx.moe_check()
+        want.append(out.numpy(f32).tobytes()); ids.append(trace_ids.numpy(np.int32).reshape(L, n).copy())
+    repeats = sum(len(set(a[l]) & set(b[l])) for a, b in zip(ids, ids[1:]) for l in range(L)) / (L * n * (len(ids) - 1))
+    print(f"skew {skew}: {repeats:.2f} of a layer's experts repeat from one token to the next")
+    for on in (1, 0, 1):
+        ctx.stack_set_speculation(stack, on)
+        for i in (0, 1, 1, 2, 3, 3, 4, 5, 0):
+            ctx.stack_decode(stack, xs[i], 1, out); ctx.moe_check()
+            assert out.numpy(f32).tobytes() == want[i], f"token {i}, guessing {'on' if on else 'off'}"
+            if i == 2:
+                ctx.stack_decode(stack, x2, 2, out2); ctx.moe_check()
+    ctx.stack_destroy(stack)
+    for l in layers:
+        for b in (l.router, l.shared_gate, l.shared_record, l.records):
+            ctx.free(b)
+    for b in xs + [x2, out, out2, trace_ids, trace_w]:
+        ctx.free(b)

@@ -671,6 +671,8 @@ struct zc_hip_stack {
     float *logits = nullptr, *gate = nullptr, *shared_act = nullptr, *act = nullptr, *layer_out = nullptr, *eout = nullptr;
     uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
     unsigned long long* tlogits = nullptr; uint32_t *tact = nullptr, *tout = nullptr;   // tagged exchange buffers of the one-token kernel
+    uint32_t* tspec = nullptr; int32_t* pred[2] = {nullptr, nullptr};   // prediction pass: its activations, the previous / this step's ids per layer
+    uint32_t pred_turn = 0; bool pred_valid = false, speculate = true;
     uint32_t epoch = 1u << 12;
     uint32_t tag_base = 0;            // tags of the one-token kernel's exchange words: advanced by that kernel's launches only
     uint32_t wait_limit = 1u << 22;   // polls before a wait on another workgroup gives up
@@ -725,7 +727,8 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         const uint64_t o_layers = take(sizeof(zc::DecodeLayer) * n_layers), o_logits = take(uint64_t(Tp) * E * 4), o_gate = take(Tp * 4),
                        o_sact = take(uint64_t(Tp) * I * 4), o_act = take(uint64_t(Tp) * k * I * 4), o_lout = take(uint64_t(Tp) * H * 4),
                        o_max = take(std::max<uint64_t>(uint64_t(n_layers) * Tp * 4, uint64_t(Tp) * (H / 64 + 1) * 4)), o_sync = take(zc::kDecodeSyncBytes), o_eout = take(uint64_t(Tp) * (k + 1) * H * 4),
-                       o_tlogits = take(uint64_t(E + 1) * 8), o_tact = take(uint64_t(k + 1) * I * 4), o_tout = take(uint64_t(2) * H * 4);
+                       o_tlogits = take(uint64_t(E + 1) * 8), o_tact = take(uint64_t(k + 1) * I * 4), o_tout = take(uint64_t(2) * H * 4),
+                       o_tspec = take(uint64_t(k + 1) * I * 4), o_pred0 = take(uint64_t(n_layers) * k * 4), o_pred1 = take(uint64_t(n_layers) * k * 4);
         if (zc_hip_alloc(ctx, at, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
         st->arena = static_cast<uint8_t*>(p); st->arena_bytes = at;
         st->dev_layers = reinterpret_cast<zc::DecodeLayer*>(st->arena + o_layers);
@@ -735,6 +738,8 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         st->sync = reinterpret_cast<uint32_t*>(st->arena + o_sync); st->eout = reinterpret_cast<float*>(st->arena + o_eout);
         st->tlogits = reinterpret_cast<unsigned long long*>(st->arena + o_tlogits); st->tact = reinterpret_cast<uint32_t*>(st->arena + o_tact);
         st->tout = reinterpret_cast<uint32_t*>(st->arena + o_tout);
+        st->tspec = reinterpret_cast<uint32_t*>(st->arena + o_tspec);
+        st->pred[0] = reinterpret_cast<int32_t*>(st->arena + o_pred0); st->pred[1] = reinterpret_cast<int32_t*>(st->arena + o_pred1);
         std::vector<zc::DecodeLayer> host(n_layers);
         for (uint32_t l = 0; l < n_layers; ++l) {
             const zc_moe_layer& y = host_layers[l];
@@ -780,6 +785,11 @@ zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_
     st->wait_limit = polls ? polls : 1u << 22;
     return ZC_OK;
 }
+zc_status zc_hip_stack_set_speculation(zc_hip_ctx* ctx, zc_hip_stack* st, int on) {
+    ZC_REQUIRE(ctx && st, "null argument");
+    st->speculate = on != 0; st->pred_valid = false;
+    return ZC_OK;
+}
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
     if (!ctx || !st) return 0;
     zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt;
@@ -805,7 +815,11 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.layers = st->dev_layers; p.x_in = x; p.out = out;
         p.logits = st->logits; p.gate = st->gate; p.shared_act = st->shared_act; p.act = st->act; p.layer_out = st->layer_out;
         p.maxabs = st->maxabs; p.eout = st->eout;
-        p.tlogits = st->tlogits; p.tact = st->tact; p.tout = st->tout;
+        p.tlogits = st->tlogits; p.tact = st->tact; p.tout = st->tout; p.tspec = st->tspec;
+        if (nt == 1 && st->speculate) {   // this step reads the ids the previous one-token step left, and leaves its own
+            p.pred_in = st->pred_valid ? st->pred[st->pred_turn] : nullptr; p.pred_out = st->pred[st->pred_turn ^ 1u];
+            st->pred_turn ^= 1u; st->pred_valid = true;
+        }
         p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
         if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
         p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;

@@ -81,6 +81,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         auto tag_of = [&](uint32_t l) { return (p.tag_base + l) % 65535u + 1u; };
         const uint32_t tag = tag_of(layer);
         auto st_logit = [&](uint32_t index, float v) { ZC_ST(p.tlogits + index, (uint64_t(tag) << 32) | __float_as_uint(v)); };
+        // one token: the experts this layer picked at the previous step (null: no guess), and where every slot's activations are
+        const int32_t* pred = (NT == 1 && p.pred_in) ? p.pred_in + uint64_t(layer) * k : nullptr;
+        int32_t* spec = reinterpret_cast<int32_t*>(lds + lp.spec);   // [k + 1] source rows, [k + 1] miss list, [1] misses
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
         // One token: the wave's first router unit starts loading its weights while the input row is staged and its image
@@ -440,6 +443,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         for (uint32_t t = wave; t < T; t += kDecodeWaves)
         {
             auto stamp = [&]() { if (t == 0) clock(); };
+            // the previous step's ids of this layer, one per lane: requested now, compared when this step's ids are final
+            const int32_t guess = (NT == 1 && pred && lane < k) ? pred[lane] : -1;
             uint32_t* scratch = reinterpret_cast<uint32_t*>(experts) + 128 * wave;   // the expert list is built later; 128 words per wave fit it for 512 experts
             // the lane's logits: written by other workgroups; one token polls the tagged words until all carry this layer's tag
             auto fetch = [&](auto& cand, uint32_t per) {
@@ -472,6 +477,26 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             // combine needs much later; the routing wave takes its tiles last.
             auto ready = [&]() {
                 if constexpr (NT == 1) {
+                    // Where every slot's gate/up activations come from: the row of the prediction pass that already ran the same
+                    // expert (slot j' of the predicted list), or this layer's own row once the tiles below have run (-1: a miss).
+                    // The misses form the tile list of the second pass; without a prediction every slot and the shared expert miss.
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the ids were written by other lanes of this wave
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    const int32_t mine = lane < k ? ids[lane] : -1;
+                    int32_t from = -1;
+                    if (pred) for (uint32_t j = 0; j < k; ++j) { const int32_t pj = __builtin_amdgcn_readlane(guess, int(j)); if (pj == mine && mine >= 0) from = int32_t(j); }
+                    const uint64_t missing = __ballot(lane < k && from < 0);
+                    if (lane < k) {
+                        spec[lane] = from;
+                        if (from < 0) spec[(k + 1) + __popcll(missing & ((1ull << lane) - 1))] = int32_t(lane);
+                    }
+                    if (lane == 0) {
+                        uint32_t misses = uint32_t(__popcll(missing));
+                        spec[k] = pred ? int32_t(k) : -1;                        // the shared expert's row
+                        if (!pred) spec[(k + 1) + misses++] = int32_t(k);
+                        spec[2 * (k + 1)] = int32_t(misses);
+                    }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                     if (lane == 0) __hip_atomic_store(misc + 11, int32_t(tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
@@ -480,13 +505,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             else route_token<16>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp, ready);
         }
         if constexpr (NT == 1) {
-            // the wave whose only tile is the shared expert's (see the tile list below) needs no ids: it starts at once
-            const bool shared_only = (k * (I / 8)) % nwg == 0 && I / 8 <= nwg && wave == k * (I / 8) / nwg + 1 && nwg - 1 - wg < I / 8;
-            if (wave != 0 && !shared_only) {
-                for (uint32_t i = 0; uint32_t(__hip_atomic_load(misc + 11, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != tag && i < (1u << 22); ++i)
-                    __builtin_amdgcn_s_sleep(1);
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            }
+            // (the waves other than the routing wave go straight to the prediction pass below and wait for the ids after it)
         } else {
             if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
             for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
@@ -498,6 +517,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); if constexpr (NT != 1) next[tid] = -1; }
             else if constexpr (NT != 1) next[tid] = atomicExch(&head[e], int32_t(tid));
             if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * n + tid, e); st_f32(p.weights_trace + uint64_t(layer) * n + tid, weights[tid]); }
+            if (NT == 1 && wg == 0 && p.pred_out) p.pred_out[uint64_t(layer) * k + tid] = e;   // the next step's guess for this layer
         }
         // One token: slot j belongs to expert ids[j] and no two slots share an expert, so there is nothing to group.
         uint32_t U = k;
@@ -524,36 +544,57 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         }
         clock();
         if constexpr (NT == 1) {
-            // the shared expert's gate/up tiles close the list (slot k): with 1280 routed tiles on 256 workgroups they land on
-            // waves that have no routed tile
-            const uint32_t tiles = I / 8, units = (k + 1) * tiles;
-            const uint32_t turn = (wave + kDecodeWaves - 1) % kDecodeWaves;   // the routing wave, still busy with the softmax, comes last
-            // With whole rounds of routed tiles the shared tiles (one more round, not a full one) go to the workgroups counted
-            // from the far end: the near end owns the router units and comes to the tiles last.
-            const bool far_end = (k * tiles) % nwg == 0 && tiles <= nwg;
-            for (uint32_t u = wg + nwg * turn; u < (far_end ? k * tiles + nwg : units); u += nwg * kDecodeWaves) {
-                uint32_t slot = u / tiles, tile = u % tiles;
-                if (far_end && u >= k * tiles) {
-                    const uint32_t s = nwg - 1 - wg;   // the shared tile of this workgroup, if it has one
-                    if (s >= tiles) continue;
-                    slot = k; tile = s;
+            // Two passes over gate/up tiles.  Pass 0 runs BEFORE the ids are known, on the seven waves that do not route: the
+            // tiles of the experts this layer picked at the previous step (the reference predicts a layer's experts for its
+            // prefetcher, model.cpp:438-445; here the guess buys the time of the router, the exchange of the logits and the
+            // selection), and the shared expert's, which needs no ids at all; results go to the prediction buffer.  Pass 1
+            // runs once the ids are final: the tiles of the slots whose expert was not predicted.  Both passes compute a slot
+            // with the same arithmetic, so a guess can only cost time, never change a bit.
+            const uint32_t tiles = I / 8;
+            for (int pass = 0; pass < 2; ++pass) {
+                uint32_t first, stride, units;
+                bool far_end = false;
+                if (pass == 0) {
+                    // With whole rounds of routed tiles the shared tiles (one more round, not a full one) go to the workgroups counted
+                    // from the far end: the near end owns the router units and comes to the tiles last.
+                    if (!pred || wave == 0) continue;
+                    far_end = (k * tiles) % nwg == 0 && tiles <= nwg;
+                    first = wg + nwg * (wave - 1); stride = nwg * (kDecodeWaves - 1); units = far_end ? k * tiles + nwg : (k + 1) * tiles;
+                } else {
+                    if (wave != 0) {
+                        for (uint32_t i = 0; uint32_t(__hip_atomic_load(misc + 11, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != tag && i < (1u << 22); ++i)
+                            __builtin_amdgcn_s_sleep(1);
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    }
+                    const uint32_t turn = (wave + kDecodeWaves - 1) % kDecodeWaves;   // the routing wave, still busy with the softmax, comes last
+                    first = wg + nwg * turn; stride = nwg * kDecodeWaves; units = uint32_t(uniform(spec[2 * (k + 1)])) * tiles;
                 }
-                const int32_t e = slot < k ? uniform(ids[slot]) : 0;
-                if (e < 0 || e >= int32_t(E)) continue;   // reported above; the combine drops the slot
-                const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                const uint8_t* rec = slot < k ? L.records + uint64_t(e) * L.stride : L.shared_record;
-                const uint64_t* off = slot < k ? p.ro : p.so;
-                const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
-                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
-                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 2]) + uint64_t(row) * (H / 64);
-                const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
-                // SwiGLU of the finished tile as tagged words, one per activation: row `slot` of the tagged buffer (row k: shared)
-                auto emit = [&](int, float v) {
-                    const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
-                    const uint32_t a = __float_as_uint(swiglu_bf(v, up));
-                    if (lane < 8) ZC_ST(p.tact + uint64_t(slot) * I + row, (a & 0xffff0000u) | tag);
-                };
-                ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
+                for (uint32_t u = first; u < units; u += stride) {
+                    uint32_t slot = u / tiles, tile = u % tiles;
+                    if (far_end && u >= k * tiles) {
+                        const uint32_t s = nwg - 1 - wg;   // the shared tile of this workgroup, if it has one
+                        if (s >= tiles) continue;
+                        slot = k; tile = s;
+                    }
+                    if (pass == 1) slot = uint32_t(uniform(spec[(k + 1) + slot]));   // the miss list
+                    const int32_t e = slot < k ? (pass == 0 ? uniform(pred[slot]) : uniform(ids[slot])) : 0;
+                    if (e < 0 || e >= int32_t(E)) continue;   // no guess for the slot, or an id reported above (the combine drops the slot)
+                    const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                    const uint8_t* rec = slot < k ? L.records + uint64_t(e) * L.stride : L.shared_record;
+                    const uint64_t* off = slot < k ? p.ro : p.so;
+                    const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
+                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
+                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 2]) + uint64_t(row) * (H / 64);
+                    const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
+                    uint32_t* out_row = (pass == 0 ? p.tspec : p.tact) + uint64_t(slot) * I;
+                    // SwiGLU of the finished tile as tagged words, one per activation: row `slot` of the tagged buffer (row k: shared)
+                    auto emit = [&](int, float v) {
+                        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+                        const uint32_t a = __float_as_uint(swiglu_bf(v, up));
+                        if (lane < 8) ZC_ST(out_row + row, (a & 0xffff0000u) | tag);
+                    };
+                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
+                }
             }
             if (tid == 64) {   // the combine's gate factor (written by another workgroup)
                 uint64_t w = 0;
@@ -628,7 +669,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         if (lane < 4) reinterpret_cast<uint32_t*>(image + LI.blocks() * 48)[lane] = 0;
                         wave_sync();
                         for (uint32_t b = lane; b < I / 16; b += 64) {
-                            const uint64_t* words = reinterpret_cast<const uint64_t*>(p.tact + uint64_t(slot) * I + b * 16);
+                            const int32_t from = uniform(spec[slot]);   // the prediction pass's row of the same expert, or this layer's own
+                            const uint64_t* words = reinterpret_cast<const uint64_t*>((from >= 0 ? p.tspec + uint64_t(from) * I : p.tact + uint64_t(slot) * I) + b * 16);
                             uint64_t w[8];
                             bar.until([&]() {
                                 uint32_t bad = 0;
@@ -684,7 +726,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                             for (int j = 0; j < kMine; ++j) {
                                 const uint32_t blk = base + j * kDecodeThreads + tid;
                                 if (wanted[j]) {
-                                    const uint64_t* src = reinterpret_cast<const uint64_t*>(p.tact + uint64_t(s0 + blk / per) * I + (blk % per) * 16);
+                                    const uint32_t at_slot = s0 + blk / per;
+                                    const int32_t from = spec[at_slot];
+                                    const uint64_t* src = reinterpret_cast<const uint64_t*>((from >= 0 ? p.tspec + uint64_t(from) * I : p.tact + uint64_t(at_slot) * I) + (blk % per) * 16);
 #pragma unroll
                                     for (int w = 0; w < 8; ++w) words[j][w] = ZC_LD(src + w);
                                 }
@@ -841,6 +885,7 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
     auto take = [&](uint32_t bytes) { const uint32_t o = at; at += align16(bytes); return o; };
     lp.ids = take(NT * topk * 4); lp.weights = take(NT * topk * 4); lp.gatev = take(NT * 4);
     lp.head = take(E * 4); lp.next = take(NT * topk * 4); lp.experts = take(E * 4); lp.misc = take(64); lp.gatew = take(H * 2);
+    lp.spec = take((2 * (topk + 1) + 1) * 4);
     lp.region = at;
     lp.img_rg = lp.region; lp.xh = lp.img_rg + NT * LH.bytes();
     lp.gprod = lp.xh + align16(NT * H * 2);   // one token: the shared gate dot's products, [32][hidden / 32 + 1] fp32

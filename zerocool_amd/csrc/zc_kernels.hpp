@@ -71,6 +71,10 @@ struct DecodeParams {
     // waiting at a grid barrier and fetching afterwards.  tlogits [E + 1] words {fp32 bits, tag << 32} (word E: the shared
     // gate dot); tact [topk + 1][I] and tout [2][H] words {BF16 value << 16 | 16-bit tag}.  All zero before the first launch.
     unsigned long long* tlogits; uint32_t *tact, *tout;
+    // One token, optional: pred_in [L][topk] = the ids every layer picked at the previous step (its gate/up tiles start on them
+    // before this step's ids are known), pred_out [L][topk] receives this step's; tspec [topk + 1][I]: the prediction pass's
+    // activations, tagged like tact.
+    const int32_t* pred_in; int32_t* pred_out; uint32_t* tspec;
     int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][T][topk], [L][T][topk], [L][T][H]
     uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
     uint32_t tag_base;               // one token: layer l exchanges under tag (tag_base + l) % 65535 + 1; advances only with one-token launches
@@ -79,7 +83,7 @@ struct DecodeParams {
 constexpr uint32_t kDecodeStamps = 15;
 struct DecodeLdsPlan {
     uint32_t ids, weights, gatev, head, next, experts, misc, region, total;
-    uint32_t img_rg, xh, gprod, img_d, ah, otile, slots_per_batch, gatew;
+    uint32_t img_rg, xh, gprod, img_d, ah, otile, slots_per_batch, gatew, spec;
 };
 DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t NT, uint32_t lds_limit);
 hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp);

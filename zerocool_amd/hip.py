@@ -381,6 +381,9 @@ class Context:
         self._call("zc_hip_stack_decode", stack, _ptr(x), C.c_uint32(tokens), _ptr(out),
                    C.byref(trace) if trace is not None else None, C.c_uint32(1 if layered else 0))
 
+    def stack_set_speculation(self, stack, on):
+        self._call("zc_hip_stack_set_speculation", stack, C.c_int(int(on)))
+
     def stack_set_wait_limit(self, stack, polls):
         self._call("zc_hip_stack_set_wait_limit", stack, C.c_uint32(polls))
 

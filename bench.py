@@ -21,9 +21,11 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-# HBM bytes per launch of the default workload (48 layers, batch 1) from the FETCH_SIZE / WRITE_SIZE counter runs summarised
-# in profiles/decode_stack_kernel_F48_batch1_pmc.txt (counters cannot be read from inside this process).
-MEASURED_TRAFFIC = 3_023_324_000
+# HBM bytes per launch of the default workload (48 layers, batch 1): counters cannot be read from inside this process, so
+# the figure comes from two rocprofv3 --pmc runs of this program (FETCH_SIZE, then WRITE_SIZE, each with --calibrate) whose
+# CSV output `bench.py --traffic-from <fetch dir> <write dir>` turns into this tracked file.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_stack_kernel_F48_batch1_traffic.json")
+INPUTS = 8   # distinct token batches the timed steps cycle through
 sys.path.insert(0, ROOT)
 
 
@@ -52,6 +54,69 @@ def single_layer(ctx, name, tokens, prefill, reps, warmup=3):
             "TFLOPs": flops / (ms_layer * 1e-3) / 1e12, "path": "bf16 matrix-core prefill" if prefill else "exact operator path"}
 
 
+def write_traffic_file(fetch_dir, write_dir):
+    """Turns the CSV output of the two counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE --output-format csv, each over
+    `bench.py --no-cpu --calibrate`) into the tracked traffic file: per-dispatch averages of the decode kernel in KiB, each
+    scaled by what the same counter reads for the 1 GiB device-to-device copy of --calibrate (1,048,576 KiB each way)."""
+    import collections, csv, glob
+    def averages(folder, counter):
+        values = collections.defaultdict(list)
+        for path in glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True):
+            for row in csv.DictReader(open(path)):
+                if row["Counter_Name"] == counter:
+                    values[row["Kernel_Name"]].append(float(row["Counter_Value"]))
+        pick = lambda word: [v for k, v in values.items() if word in k]
+        copies, = pick("copyBuffer")          # the runtime's copy kernel also serves small copies: the 1 GiB one is the largest
+        kernel, = pick("decode_stack_kernel")
+        return sum(kernel) / len(kernel), max(copies), len(kernel)
+    fetch, fetch_copy, calls = averages(fetch_dir, "FETCH_SIZE")
+    write, write_copy, _ = averages(write_dir, "WRITE_SIZE")
+    read_bytes = fetch * (1048576.0 / fetch_copy) * 1024
+    written_bytes = write * (1048576.0 / write_copy) * 1024
+    record = {"kernel": "zc::decode_stack_kernel<1>", "workload": "48 F-shape layers, batch 1 (the default run of bench.py)",
+              "dispatches_averaged": calls, "FETCH_SIZE_KiB": fetch, "FETCH_SIZE_KiB_of_1GiB_copy": fetch_copy,
+              "WRITE_SIZE_KiB": write, "WRITE_SIZE_KiB_of_1GiB_copy": write_copy,
+              "hbm_bytes_read": int(read_bytes), "hbm_bytes_written": int(written_bytes),
+              "hbm_bytes_per_launch": int(read_bytes + written_bytes)}
+    json.dump(record, open(TRAFFIC_FILE, "w"), indent=1)
+    print(json.dumps(record))
+
+
+def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), speculate=True):
+    """The same single-layer configuration through the persistent decode kernel as a stack of one layer: one launch per
+    step, over 8 distinct inputs in rotation."""
+    import numpy as np
+    from zerocool_amd import workload
+    c = workload.config(name)
+    lw = workload.LayerWeights(ctx, c, workload.BASE_SEED + 77, skew)
+    stack = ctx.stack_create(c, [lw.layer], 8)
+    ctx.stack_set_speculation(stack, speculate)
+    xs = [workload.hidden_rows(ctx, tokens, c.hidden, workload.BASE_SEED + 78 + tokens + 97 * i) for i in range(INPUTS)]
+    out = ctx.alloc(tokens * c.hidden * 4)
+    ws = ctx.alloc(ctx.moe_workspace_bytes(c, tokens))
+    ref = ctx.alloc(tokens * c.hidden * 4)
+    for x in xs:   # parity gate: the operator path's bytes (glue of layer 0 is the identity on the input)
+        ctx.stack_decode(stack, x, tokens, out)
+        ctx.moe_forward(c, lw.layer, x, tokens, ref, ws)
+        ctx.moe_check()
+        if out.numpy(np.float32).tobytes() != ref.numpy(np.float32).tobytes():
+            raise SystemExit("bench.py: one-launch layer and operator path disagree; refusing to time")
+    for i in range(warmup):
+        ctx.stack_decode(stack, xs[i % INPUTS], tokens, out)
+    ctx.finish()
+    ctx.timer_start()
+    for i in range(reps):
+        ctx.stack_decode(stack, xs[i % INPUTS], tokens, out)
+    ms = ctx.timer_stop() / reps
+    ctx.moe_check()
+    persistent = ctx.stack_is_persistent(stack, tokens)
+    ctx.stack_destroy(stack)
+    for b in xs + [out, ws, ref, lw.router, lw.shared_gate, lw.shared_record, lw.records]:
+        ctx.free(b)
+    return {"tokens": tokens, "us_per_layer": ms * 1e3, "tokens_per_s": tokens / (ms * 1e-3), "router_skew": list(skew) if skew else None,
+            "guessing": bool(speculate), "path": "persistent single-launch kernel" if persistent else "layer by layer"}
+
+
 def prefill_workload(ctx, args):
     r = single_layer(ctx, "S", 2048, True, args.steps, args.warmup)
     print(json.dumps({
@@ -78,7 +143,11 @@ def main():
                     help="stack: the 48-layer decode stack (the headline); prefill: one 2048-token batch through one layer of "
                          "hidden 2048 / 512 experts / top-10 / intermediate 512 on the bf16 matrix cores")
     ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no GPU work: rewrite the tracked traffic file from the output folders of the two counter runs")
     args = ap.parse_args()
+    if args.traffic_from:
+        return write_traffic_file(*args.traffic_from)
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
               "(the design notes describe how the path would shard by expert)", file=sys.stderr)
@@ -86,7 +155,7 @@ def main():
 
     import numpy as np
     import zerocool_amd as z
-    from zerocool_amd import workload
+    from zerocool_amd import synth, workload
 
     ctx = z.Context(0)
     if args.workload == "prefill":
@@ -97,32 +166,44 @@ def main():
     ctx.finish()
     stack = ctx.stack_create(cfg, [l.layer for l in layers], max(T, 8))
 
-    def run(tokens, steps, warmup):
-        x = workload.hidden_rows(ctx, tokens, cfg.hidden, workload.BASE_SEED + 4 * 7 + tokens)
+    def run(stack, cfg, n_layers, tokens, steps, warmup, speculate=True, inputs=INPUTS, seed=workload.BASE_SEED + 4 * 7):
+        """Times `steps` launches that cycle through `inputs` distinct token batches (a decode loop never sees the same
+        hidden rows twice; the one-token kernel guesses each layer's experts from the step before, so a replayed input
+        would make every guess a hit).  Every input is first checked against the layer-by-layer operator path, byte for
+        byte, and its route ids are kept: they give the distinct records (the algorithmic bytes) of each launch and the
+        share of a step's experts that the step before had also chosen (what the guessing can hit)."""
+        xs = [workload.hidden_rows(ctx, tokens, cfg.hidden, seed + tokens + 97 * i) for i in range(inputs)]
         out = ctx.alloc(tokens * cfg.hidden * 4)
         n = tokens * cfg.topk
-        ids, w = ctx.alloc(L * n * 4), ctx.alloc(L * n * 4)
-        ctx.stack_decode(stack, x, tokens, out, z.StackTrace(ids.ptr, w.ptr, None, None))
-        ctx.moe_check()
-        # parity gate before any timing: the single-launch kernel and the layer-by-layer operator path must agree byte for byte
-        fused = out.numpy(np.float32).tobytes()
-        ctx.stack_decode(stack, x, tokens, out, layered=True)
-        ctx.moe_check()
-        if out.numpy(np.float32).tobytes() != fused:
-            raise SystemExit("bench.py: persistent kernel and layer-by-layer path disagree; refusing to time")
-        unique = [len(np.unique(r)) for r in ids.numpy(np.int32).reshape(L, n)]
-        nbytes = sum(workload.layer_bytes(cfg, u, tokens, ctx) for u in unique)
-        for _ in range(warmup):
-            ctx.stack_decode(stack, x, tokens, out)
+        ids, w = ctx.alloc(n_layers * n * 4), ctx.alloc(n_layers * n * 4)
+        ctx.stack_set_speculation(stack, speculate)
+        chosen, nbytes, unique = [], [], []
+        for x in xs:
+            ctx.stack_decode(stack, x, tokens, out, z.StackTrace(ids.ptr, w.ptr, None, None))
+            ctx.moe_check()
+            fused = out.numpy(np.float32).tobytes()
+            ctx.stack_decode(stack, x, tokens, out, layered=True)
+            ctx.moe_check()
+            if out.numpy(np.float32).tobytes() != fused:
+                raise SystemExit("bench.py: persistent kernel and layer-by-layer path disagree; refusing to time")
+            rows = ids.numpy(np.int32).reshape(n_layers, n).copy()
+            chosen.append(rows)
+            u = [len(np.unique(r)) for r in rows]
+            unique.append(float(np.mean(u)))
+            nbytes.append(sum(workload.layer_bytes(cfg, v, tokens, ctx) for v in u))
+        repeats = [np.mean([len(np.intersect1d(a[l], b[l])) / len(np.unique(a[l])) for l in range(n_layers)])
+                   for a, b in zip(chosen[1:] + chosen[:1], chosen)] if inputs > 1 else [1.0]
+        for i in range(warmup):
+            ctx.stack_decode(stack, xs[i % inputs], tokens, out)
         ctx.finish()
         ctx.timer_start()
-        for _ in range(steps):
-            ctx.stack_decode(stack, x, tokens, out)
+        for i in range(steps):
+            ctx.stack_decode(stack, xs[(warmup + i) % inputs], tokens, out)
         ms = ctx.timer_stop() / steps
         ctx.moe_check()
-        for b in (x, out, ids, w):
+        for b in xs + [out, ids, w]:
             ctx.free(b)
-        return ms, nbytes, unique
+        return {"ms": ms, "bytes": float(np.mean(nbytes)), "unique": float(np.mean(unique)), "repeat_share": float(np.mean(repeats))}
 
     if args.calibrate:
         gib = 1 << 30
@@ -131,9 +212,13 @@ def main():
         ctx.copy(b, a, gib)
         ctx.finish()
         ctx.free(a); ctx.free(b)
-    ms, nbytes, unique = run(T, args.steps, args.warmup)
+    r = run(stack, cfg, L, T, args.steps, args.warmup)
+    ms, nbytes = r["ms"], r["bytes"]
     persistent = ctx.stack_is_persistent(stack, T)
     achieved = nbytes / (ms * 1e-3) / 1e9
+    traffic = None
+    if (L, T) == (48, 1) and os.path.exists(TRAFFIC_FILE):
+        traffic = json.load(open(TRAFFIC_FILE))["hbm_bytes_per_launch"]
     result = {
         "metric": "moe_decode_tokens_per_s", "value": T / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
@@ -143,11 +228,13 @@ def main():
                                "intermediate 1024, affine Q4 group 64, ~130 GB of expert records resident in HBM, "
                                "Zipf(1.1) router offsets, one seed per layer",
                    "layers": L, "decode_batch": T, "hbm_resident_bytes": int(ctx.allocated),
-                   "distinct_experts_per_layer": float(np.mean(unique)),
+                   "inputs": f"{INPUTS} distinct token batches in rotation", "distinct_experts_per_layer": r["unique"],
+                   "experts_repeated_from_previous_step": r["repeat_share"],
                    "path": "persistent single-launch kernel" if persistent else "layer by layer",
                    "parity_gate": "output bytes equal the layer-by-layer operator path on this input (checked before timing)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s", "frac": achieved / 8000.0,
-                     "traffic": MEASURED_TRAFFIC if (L, T) == (48, 1) else None, "kernel": "zc::decode_stack_kernel (one launch = one step)",
+                     "traffic": traffic, "traffic_source": os.path.relpath(TRAFFIC_FILE, ROOT) if traffic else None,
+                     "kernel": "zc::decode_stack_kernel (one launch = one step)" if T == 1 else "zc::decode_multi_kernel (one launch = one step)",
                      "algorithmic_bytes_per_launch": int(nbytes), "launch_us": ms * 1e3},
     }
 
@@ -174,9 +261,32 @@ def main():
                                   "ms_per_layer": per_layer * 1e3}
     if args.extra:
         extra = {}
-        ms8, b8, u8 = run(8, max(5, args.steps // 4), 2)
-        extra["stack_batch8"] = {"tokens_per_s": 8 / (ms8 * 1e-3), "ms_per_step": ms8, "GBps": b8 / (ms8 * 1e-3) / 1e9,
-                                 "distinct_experts_per_layer": float(np.mean(u8))}
+        quick = max(8, args.steps // 2)
+        if T == 1:
+            off = run(stack, cfg, L, 1, quick, 2, speculate=False)
+            extra["stack_batch1_without_guessing"] = {"tokens_per_s": 1 / (off["ms"] * 1e-3), "ms_per_step": off["ms"],
+                                                      "GBps": off["bytes"] / (off["ms"] * 1e-3) / 1e9}
+        r8 = run(stack, cfg, L, 8, quick, 2)
+        extra["stack_batch8"] = {"tokens_per_s": 8 / (r8["ms"] * 1e-3), "ms_per_step": r8["ms"], "GBps": r8["bytes"] / (r8["ms"] * 1e-3) / 1e9,
+                                 "frac_of_hbm_peak": r8["bytes"] / (r8["ms"] * 1e-3) / 8e12, "distinct_experts_per_layer": r8["unique"],
+                                 "kernel": "zc::decode_multi_kernel"}
+        # The same records behind routers with a milder popularity skew (Zipf exponent 0.5: the offsets span 3.1 instead
+        # of 6.9) and with none at all, so that consecutive tokens share fewer experts and a batch of eight touches
+        # several times more records.
+        for name, exponent in (("mild_skew_zipf_0.5", 0.5), ("no_skew", None)):
+            offsets = [ctx.upload(synth.zipf_offsets(cfg.experts, (workload.BASE_SEED + 4 * 1000 + l) * 16 + 5, exponent))
+                       for l in range(L)] if exponent else [None] * L
+            other = ctx.stack_create(cfg, [z.Layer(w.router.ptr, o.ptr if o else None, w.shared_gate.ptr, w.shared_record.ptr,
+                                                   w.records.ptr, w.stride) for w, o in zip(layers, offsets)], 8)
+            extra[name] = {}
+            for tokens, spec in ((1, True), (1, False), (8, True)):
+                m = run(other, cfg, L, tokens, quick, 2, speculate=spec)
+                extra[name][f"batch{tokens}" + ("" if spec else "_without_guessing")] = {
+                    "tokens_per_s": tokens / (m["ms"] * 1e-3), "ms_per_step": m["ms"], "GBps": m["bytes"] / (m["ms"] * 1e-3) / 1e9,
+                    "distinct_experts_per_layer": m["unique"], "experts_repeated_from_previous_step": m["repeat_share"]}
+            ctx.stack_destroy(other)
+            for o in offsets:
+                if o: ctx.free(o)
         # The capped-HBM run of the same configuration: the records' home is pinned host memory, 2000 of the 24576
         # records fit in HBM slots (the same fraction here, on fewer layers so that the pinned home stays modest), the
         # rest arrive by hipMemcpyAsync on the store's side stream.  The step is the reference's orchestration with one
@@ -215,6 +325,10 @@ def main():
         capped.close()
         # Single-layer configurations: decode batches through the exact operator path, and batches through the
         # sorted-token grouped product on the bf16 matrix cores.
+        extra["single_layer_q4_one_launch"] = [one_launch_layer(ctx, "S", t, 200) for t in (1, 8)]
+        # raw random inputs behind an unskewed router share next to no experts from one step to the next: every guess of
+        # the one-token kernel misses, which prices the guessing at its worst
+        extra["single_layer_q4_one_launch_all_guesses_miss"] = [one_launch_layer(ctx, "S", 1, 200, skew=None, speculate=on) for on in (True, False)]
         extra["single_layer_q4"] = [single_layer(ctx, "S", t, False, 50) for t in (1, 8, 32, 64)]
         extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8)]
         extra["prefill_q4"] = [single_layer(ctx, "S", t, True, 20) for t in (32, 64, 256, 2048)]

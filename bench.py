@@ -142,6 +142,7 @@ def main():
     ap.add_argument("--workload", choices=("stack", "prefill"), default="stack",
                     help="stack: the 48-layer decode stack (the headline); prefill: one 2048-token batch through one layer of "
                          "hidden 2048 / 512 experts / top-10 / intermediate 512 on the bf16 matrix cores")
+    ap.add_argument("--capped-layers", type=int, default=12, help="--extra: layers of the capped-HBM run (48 pins 130 GB of host memory)")
     ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: rewrite the tracked traffic file from the output folders of the two counter runs")
@@ -287,41 +288,49 @@ def main():
             ctx.stack_destroy(other)
             for o in offsets:
                 if o: ctx.free(o)
-        # The capped-HBM run of the same configuration: the records' home is pinned host memory, 2000 of the 24576
-        # records fit in HBM slots (the same fraction here, on fewer layers so that the pinned home stays modest), the
-        # rest arrive by hipMemcpyAsync on the store's side stream.  The step is the reference's orchestration with one
-        # readback of the ids per layer, driven from Python: the figure shows the store at work, not a tuned decode loop.
+        # The capped-HBM run of the same configuration: the records' home is pinned host memory and 2000 of the 24576
+        # records fit in HBM slots (the same fraction on --capped-layers layers, so that the pinned home stays modest by
+        # default).  Each step is one launch of the same persistent kernels, which take every record's address from the
+        # store's table: an HBM slot, or the record's home over the host link; after the launch the store admits what was
+        # read from home (fills on its side stream).  Timed by the host clock: the step includes the wait for the launch,
+        # the readback of the routes and the store's bookkeeping.
         ctx.stack_destroy(stack)
         for l in layers:
             for b in (l.router, l.shared_gate, l.shared_record, l.records):
                 ctx.free(b)
-        capped_layers = 6
-        slots = max(cfg.topk + 2, 2000 * capped_layers // 48)
-        capped = workload.StoreBackedStack(ctx, cfg, [workload.BASE_SEED + 4 * 1000 + l for l in range(capped_layers)], ("zipf", 1.1), slots)
-        def capped_step(seed):
-            x = workload.hidden_rows(ctx, 1, cfg.hidden, seed)
-            for l in range(capped_layers):
-                y, _ = capped.layer_forward(l, x, 1)
-                ctx.free(x)
-                x = ctx.alloc(cfg.hidden * 4)
-                ctx.stack_glue(y, 1, cfg.hidden, x)
-                ctx.free(y)
-            ctx.finish(); ctx.free(x)
-        for i in range(3):
-            capped_step(900 + i)
-        before = capped.store.stats()
-        hits0, misses0, bytes0 = before.hits, before.misses, before.bytes
-        t0 = time.perf_counter(); n_steps = 20
-        for i in range(n_steps):
-            capped_step(1000 + i)
-        dt = time.perf_counter() - t0
-        st = capped.store.stats()
-        extra["capped_hbm"] = {"layers": capped_layers, "hbm_slots": int(slots), "records": capped_layers * cfg.experts,
-                               "ms_per_layer": dt / n_steps / capped_layers * 1e3,
-                               "tokens_per_s_scaled_to_48_layers": n_steps / dt * capped_layers / 48,
-                               "hit_rate": (st.hits - hits0) / max(1, st.hits - hits0 + st.misses - misses0),
-                               "host_to_hbm_bytes_per_token_layer": (st.bytes - bytes0) / n_steps / capped_layers,
-                               "evictions": int(st.evictions), "note": "Python-driven reference orchestration over zc_hip_store_*"}
+        CL = args.capped_layers
+        slots = max(cfg.topk + 2, 2000 * CL // 48)
+        capped = workload.StoreBackedStack(ctx, cfg, [workload.BASE_SEED + 4 * 1000 + l for l in range(CL)], ("zipf", 1.1), slots)
+        cstack = capped.decode_stack(8)
+        extra["capped_hbm"] = {"layers": CL, "hbm_slots": int(slots), "records": CL * cfg.experts,
+                               "pinned_home_bytes": CL * cfg.experts * int(capped.store.stride)}
+        for tokens in (1, 8):
+            xs = [workload.hidden_rows(ctx, tokens, cfg.hidden, workload.BASE_SEED + 4 * 7 + tokens + 97 * i) for i in range(INPUTS)]
+            out = ctx.alloc(tokens * cfg.hidden * 4)
+            t0 = time.perf_counter()
+            ctx.stack_decode(cstack, xs[0], tokens, out)      # cold: every record comes over the host link
+            cold = time.perf_counter() - t0
+            for i in range(2 * INPUTS):
+                ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
+            ctx.finish(); ctx.moe_check()
+            seen0, st0 = capped.store.table_stats(), capped.store.stats()
+            reads0, slot0, home0, fill0 = seen0.reads, seen0.slot_reads, seen0.home_read_bytes, st0.bytes
+            n_steps = max(16, args.steps)
+            t0 = time.perf_counter()
+            for i in range(n_steps):
+                ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
+            dt = (time.perf_counter() - t0) / n_steps
+            ctx.moe_check()
+            seen, st = capped.store.table_stats(), capped.store.stats()
+            extra["capped_hbm"][f"batch{tokens}"] = {
+                "ms_per_step": dt * 1e3, "us_per_layer": dt / CL * 1e6, "tokens_per_s_at_48_layers": tokens / (dt / CL * 48),
+                "first_step_ms": cold * 1e3, "slot_hit_rate": (seen.slot_reads - slot0) / max(1, seen.reads - reads0),
+                "bytes_read_from_home_per_token": (seen.home_read_bytes - home0) / n_steps / tokens * 48 / CL,
+                "bytes_filled_into_slots_per_token": (st.bytes - fill0) / n_steps / tokens * 48 / CL}
+            for b in xs + [out]:
+                ctx.free(b)
+        extra["capped_hbm"]["evictions"] = int(capped.store.stats().evictions)
+        ctx.stack_destroy(cstack)
         capped.close()
         # Single-layer configurations: decode batches through the exact operator path, and batches through the
         # sorted-token grouped product on the bf16 matrix cores.

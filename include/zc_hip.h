@@ -269,6 +269,42 @@ zc_status zc_hip_store_clear(zc_hip_store* store);                    /* ZC_LOGI
 zc_status zc_hip_store_resize(zc_hip_store* store, uint64_t slots);   /* survivors keep their bytes; ZC_LOGIC_ERROR while a lease is out */
 zc_status zc_hip_store_stats(const zc_hip_store* store, zc_store_stats* out);
 zc_status zc_hip_store_layer_stats(const zc_hip_store* store, uint32_t layer, uint64_t* hits, uint64_t* misses);
+/* The store as a kernel sees it: a table of layers * experts record addresses, entry [layer * experts + expert].  An entry
+ * points at the record's HBM slot while that slot holds the finished record and at the record's home otherwise (pinned
+ * host memory, which the GPU reads over the host link), so a kernel that takes its records from the table always finds
+ * the right bytes and never waits for the host: the reference's acquire -> wait -> encode -> release around every expert
+ * (pipeline.cpp:158-214, storage.cpp:628-676) becomes one table lookup on the device and the two host calls below around
+ * a whole launch.  Create the table while the store is empty.
+ *   zc_hip_store_table_refresh  before a launch: entries of fills that have finished switch to their slots; the changed
+ *                               table is copied to the device on the context's stream.
+ *   zc_hip_store_table_observe  after the launch has FINISHED (the host has synchronised): the expert ids one layer chose.
+ *                               Records read from a slot are touched (ExpertCache::acquire's hit), records read from home
+ *                               are admitted (its miss: a victim by CLOCK, the fill starts on the side stream and serves
+ *                               later launches); no lease stays out.  A fill never starts while a launch that may read
+ *                               its slot is in flight, because fills start here only.
+ * Leases and the table may not be mixed on one store while launches are in flight. */
+typedef struct {
+    uint64_t reads;            /* distinct (layer, expert) records that observed launches read */
+    uint64_t slot_reads;       /* ... from an HBM slot */
+    uint64_t home_reads;       /* ... from the record's home over the host link */
+    uint64_t home_read_bytes;
+    uint64_t switched;         /* finished fills whose table entry moved to the slot */
+    uint64_t not_admitted;     /* misses that found every slot still loading */
+} zc_store_table_stats;
+zc_status zc_hip_store_table(zc_hip_store* store, const void* const** table);
+zc_status zc_hip_store_table_refresh(zc_hip_store* store);
+zc_status zc_hip_store_table_observe(zc_hip_store* store, uint32_t layer, const int32_t* ids, uint32_t count);
+zc_status zc_hip_store_table_stats(const zc_hip_store* store, zc_store_table_stats* out);
+zc_status zc_hip_store_geometry(const zc_hip_store* store, uint32_t* layers, uint32_t* experts, uint64_t* record_bytes);
+/* A decode stack whose routed records live in an expert store (the capped-HBM run: model.cpp:431-557 with the cache of
+ * storage.cpp:525-725 in the loop).  host_layers[l].expert_records is ignored; the store must have n_layers layers of
+ * cfg's records, and max_tokens <= 8.  zc_hip_stack_decode on such a stack is ONE launch that reads every record
+ * through the store's table (zc_hip_store_table), then waits for the launch on the host, copies the routes back and
+ * hands them to zc_hip_store_table_observe, so that the records this step read from their homes are in HBM slots for
+ * the steps to come.  Output bytes are those of a stack with all records resident.  flags bit 0 (layer by layer) is
+ * refused with ZC_INVALID_ARGUMENT. */
+zc_status zc_hip_stack_create_with_store(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
+                                         uint32_t n_layers, uint32_t max_tokens, zc_hip_store* store, zc_hip_stack** out);
 /* Stores without a context only: fills of this record stay "loading" while held (what a slow read is to the reference's tests). */
 zc_status zc_hip_store_hold(zc_hip_store* store, uint32_t layer, uint32_t expert, int hold);
 

@@ -66,14 +66,65 @@ int main() {
     }
     MoeShape other = s; other.inter = 256;
     CHECK_THROWS(PreparedExperts(dir, other));                            // "unsupported prepared expert projection"
+    // Geometry refusals: the manifest is changed and the verification pass run again, so that only the named defect is left.
     const std::string manifest = slurp(dir / "manifest.json");
-    spit(dir / "manifest.json", replaced(manifest, "zc-affine-records-v1", "zc-affine-records-v2")); CHECK_THROWS(PreparedExperts(dir, s));
-    spit(dir / "manifest.json", replaced(manifest, "\"alignment\": 16384", "\"alignment\": 4096")); CHECK_THROWS(PreparedExperts(dir, s));
-    spit(dir / "manifest.json", replaced(manifest, "experts-01.bin", "experts-00.bin")); CHECK_THROWS(PreparedExperts(dir, s));   // duplicate range
-    spit(dir / "manifest.json", replaced(manifest, "experts-01.bin", "../experts-01.bin")); CHECK_THROWS(PreparedExperts(dir, s));
-    spit(dir / "manifest.json", replaced(manifest, "\"group_size\": 64", "\"group_size\": 32")); CHECK_THROWS(PreparedExperts(dir, s));
+    const auto refused_after_verification = [&](const std::string& from, const std::string& to) {
+        spit(dir / "manifest.json", replaced(manifest, from, to));
+        try { verify_prepared_experts(dir); } catch (const std::exception&) { return true; }   // the pass itself may already refuse
+        try { PreparedExperts p(dir, s); } catch (const std::exception&) { return true; }
+        return false;
+    };
+    CHECK(refused_after_verification("zc-affine-records-v1", "zc-affine-records-v2"));
+    CHECK(refused_after_verification("\"alignment\": 16384", "\"alignment\": 4096"));
+    CHECK(refused_after_verification("\"file\": \"experts-01.bin\"", "\"file\": \"experts-00.bin\""));   // duplicate range
+    CHECK(refused_after_verification("\"file\": \"experts-01.bin\"", "\"file\": \"../experts-01.bin\""));
+    CHECK(refused_after_verification("\"group_size\": 64", "\"group_size\": 32"));
+    spit(dir / "manifest.json", manifest); verify_prepared_experts(dir);
+    { PreparedExperts again(dir, s); CHECK(again.layers() == 2); }
+
+    std::printf("prepared directory: identity (manifest digest, verification receipt, file digests)\n");
+    CHECK(sha256_hex("") == "e3b0c44298fc1c149afbf4c8996fb92427ae41e4649b934ca495991b7852b855");          // FIPS 180-4 examples
+    CHECK(sha256_hex("abc") == "ba7816bf8f01cfea414140de5dae2223b00361a396177a9cb410ff61f20015ad");
+    CHECK(sha256_hex("abcdbcdecdefdefgefghfghighijhijkijkljklmklmnlmnomnopnopq") == "248d6a61d20638b8e5c026930c3e6039a33ce45964ff2167f6ecedd419db06c1");
+    { Sha256 h; const std::string a(1000, 'a'); for (int i = 0; i < 1000; ++i) h.update(std::as_bytes(std::span<const char>(a.data(), a.size())));
+      CHECK(h.hex() == "cdc76e5c9914fb9281a1c7e284d73e67f1809a48a497200e046d39ccc7112cd0"); }              // one million 'a'
+    {
+        PreparedExperts p(dir, s);
+        CHECK(p.identity() == sha256_hex(manifest) && p.identity().size() == 64);
+        PreparedIdentity pinned; pinned.pinned_manifest_sha256 = p.identity();
+        { PreparedExperts q(dir, s, pinned); CHECK(q.layers() == 2); }
+        pinned.pinned_manifest_sha256[0] = pinned.pinned_manifest_sha256[0] == '0' ? '1' : '0';
+        CHECK_THROWS(PreparedExperts(dir, s, pinned));                    // "prepared manifest differs from the pinned one"
+        PreparedIdentity elsewhere; elsewhere.source_revision = "another-checkpoint";
+        CHECK_THROWS(PreparedExperts(dir, s, elsewhere));
+        PreparedIdentity recipe; recipe.recipe = "q8";
+        CHECK_THROWS(PreparedExperts(dir, s, recipe));
+    }
+    const std::string receipt = slurp(dir / "verification.json");
+    spit(dir / "manifest.json", manifest + " "); CHECK_THROWS(PreparedExperts(dir, s));            // the receipt names another manifest
     spit(dir / "manifest.json", manifest);
+    { PreparedExperts again(dir, s); CHECK(again.layers() == 2); }        // the manifest's bytes decide, not its time stamps
+    std::filesystem::remove(dir / "verification.json"); CHECK_THROWS(PreparedExperts(dir, s));    // never verified
+    spit(dir / "verification.json", receipt);
+    {   // one byte of a record file flipped in place: same size, same name
+        std::fstream f(dir / "experts-00.bin", std::ios::in | std::ios::out | std::ios::binary);
+        f.seekg(4321); char c = 0; f.get(c); f.seekp(4321); f.put(char(c ^ 1));
+    }
+    bool named = false;
+    try { PreparedExperts p(dir, s); } catch (const std::exception& e) { named = std::string(e.what()) == "prepared file changed since verification: experts-00.bin"; }
+    CHECK(named);
+    named = false;
+    try { verify_prepared_experts(dir); } catch (const std::exception& e) { named = std::string(e.what()) == "prepared file differs from its manifest entry: experts-00.bin"; }
+    CHECK(named);                                                         // and a new receipt cannot be had for the changed bytes
+    {
+        std::fstream f(dir / "experts-00.bin", std::ios::in | std::ios::out | std::ios::binary);
+        f.seekg(4321); char c = 0; f.get(c); f.seekp(4321); f.put(char(c ^ 1));
+    }
+    CHECK_THROWS(PreparedExperts(dir, s));                                // the bytes are back, the receipt's time stamps are stale
+    verify_prepared_experts(dir);
+    { PreparedExperts again(dir, s); CHECK(again.layers() == 2); }
     std::filesystem::resize_file(dir / "experts-01.bin", std::filesystem::file_size(dir / "experts-01.bin") - 1); CHECK_THROWS(PreparedExperts(dir, s));
+    CHECK_THROWS(verify_prepared_experts(dir));
     std::filesystem::remove(dir / "experts-01.bin"); CHECK_THROWS(PreparedExperts(dir, s));
     CHECK_THROWS(PreparedExperts(root / "nowhere", s));
 

@@ -108,3 +108,62 @@ def test_capped_layer_at_the_stack_shape_against_the_oracle(ctx):
     st = capped.store.stats()
     assert st.misses >= 10 and st.hits > 0      # the second and third steps find most of their experts in the slots
     capped.close()
+
+
+def _stack_pair(ctx, cfg, seeds, skew, slots):
+    """The same layers twice: records resident in HBM, and records behind an expert store with `slots` HBM slots."""
+    resident = [workload.LayerWeights(ctx, cfg, seed, skew) for seed in seeds]
+    capped = workload.StoreBackedStack(ctx, cfg, seeds, skew, slots)
+    return resident, ctx.stack_create(cfg, [w.layer for w in resident], 8), capped, capped.decode_stack(8)
+
+
+def test_decode_stack_behind_a_store_equals_the_resident_stack(ctx):
+    # Three layers of 32 experts (96 records) behind ten HBM slots: every launch reads some records from their slots and
+    # the others from their pinned-host homes, fills follow between the launches, slots are given away again and again.
+    # The bytes must be those of the stack whose records all sit in HBM, at one token and at several, launch after launch.
+    cfg = workload.tiny_config(hidden=512, experts=32, topk=4, inter=512)
+    resident, full, capped, stack = _stack_pair(ctx, cfg, [51, 52, 53], ("normal", 0.5), slots=10)
+    assert ctx.stack_is_persistent(stack, 1) and ctx.stack_is_persistent(stack, 8)
+    n = 3 * 8 * cfg.topk
+    ids_a, w_a, ids_b, w_b = (ctx.alloc(n * 4) for _ in range(4))
+    for step, tokens in enumerate((1, 1, 3, 1, 8, 1, 1, 2, 1, 1, 5, 1, 1, 1)):
+        x = workload.hidden_rows(ctx, tokens, cfg.hidden, 7000 + step)
+        want, got = ctx.alloc(tokens * cfg.hidden * 4), ctx.alloc(tokens * cfg.hidden * 4)
+        traced = step % 2 == 0   # with the caller's trace buffers and with the stack's own
+        ctx.stack_decode(full, x, tokens, want, z.StackTrace(ids_a.ptr, w_a.ptr, None, None))
+        ctx.stack_decode(stack, x, tokens, got, z.StackTrace(ids_b.ptr, w_b.ptr, None, None) if traced else None)
+        ctx.moe_check()
+        assert got.numpy(f32).tobytes() == want.numpy(f32).tobytes(), f"step {step} ({tokens} tokens)"
+        if traced:
+            m = 3 * tokens * cfg.topk
+            assert ids_b.numpy(np.int32, m).tobytes() == ids_a.numpy(np.int32, m).tobytes()
+        for b in (x, want, got):
+            ctx.free(b)
+    seen, st = capped.store.table_stats(), capped.store.stats()
+    assert seen.reads == seen.slot_reads + seen.home_reads and seen.slot_reads > 0 and seen.home_reads > 10
+    assert seen.home_read_bytes == seen.home_reads * ctx.record_bytes(cfg)
+    assert seen.switched > 10 and st.evictions > 0 and st.misses + st.hits + seen.not_admitted == seen.reads
+    with pytest.raises(z.ZcError):   # layer by layer would need every record resident
+        x = workload.hidden_rows(ctx, 1, cfg.hidden, 1)
+        ctx.stack_decode(stack, x, 1, ids_a, layered=True)
+    ctx.stack_destroy(stack); ctx.stack_destroy(full)
+    capped.close()
+
+
+def test_stack_shape_behind_a_store(ctx):
+    # Two layers of the 48-layer configuration behind 40 slots (1024 records of 5.3 MB): a cold launch that reads all of its
+    # records over the host link, then launches that find them in HBM.
+    cfg = workload.config("F")
+    resident, full, capped, stack = _stack_pair(ctx, cfg, [81, 82], ("zipf", 1.1), slots=40)
+    for step, tokens in enumerate((1, 1, 8, 1)):
+        x = workload.hidden_rows(ctx, tokens, cfg.hidden, 7100 + step)
+        want, got = ctx.alloc(tokens * cfg.hidden * 4), ctx.alloc(tokens * cfg.hidden * 4)
+        ctx.stack_decode(full, x, tokens, want)
+        ctx.stack_decode(stack, x, tokens, got)
+        ctx.finish()   # the fills that the launch caused are given time to land
+        ctx.moe_check()
+        assert got.numpy(f32).tobytes() == want.numpy(f32).tobytes(), f"step {step} ({tokens} tokens)"
+    seen = capped.store.table_stats()
+    assert seen.home_reads >= 20 and seen.slot_reads > 0
+    ctx.stack_destroy(stack); ctx.stack_destroy(full)
+    capped.close()

@@ -180,3 +180,71 @@ def test_ids_are_checked():
         z.Store(None, 1, 4, RECORD, 0)
     assert s.layer_stats(0) == (0, 0)
     s.close()
+
+
+def test_record_table_shows_a_slot_only_while_it_holds_the_finished_record():
+    # The device-side view (zc_hip_store_table): entries start at the records' homes, move to a slot when the slot's fill has
+    # finished and a refresh has run, and go back home the moment the slot is given to another record.
+    import ctypes as C
+    s = make(3, layers=2, experts=8)
+    for layer in range(2):
+        for e in range(8):
+            put(s, layer, e)
+    homes = np.array([s.lib.zc_hip_store_backing(s.handle, l, e) for l in range(2) for e in range(8)], np.uint64)
+    table = s.table_entries()
+    assert (table == homes).all()
+
+    def shown_value(key):   # what a kernel would read as the record's first float
+        return float(np.ctypeslib.as_array(C.cast(int(table[key]), C.POINTER(C.c_float)), shape=(1,))[0])
+
+    def check_every_entry():
+        for key in range(16):
+            assert shown_value(key) == key
+
+    s.table_observe(0, [1, 2, 2, 1])            # two distinct records, both read from home; their fills start
+    st = s.table_stats()
+    assert (st.reads, st.slot_reads, st.home_reads, st.home_read_bytes) == (2, 0, 2, 2 * RECORD)
+    assert (table == homes).all()               # nothing moves before a refresh
+    s.table_refresh()
+    assert table[1] != homes[1] and table[2] != homes[2] and s.table_stats().switched == 2
+    check_every_entry()
+    s.table_observe(0, [1, 2])
+    st = s.table_stats()
+    assert (st.reads, st.slot_reads, st.home_reads) == (4, 2, 2)
+    assert s.stats().hits == 2 and s.stats().misses == 2
+
+    s.hold(1, 3)                                # a slow fill: the entry stays at home until it has finished
+    s.table_observe(1, [3])
+    s.table_refresh()
+    assert table[8 + 3] == homes[8 + 3]
+    s.table_observe(1, [3])                     # read from home again, joined to the fill in flight: no second fill
+    assert s.stats().loading_joins == 1 and s.stats().misses == 3
+    s.hold(1, 3, False)
+    s.table_refresh()
+    assert table[8 + 3] != homes[8 + 3]
+    check_every_entry()
+
+    s.table_observe(0, [4, 5, 6])               # three slots, three more records: earlier ones lose their slots at once
+    assert sum(table[k] != homes[k] for k in range(16)) <= 3
+    check_every_entry()                         # entries of evicted records are back at home before the slot is overwritten
+    s.table_refresh()
+    check_every_entry()
+    assert s.stats().evictions >= 3
+    s.resize(5)
+    check_every_entry()
+    s.clear()
+    assert (table == homes).all()
+    with pytest.raises(z.ZcError):
+        s.table_observe(0, [8])
+    s.close()
+
+
+def test_record_table_must_be_created_on_an_empty_store():
+    s = make(2)
+    use(s, 0, 1)
+    with pytest.raises(z.ZcError) as err:
+        s.table()
+    assert "while the store is empty" in str(err.value)
+    with pytest.raises(z.ZcError):
+        s.table_refresh()
+    s.close()

@@ -105,7 +105,87 @@ int open_file(const std::filesystem::path& path) {
 }
 constexpr uint64_t kAlignment = 16384;   // storage.cpp:374
 
+struct FileIdentity { uint64_t size, device, inode, mtime_ns, ctime_ns; };
+FileIdentity identity_of(const std::filesystem::path& path) {
+    struct stat st{};
+    if (::stat(path.c_str(), &st) != 0 || st.st_size < 0) throw std::runtime_error("missing prepared file");
+    return {uint64_t(st.st_size), uint64_t(st.st_dev), uint64_t(st.st_ino),
+            uint64_t(st.st_mtim.tv_sec) * 1000000000ull + uint64_t(st.st_mtim.tv_nsec),
+            uint64_t(st.st_ctim.tv_sec) * 1000000000ull + uint64_t(st.st_ctim.tv_nsec)};
+}
+bool plain_filename(const std::string& name) { return !name.empty() && std::filesystem::path(name).filename() == name && name != "." && name != ".."; }
+// Nanosecond stamps exceed 2^53: the receipt keeps them as decimal strings.
+std::string quoted(uint64_t v) { return "\"" + std::to_string(v) + "\""; }
+uint64_t stamp(const Json& j) {
+    const std::string& s = j.str(); uint64_t v = 0;
+    const auto r = std::from_chars(s.data(), s.data() + s.size(), v);
+    if (r.ec != std::errc() || r.ptr != s.data() + s.size()) throw std::runtime_error("invalid time stamp in the verification receipt");
+    return v;
+}
+
 }  // namespace
+
+// ---- SHA-256
+namespace {
+constexpr uint32_t kRound[64] = {
+    0x428a2f98, 0x71374491, 0xb5c0fbcf, 0xe9b5dba5, 0x3956c25b, 0x59f111f1, 0x923f82a4, 0xab1c5ed5, 0xd807aa98, 0x12835b01, 0x243185be, 0x550c7dc3,
+    0x72be5d74, 0x80deb1fe, 0x9bdc06a7, 0xc19bf174, 0xe49b69c1, 0xefbe4786, 0x0fc19dc6, 0x240ca1cc, 0x2de92c6f, 0x4a7484aa, 0x5cb0a9dc, 0x76f988da,
+    0x983e5152, 0xa831c66d, 0xb00327c8, 0xbf597fc7, 0xc6e00bf3, 0xd5a79147, 0x06ca6351, 0x14292967, 0x27b70a85, 0x2e1b2138, 0x4d2c6dfc, 0x53380d13,
+    0x650a7354, 0x766a0abb, 0x81c2c92e, 0x92722c85, 0xa2bfe8a1, 0xa81a664b, 0xc24b8b70, 0xc76c51a3, 0xd192e819, 0xd6990624, 0xf40e3585, 0x106aa070,
+    0x19a4c116, 0x1e376c08, 0x2748774c, 0x34b0bcb5, 0x391c0cb3, 0x4ed8aa4a, 0x5b9cca4f, 0x682e6ff3, 0x748f82ee, 0x78a5636f, 0x84c87814, 0x8cc70208,
+    0x90befffa, 0xa4506ceb, 0xbef9a3f7, 0xc67178f2};
+inline uint32_t rotr(uint32_t v, int n) { return (v >> n) | (v << (32 - n)); }
+}  // namespace
+Sha256::Sha256() : h_{0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19}, tail_{} {}
+void Sha256::block(const uint8_t* p) {
+    uint32_t w[64];
+    for (int i = 0; i < 16; ++i) w[i] = uint32_t(p[4 * i]) << 24 | uint32_t(p[4 * i + 1]) << 16 | uint32_t(p[4 * i + 2]) << 8 | p[4 * i + 3];
+    for (int i = 16; i < 64; ++i) {
+        const uint32_t s0 = rotr(w[i - 15], 7) ^ rotr(w[i - 15], 18) ^ (w[i - 15] >> 3), s1 = rotr(w[i - 2], 17) ^ rotr(w[i - 2], 19) ^ (w[i - 2] >> 10);
+        w[i] = w[i - 16] + s0 + w[i - 7] + s1;
+    }
+    uint32_t a = h_[0], b = h_[1], c = h_[2], d = h_[3], e = h_[4], f = h_[5], g = h_[6], h = h_[7];
+    for (int i = 0; i < 64; ++i) {
+        const uint32_t t1 = h + (rotr(e, 6) ^ rotr(e, 11) ^ rotr(e, 25)) + ((e & f) ^ (~e & g)) + kRound[i] + w[i];
+        const uint32_t t2 = (rotr(a, 2) ^ rotr(a, 13) ^ rotr(a, 22)) + ((a & b) ^ (a & c) ^ (b & c));
+        h = g; g = f; f = e; e = d + t1; d = c; c = b; b = a; a = t1 + t2;
+    }
+    h_[0] += a; h_[1] += b; h_[2] += c; h_[3] += d; h_[4] += e; h_[5] += f; h_[6] += g; h_[7] += h;
+}
+void Sha256::update(std::span<const std::byte> bytes) {
+    const uint8_t* p = reinterpret_cast<const uint8_t*>(bytes.data()); size_t n = bytes.size();
+    size_t held = size_t(bytes_ % 64); bytes_ += n;
+    if (held) {
+        const size_t take = std::min(n, 64 - held);
+        std::memcpy(tail_ + held, p, take); p += take; n -= take; held += take;
+        if (held < 64) return;
+        block(tail_);
+    }
+    for (; n >= 64; p += 64, n -= 64) block(p);
+    std::memcpy(tail_, p, n);
+}
+std::string Sha256::hex() {
+    const uint64_t bits = bytes_ * 8;
+    size_t held = size_t(bytes_ % 64);
+    tail_[held++] = 0x80;
+    if (held > 56) { std::memset(tail_ + held, 0, 64 - held); block(tail_); held = 0; }
+    std::memset(tail_ + held, 0, 56 - held);
+    for (int i = 0; i < 8; ++i) tail_[56 + i] = uint8_t(bits >> (56 - 8 * i));
+    block(tail_);
+    std::string out; constexpr char digits[] = "0123456789abcdef";
+    for (uint32_t v : h_) for (int s = 28; s >= 0; s -= 4) out += digits[(v >> s) & 15];
+    return out;
+}
+std::string sha256_hex(std::string_view text) {
+    Sha256 h; h.update(std::as_bytes(std::span<const char>(text.data(), text.size()))); return h.hex();
+}
+std::string sha256_hex_file(const std::filesystem::path& path) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("missing prepared file");
+    Sha256 h; std::vector<char> buffer(1 << 20);
+    while (f) { f.read(buffer.data(), std::streamsize(buffer.size())); h.update(std::as_bytes(std::span<const char>(buffer.data(), size_t(f.gcount())))); }
+    return h.hex();
+}
 
 Json Json::parse(std::string_view text) { Parser p{text}; Json j = p.value(); p.space(); if (p.i != text.size()) p.fail("trailing characters"); return j; }
 const Json::Object& Json::object() const { if (auto* o = std::get_if<Object>(&value)) return *o; throw std::out_of_range("JSON value is not an object"); }
@@ -140,10 +220,33 @@ void ExpertSource::layer(uint32_t l, std::span<std::byte> into, uint64_t stride)
     for (uint32_t e = 0; e < shape_.experts; ++e) expert({l, e}, into.subspan(e * stride, bytes));
 }
 
-PreparedExperts::PreparedExperts(const std::filesystem::path& dir, const MoeShape& shape) : ExpertSource(shape) {
-    const Json m = Json::parse(read_text(dir / "manifest.json"));
-    if (!m.contains("schema") || m.at("schema").u64() != 1 || !m.contains("format") || m.at("format").str() != "zc-affine-records-v1")
-        throw std::runtime_error("unverified or incompatible prepared artifact");                       // storage.cpp:322-326
+PreparedExperts::PreparedExperts(const std::filesystem::path& dir, const MoeShape& shape, const PreparedIdentity& want) : ExpertSource(shape) {
+    const std::string text = read_text(dir / "manifest.json");
+    const Json m = Json::parse(text);
+    identity_ = sha256_hex(text);                                                                       // storage.cpp:318-320
+    const Json receipt = Json::parse(read_text(dir / "verification.json"));
+    const auto text_of = [](const Json& j, const char* key) { return j.contains(key) ? j.at(key).str() : std::string(); };
+    if (!m.contains("schema") || m.at("schema").u64() != 1 || text_of(m, "format") != "zc-affine-records-v1" ||
+        text_of(m, "source_revision") != want.source_revision || text_of(receipt, "manifest_sha256") != identity_ ||
+        text_of(receipt, "source_revision") != want.source_revision || text_of(m, "recipe") != want.recipe)
+        throw std::runtime_error("unverified or incompatible prepared artifact; run the verification pass");   // storage.cpp:322-326
+    if (!want.pinned_manifest_sha256.empty() && want.pinned_manifest_sha256 != identity_)
+        throw std::runtime_error("prepared manifest differs from the pinned one");                      // storage.cpp:327-329
+    std::map<std::string, bool> listed;
+    uint64_t total = 0;
+    for (size_t i = 0; i < m.at("files").size(); ++i) {                                                 // storage.cpp:337-350
+        const Json& entry = m.at("files").at(i);
+        const std::string& name = entry.at("path").str();
+        if (!plain_filename(name) || !listed.emplace(name, true).second) throw std::runtime_error("invalid prepared filename");
+        const Json& saved = receipt.at("files").at(name);
+        const FileIdentity now = identity_of(dir / name);
+        if (entry.at("size").u64() != now.size || saved.at("sha256").str() != entry.at("sha256").str() || saved.at("size").u64() != now.size ||
+            saved.at("device").u64() != now.device || saved.at("inode").u64() != now.inode || stamp(saved.at("mtime_ns")) != now.mtime_ns ||
+            stamp(saved.at("ctime_ns")) != now.ctime_ns)
+            throw std::runtime_error("prepared file changed since verification: " + name);
+        total += now.size;
+    }
+    if (m.at("prepared_bytes").u64() != total || listed.size() != m.at("experts").size()) throw std::runtime_error("incomplete prepared layout");   // storage.cpp:351-354
     const auto layout = expert_layout(shape);
     if (m.at("expert_layout").size() != 9) throw std::runtime_error("incomplete prepared layout");      // storage.cpp:352-354
     uint64_t offset = 0;
@@ -167,8 +270,9 @@ PreparedExperts::PreparedExperts(const std::filesystem::path& dir, const MoeShap
                 e.at("stride").u64() != stride_ || e.at("alignment").u64() != kAlignment)
                 throw std::runtime_error("unsupported prepared expert range");
             const std::string& name = e.at("file").str();
-            if (name.empty() || std::filesystem::path(name).filename() != name || name == "." || name == "..") throw std::runtime_error("invalid prepared filename");
+            if (!plain_filename(name)) throw std::runtime_error("invalid prepared filename");
             if (!used.emplace(name, true).second) throw std::runtime_error("duplicate prepared file range");
+            if (!listed.count(name)) throw std::runtime_error("prepared expert range names an unlisted file");
             files_.push_back(open_file(dir / name));
             if (file_size(files_.back()) != stride_ * shape.experts) throw std::runtime_error("invalid prepared expert length");
         }
@@ -234,12 +338,14 @@ void SafetensorsExperts::expert(ExpertKey key, std::span<std::byte> into) const 
 }
 
 void write_prepared_experts(const std::filesystem::path& dir, const MoeShape& shape, uint32_t layers,
-                            const std::function<void(ExpertKey, std::span<std::byte>)>& record) {
+                            const std::function<void(ExpertKey, std::span<std::byte>)>& record, const PreparedIdentity& identity) {
     std::filesystem::create_directories(dir);
     const auto layout = expert_layout(shape);
     const uint64_t bytes = shape.expert_bytes(), stride = (bytes + kAlignment - 1) / kAlignment * kAlignment;
     std::ostringstream m;
-    m << "{\n \"schema\": 1,\n \"format\": \"zc-affine-records-v1\",\n \"expert_layout\": [";
+    m << "{\n \"schema\": 1,\n \"format\": \"zc-affine-records-v1\",\n \"source_revision\": \"" << identity.source_revision
+      << "\",\n \"recipe\": \"" << identity.recipe << "\",\n \"expert_layout\": [";
+    std::ostringstream files; uint64_t total = 0;
     uint64_t offset = 0;
     for (size_t p = 0; p < 9; ++p) {
         m << (p ? "," : "") << "\n  {\"name\": \"" << layout[p].first << "\", \"offset\": " << offset << ", \"length\": " << layout[p].second
@@ -251,18 +357,45 @@ void write_prepared_experts(const std::filesystem::path& dir, const MoeShape& sh
     for (uint32_t l = 0; l < layers; ++l) {
         char name[32]; std::snprintf(name, sizeof name, "experts-%02u.bin", l);                        // prepare.cpp:272-273
         std::ofstream out(dir / name, std::ios::binary | std::ios::trunc);
+        Sha256 digest;
         for (uint32_t e = 0; e < shape.experts; ++e) {
             std::memset(buffer.data(), 0, buffer.size());                                               // the pad after the nine pieces is zero
             record({l, e}, std::span<std::byte>(buffer).first(bytes));
             out.write(reinterpret_cast<const char*>(buffer.data()), std::streamsize(stride));
+            digest.update(buffer);
         }
+        out.close();
         if (!out) throw std::runtime_error("cannot write " + (dir / name).string());
+        files << (l ? "," : "") << "\n  {\"path\": \"" << name << "\", \"size\": " << stride * shape.experts << ", \"sha256\": \"" << digest.hex() << "\"}";
+        total += stride * shape.experts;
         m << (l ? "," : "") << "\n  {\"layer\": " << l << ", \"file\": \"" << name << "\", \"count\": " << shape.experts << ", \"offset\": 0, \"length\": " << bytes
           << ", \"stride\": " << stride << ", \"alignment\": " << kAlignment << "}";
     }
-    m << "\n ]\n}\n";
-    std::ofstream f(dir / "manifest.json", std::ios::trunc); f << m.str();
+    m << "\n ],\n \"files\": [" << files.str() << "\n ],\n \"prepared_bytes\": " << total << "\n}\n";
+    std::ofstream f(dir / "manifest.json", std::ios::trunc); f << m.str(); f.close();
     if (!f) throw std::runtime_error("cannot write the prepared manifest");
+    verify_prepared_experts(dir);
+}
+
+void verify_prepared_experts(const std::filesystem::path& dir) {
+    const std::string text = read_text(dir / "manifest.json");
+    const Json m = Json::parse(text);
+    std::ostringstream r;
+    r << "{\n \"manifest_sha256\": \"" << sha256_hex(text) << "\",\n \"source_revision\": \"" << m.at("source_revision").str() << "\",\n \"files\": {";
+    for (size_t i = 0; i < m.at("files").size(); ++i) {
+        const Json& entry = m.at("files").at(i);
+        const std::string& name = entry.at("path").str();
+        if (!plain_filename(name)) throw std::runtime_error("invalid prepared filename");
+        const FileIdentity now = identity_of(dir / name);
+        const std::string digest = sha256_hex_file(dir / name);
+        if (now.size != entry.at("size").u64() || digest != entry.at("sha256").str())
+            throw std::runtime_error("prepared file differs from its manifest entry: " + name);
+        r << (i ? "," : "") << "\n  \"" << name << "\": {\"sha256\": \"" << digest << "\", \"size\": " << now.size << ", \"device\": " << now.device
+          << ", \"inode\": " << now.inode << ", \"mtime_ns\": " << quoted(now.mtime_ns) << ", \"ctime_ns\": " << quoted(now.ctime_ns) << "}";
+    }
+    r << "\n }\n}\n";
+    std::ofstream f(dir / "verification.json", std::ios::trunc); f << r.str(); f.close();
+    if (!f) throw std::runtime_error("cannot write the verification receipt");
 }
 
 }  // namespace zerocool::engine

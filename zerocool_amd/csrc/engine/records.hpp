@@ -8,8 +8,10 @@
 //    is gathered from nine slices (ExpertStore, src/engine/storage.cpp:493-516).
 // Both hand out records byte-identical to what the kernels expect (zc_hip_expert_linear), so a record read here can
 // be written straight into ExpertCache::home() or an HBM layer array.  No GPU is needed to use this file's classes.
-// The reference also pins file digests and a verification receipt (storage.cpp:318-353); that integrity layer is not
-// part of this reader: geometry and sizes are checked, contents are not hashed.
+// The prepared directory carries its identity as the reference's does (storage.cpp:316-349): manifest.json names the
+// source revision, the recipe and every file with its size and SHA-256; verification.json is the receipt of a
+// verification pass (the manifest's own SHA-256, the source revision, and per file the digest, size, device, inode,
+// mtime and ctime seen then).  PreparedExperts refuses a directory whose manifest, receipt and files disagree.
 #pragma once
 #include "engine.hpp"
 #include <filesystem>
@@ -33,6 +35,27 @@ struct Json {
     const Object& object() const;
 };
 
+// SHA-256 (FIPS 180-4), streaming; hex() gives 64 lowercase digits and may be called once.
+class Sha256 {
+public:
+    Sha256();
+    void update(std::span<const std::byte> bytes);
+    std::string hex();
+private:
+    void block(const uint8_t* p);
+    uint32_t h_[8]; uint8_t tail_[64]; uint64_t bytes_ = 0;
+};
+std::string sha256_hex(std::string_view text);
+std::string sha256_hex_file(const std::filesystem::path& path);
+
+// What a prepared directory must say about where it comes from.  The reference compiles these in (ModelRevision, the
+// recipe name and the manifest digest pinned in its model lock, storage.cpp:322-329); here the caller names them.
+struct PreparedIdentity {
+    std::string source_revision = "synthetic";
+    std::string recipe = "q4-control-lossless";
+    std::string pinned_manifest_sha256;     // empty: any verified manifest of this revision and recipe
+};
+
 class ExpertSource {
 public:
     virtual ~ExpertSource() = default;
@@ -48,14 +71,16 @@ protected:
 
 class PreparedExperts final : public ExpertSource {
 public:
-    PreparedExperts(const std::filesystem::path& dir, const MoeShape& shape);
+    PreparedExperts(const std::filesystem::path& dir, const MoeShape& shape, const PreparedIdentity& identity = {});
     ~PreparedExperts() override;
+    const std::string& identity() const { return identity_; }                  // SHA-256 of manifest.json (storage.cpp:318-320)
     uint32_t layers() const override { return uint32_t(files_.size()); }
     uint64_t stride() const { return stride_; }
     void expert(ExpertKey key, std::span<std::byte> into) const override;      // storage.cpp:391-394
 private:
     std::vector<int> files_;
     uint64_t stride_ = 0;
+    std::string identity_;
 };
 
 class SafetensorsExperts final : public ExpertSource {
@@ -76,7 +101,11 @@ private:
 std::array<std::pair<std::string, uint64_t>, 9> expert_layout(const MoeShape& shape);
 // Writes a prepared directory (manifest.json + experts-NN.bin) from a record generator, as the reference's prepare
 // step does from a checkpoint (prepare.cpp:268-300): used to convert synthetic or gathered records, and by the tests.
+// Ends with a verification pass, so the directory is ready to open.
 void write_prepared_experts(const std::filesystem::path& dir, const MoeShape& shape, uint32_t layers,
-                            const std::function<void(ExpertKey, std::span<std::byte>)>& record);
+                            const std::function<void(ExpertKey, std::span<std::byte>)>& record, const PreparedIdentity& identity = {});
+// The verification pass (the reference's `prepare_storage.py --verify`): re-reads every file the manifest names, compares
+// size and SHA-256 with the manifest and writes the receipt verification.json.  std::runtime_error when a file differs.
+void verify_prepared_experts(const std::filesystem::path& dir);
 
 }  // namespace zerocool::engine

@@ -680,6 +680,10 @@ struct zc_hip_stack {
     bool persistent_ok = false;
     // layered path
     void* workspace = nullptr; float *xa = nullptr, *xb = nullptr;
+    // routed records behind an expert store: the kernels take every record's address from the store's table
+    zc_hip_store* store = nullptr;
+    int32_t* route_ids = nullptr; float* route_weights = nullptr;   // [L][tokens][topk] device copies of every launch's routes
+    int32_t* route_ids_host = nullptr;                               // pinned
 };
 
 namespace {
@@ -691,19 +695,28 @@ uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : 8; }   // kernel
 }  // namespace
 
 extern "C" {
-zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* host_layers, uint32_t n_layers,
-                              uint32_t max_tokens, zc_hip_stack** out) {
+static zc_status create_stack(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* host_layers, uint32_t n_layers,
+                              uint32_t max_tokens, zc_hip_store* store, zc_hip_stack** out) {
     if (const zc_status s = validate_config(c)) return s;
     ZC_REQUIRE(ctx && host_layers && n_layers && max_tokens && max_tokens <= 8192 && out, "invalid stack geometry");
+    const void* const* table = nullptr;
+    if (store) {
+        uint32_t store_layers = 0, store_experts = 0; uint64_t store_record = 0;
+        if (const zc_status s = zc_hip_store_geometry(store, &store_layers, &store_experts, &store_record)) return s;
+        ZC_REQUIRE(store_layers == n_layers && store_experts == c->experts && store_record == zc_hip_record_bytes(c, 0),
+                   "the expert store does not hold this stack's records");
+        ZC_REQUIRE(max_tokens <= 8, "a stack behind an expert store decodes at most 8 tokens a launch");
+        if (const zc_status s = zc_hip_store_table(store, &table)) return s;
+    }
     for (uint32_t l = 0; l < n_layers; ++l) {
         const zc_moe_layer& y = host_layers[l];
-        ZC_REQUIRE(y.router && y.shared_gate && y.shared_record && y.expert_records, "missing MoE layer weights");
-        ZC_REQUIRE(y.record_stride >= zc_hip_record_bytes(c, 0) && y.record_stride % 16 == 0, "expert record stride is too small");
+        ZC_REQUIRE(y.router && y.shared_gate && y.shared_record && (store || y.expert_records), "missing MoE layer weights");
+        ZC_REQUIRE(store || (y.record_stride >= zc_hip_record_bytes(c, 0) && y.record_stride % 16 == 0), "expert record stride is too small");
         ZC_REQUIRE(reinterpret_cast<uintptr_t>(y.router) % 16 == 0 && reinterpret_cast<uintptr_t>(y.expert_records) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(y.shared_record) % 16 == 0, "MoE layer operands are misaligned");
     }
     auto* st = new zc_hip_stack;
-    st->cfg = *c; st->layers.assign(host_layers, host_layers + n_layers); st->max_tokens = max_tokens;
+    st->cfg = *c; st->layers.assign(host_layers, host_layers + n_layers); st->max_tokens = max_tokens; st->store = store;
     auto cleanup = [&](zc_status code) { zc_hip_stack_destroy(ctx, st); return code; };
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, ctx->device) != hipSuccess) return cleanup(fail(ZC_RUNTIME_ERROR, "HIP execution: cannot query device"));
@@ -744,20 +757,41 @@ zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         for (uint32_t l = 0; l < n_layers; ++l) {
             const zc_moe_layer& y = host_layers[l];
             host[l] = zc::DecodeLayer{static_cast<const uint16_t*>(y.router), y.router_offsets, static_cast<const uint16_t*>(y.shared_gate),
-                                      static_cast<const uint8_t*>(y.shared_record), static_cast<const uint8_t*>(y.expert_records), y.record_stride};
+                                      static_cast<const uint8_t*>(y.shared_record), static_cast<const uint8_t*>(y.expert_records), y.record_stride,
+                                      table ? reinterpret_cast<const uint8_t* const*>(table) + uint64_t(l) * c->experts : nullptr};
         }
         if (hipMemsetAsync(st->arena, 0, at, ctx->stream) != hipSuccess ||
             hipMemcpyAsync(st->dev_layers, host.data(), sizeof(zc::DecodeLayer) * n_layers, hipMemcpyHostToDevice, ctx->stream) != hipSuccess ||
             hipStreamSynchronize(ctx->stream) != hipSuccess)
             return cleanup(fail(ZC_RUNTIME_ERROR, "HIP execution: cannot initialise the decode stack"));
     }
+    if (store) {
+        if (!st->persistent_ok) return cleanup(fail(ZC_INVALID_ARGUMENT, "a stack behind an expert store needs a shape the single-launch kernels take"));
+        const uint64_t routes = uint64_t(n_layers) * max_tokens * k * 4;
+        if (zc_hip_alloc(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+        st->route_ids = static_cast<int32_t*>(p);
+        if (zc_hip_alloc(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+        st->route_weights = static_cast<float*>(p);
+        if (zc_hip_alloc_host(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+        st->route_ids_host = static_cast<int32_t*>(p);
+    }
     *out = st;
     return ZC_OK;
+}
+zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* host_layers, uint32_t n_layers,
+                              uint32_t max_tokens, zc_hip_stack** out) {
+    return create_stack(ctx, c, host_layers, n_layers, max_tokens, nullptr, out);
+}
+zc_status zc_hip_stack_create_with_store(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* host_layers, uint32_t n_layers,
+                                         uint32_t max_tokens, zc_hip_store* store, zc_hip_stack** out) {
+    ZC_REQUIRE(store, "null expert store");
+    return create_stack(ctx, c, host_layers, n_layers, max_tokens, store, out);
 }
 zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* st) {
     if (!st) return ZC_OK;
     ZC_REQUIRE(ctx, "null context");
-    for (void* p : {static_cast<void*>(st->workspace), static_cast<void*>(st->xa), static_cast<void*>(st->xb), static_cast<void*>(st->arena)})
+    for (void* p : {static_cast<void*>(st->workspace), static_cast<void*>(st->xa), static_cast<void*>(st->xb), static_cast<void*>(st->arena),
+                    static_cast<void*>(st->route_ids), static_cast<void*>(st->route_weights), static_cast<void*>(st->route_ids_host)})
         if (p) zc_hip_free(ctx, p);
     delete st;
     return ZC_OK;
@@ -802,6 +836,10 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
     const zc_moe_config& c = st->cfg;
     const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
     zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt = 0;
+    if (st->store) {
+        ZC_REQUIRE(!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt), "a stack behind an expert store runs as one launch only");
+        if (const zc_status s = zc_hip_store_table_refresh(st->store)) return s;
+    }
     if (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt)) {
         zc::DecodeParams p{};
         p.H = H; p.E = c.experts; p.topk = k; p.I = c.inter; p.T = tokens; p.L = L;
@@ -822,6 +860,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         }
         p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
         if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
+        if (st->store && !p.ids_trace) { p.ids_trace = st->route_ids; p.weights_trace = st->route_weights; }
         p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
         st->epoch += 4 * L + 16;   // at most four barriers per layer; wraps modulo 2^32, the barrier compares epochs as signed differences
@@ -833,6 +872,18 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         const uint32_t workgroups = uint32_t(st->cus);
         if (nt == 1) ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
         else ZC_HIP(zc::launch_decode_multi(ctx->stream, p, workgroups, multi));
+        if (st->store) {
+            // The launch has read every record through the store's table.  Once it has finished, the store learns which
+            // records those were: hits are touched, misses are admitted and their fills start on the side stream.
+            const uint64_t per_layer = uint64_t(tokens) * k;
+            ZC_HIP(hipMemcpyAsync(st->route_ids_host, p.ids_trace, L * per_layer * 4, hipMemcpyDeviceToHost, ctx->stream));
+            ZC_HIP(hipStreamSynchronize(ctx->stream));
+            int32_t status = 0;
+            ZC_HIP(hipMemcpy(&status, ctx->moe_status, 4, hipMemcpyDeviceToHost));
+            if (!status)   // ids of a launch that gave up are not routes
+                for (uint32_t l = 0; l < L; ++l)
+                    if (const zc_status s = zc_hip_store_table_observe(st->store, l, st->route_ids_host + l * per_layer, uint32_t(per_layer))) return s;
+        }
         return ZC_OK;
     }
     // layer by layer: y = moe(x); x_next = glue(y)

@@ -580,7 +580,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     const int32_t e = slot < k ? (pass == 0 ? uniform(pred[slot]) : uniform(ids[slot])) : 0;
                     if (e < 0 || e >= int32_t(E)) continue;   // no guess for the slot, or an id reported above (the combine drops the slot)
                     const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                    const uint8_t* rec = slot < k ? L.records + uint64_t(e) * L.stride : L.shared_record;
+                    const uint8_t* rec = slot < k ? record_of(L, e) : L.shared_record;
                     const uint64_t* off = slot < k ? p.ro : p.so;
                     const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
@@ -606,7 +606,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
                 const uint32_t e = uint32_t(uniform(experts[u / tiles])), tile = u % tiles;
                 const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                const uint8_t* rec = L.records + uint64_t(e) * L.stride;
+                const uint8_t* rec = record_of(L, e);
                 const uint8_t* w_row = rec + p.ro[pr] + uint64_t(row) * (H / 2);
                 const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64);
                 const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64);
@@ -652,7 +652,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     if (slot < k) {
                         const int32_t e = uniform(ids[slot]);
                         if (e < 0 || e >= int32_t(E)) { if (G == 0) otile[slot * 16 + col] = 0.0f * factor; continue; }
-                        rec = L.records + uint64_t(e) * L.stride; off = p.ro;
+                        rec = record_of(L, e); off = p.ro;
                     }
                     const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
@@ -783,7 +783,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         if (slot < k) {
                             const int32_t e = uniform(ids[slot]);
                             if (e < 0 || e >= int32_t(E)) continue;
-                            rec = L.records + uint64_t(e) * L.stride; off = p.ro;
+                            rec = record_of(L, e); off = p.ro;
                         }
                         const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
                         const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
@@ -795,7 +795,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 } else
                 for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
                     const uint8_t* rec; const uint64_t* off; int32_t s;
-                    if (u < U) { const uint32_t e = uint32_t(uniform(experts[u])); s = uniform(head[e]); rec = L.records + uint64_t(e) * L.stride; off = p.ro; }
+                    if (u < U) { const uint32_t e = uint32_t(uniform(experts[u])); s = uniform(head[e]); rec = record_of(L, e); off = p.ro; }
                     else { s = int32_t(n); rec = L.shared_record; off = p.so; }
                     const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);

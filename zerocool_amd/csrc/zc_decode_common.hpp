@@ -12,6 +12,11 @@ namespace zc {
 
 // A value every lane holds alike (read from LDS), moved to a scalar register so that control flow on it is scalar.
 __device__ __forceinline__ int32_t uniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+// Where expert e's record is: in the layer's own array, or wherever the expert store's table says (an HBM slot, or the
+// record's home in pinned host memory).  e is the same in every lane, so the table word comes through a scalar load.
+__device__ __forceinline__ const uint8_t* record_of(const DecodeLayer& L, uint32_t e) {
+    return L.table ? L.table[e] : L.records + uint64_t(e) * L.stride;
+}
 // Workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load in flight, which would
 // end a prefetch early.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }

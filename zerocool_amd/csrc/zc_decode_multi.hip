@@ -325,7 +325,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                 const uint32_t first = tiles * uint32_t(uniform(cum[ei])), seg_end = min(i1, tiles * uint32_t(uniform(cum[ei + 1])));
                 int32_t all[MT]; bool routed; uint32_t e;
                 const int na = slots_of(ei, all, routed, e);
-                const uint8_t* rec = routed ? L.records + uint64_t(e) * L.stride : L.shared_record;
+                const uint8_t* rec = routed ? record_of(L, e) : L.shared_record;
                 const uint64_t* off = routed ? p.ro : p.so;
                 const uint32_t passes = uint32_t(na + PT - 1) / PT;
                 for (uint32_t item = at + wave; item < seg_end; item += kMultiWaves) {
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                 }
                 __syncthreads();
                 xint_prepare_batch([&](uint32_t t) { return LdsBf16{ah + t * I}; }, uint32_t(na), LI, lds + lp.img_d);
-                const uint8_t* rec = routed ? L.records + uint64_t(e) * L.stride : L.shared_record;
+                const uint8_t* rec = routed ? record_of(L, e) : L.shared_record;
                 const uint64_t* off = routed ? p.ro : p.so;
                 const uint32_t passes = uint32_t(na + PT - 1) / PT;
                 for (uint32_t item = at + wave; item < seg_end; item += kMultiWaves) {

@@ -58,6 +58,7 @@ void launch_synth_records(hipStream_t s, void* records, uint64_t stride, uint32_
 struct DecodeLayer {
     const uint16_t* router; const float* offsets; const uint16_t* shared_gate;
     const uint8_t* shared_record; const uint8_t* records; uint64_t stride;
+    const uint8_t* const* table;   // if set: expert e's record is at table[e] (an expert store's view); else at records + e * stride
 };
 struct DecodeParams {
     uint32_t H, E, topk, I, T, L;

@@ -6,6 +6,7 @@
 // A store created without a context keeps its slots in ordinary host memory and finishes a fill when the caller
 // says so (zc_hip_store_hold): the policy can then be tested without a GPU, loading states included.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <cstring>
 #include <memory>
 #include <string>
@@ -20,7 +21,8 @@ struct zc_hip_store {
     zc_hip_ctx* ctx = nullptr;          // nullptr: host-memory slots
     uint32_t layers = 0, experts = 0;
     uint64_t record_bytes = 0, stride = 0;
-    uint8_t* backing = nullptr;         // [layers * experts] records, pinned host memory (or plain, without a context)
+    std::vector<uint8_t*> homes;        // per layer: [experts] records, pinned host memory (or plain, without a context); one allocation
+                                        // per layer, because a single pinned block for a large model can exceed what the driver grants
     uint8_t* pool = nullptr;            // [capacity] slots, HBM (or plain host memory)
     hipStream_t side = nullptr;
     std::vector<hipEvent_t> filled;     // per slot: recorded after the slot's last fill
@@ -29,11 +31,20 @@ struct zc_hip_store {
     std::unordered_set<uint64_t> held;  // host-memory store: keys whose fills wait
     std::unique_ptr<zc::SlotCache> cache;
     std::vector<uint64_t> layer_hits, layer_misses;
+    // Device-side view (zc_hip_store_table): one pointer per record, to its slot while the slot holds the finished record,
+    // to its home otherwise.  `mirror` is the host's copy (pinned), `table` what kernels read.
+    const uint8_t** mirror = nullptr; const uint8_t** table = nullptr;
+    bool table_changed = false;
+    std::vector<uint64_t> shown;        // per slot: the key whose table entry points at the slot, or ~0
+    std::vector<uint64_t> arriving;     // per slot: the key of a fill whose entry has not been switched to the slot yet, or ~0
+    std::vector<size_t> in_flight;      // the slots with an `arriving` key
+    zc_store_table_stats seen{};
 };
 
 namespace {
 constexpr uint64_t kNone = ~0ull;
 uint64_t key_of(const zc_hip_store* s, uint32_t layer, uint32_t expert) { return uint64_t(layer) * s->experts + expert; }
+uint8_t* home_of(const zc_hip_store* s, uint64_t key) { return s->homes[key / s->experts] + (key % s->experts) * s->stride; }
 
 template <class F> zc_status guarded(F f) {
     try { return f(); }
@@ -47,17 +58,27 @@ template <class F> zc_status guarded(F f) {
 void finish_host_fill(zc_hip_store* s, size_t slot) {
     const uint64_t key = s->pending[slot];
     if (key == kNone) return;
-    std::memcpy(s->pool + slot * s->stride, s->backing + key * s->stride, s->record_bytes);
+    std::memcpy(s->pool + slot * s->stride, home_of(s, key), s->record_bytes);
     s->pending[slot] = kNone;
+}
+// A fill of `slot` begins: whatever record the table showed there goes back to its home, and the new record's entry
+// stays at its home until zc_hip_store_table_refresh finds the fill finished.
+void table_fill_begins(zc_hip_store* s, size_t slot, uint64_t key) {
+    if (!s->mirror) return;
+    if (slot >= s->shown.size()) { s->shown.resize(slot + 1, kNone); s->arriving.resize(slot + 1, kNone); }
+    if (s->shown[slot] != kNone) { s->mirror[s->shown[slot]] = home_of(s, s->shown[slot]); s->shown[slot] = kNone; s->table_changed = true; }
+    if (s->arriving[slot] == kNone) s->in_flight.push_back(slot);
+    s->arriving[slot] = key;
 }
 zc::SlotCache::Hooks hooks_of(zc_hip_store* s) {
     zc::SlotCache::Hooks h;
     if (s->ctx) {
         h.start = [s](size_t slot, uint64_t key) {
+            table_fill_begins(s, slot, key);
             // The slot's previous record may still be read by kernels that were enqueued before its lease was released:
             // the fill is ordered after the compute stream's position at that release, on the device, without the host.
             ZC_STORE_HIP(hipStreamWaitEvent(s->side, s->released[slot], 0));
-            ZC_STORE_HIP(hipMemcpyAsync(s->pool + slot * s->stride, s->backing + key * s->stride, s->record_bytes, hipMemcpyHostToDevice, s->side));
+            ZC_STORE_HIP(hipMemcpyAsync(s->pool + slot * s->stride, home_of(s, key), s->record_bytes, hipMemcpyHostToDevice, s->side));
             ZC_STORE_HIP(hipEventRecord(s->filled[slot], s->side));
         };
         h.done = [s](size_t slot) {
@@ -73,7 +94,7 @@ zc::SlotCache::Hooks hooks_of(zc_hip_store* s) {
             ZC_STORE_HIP(hipEventRecord(s->filled[to], s->side));
         };
     } else {
-        h.start = [s](size_t slot, uint64_t key) { s->pending[slot] = key; if (!s->held.count(key)) finish_host_fill(s, slot); };
+        h.start = [s](size_t slot, uint64_t key) { table_fill_begins(s, slot, key); s->pending[slot] = key; if (!s->held.count(key)) finish_host_fill(s, slot); };
         h.done = [s](size_t slot) { return s->pending[slot] == kNone; };
         h.wait = [s](size_t slot) {
             if (s->pending[slot] != kNone && s->held.count(s->pending[slot])) throw std::logic_error("waiting for a fill that the test still holds");
@@ -82,6 +103,16 @@ zc::SlotCache::Hooks hooks_of(zc_hip_store* s) {
         h.move = [s](size_t from, size_t to) { std::memcpy(s->pool + to * s->stride, s->pool + from * s->stride, s->record_bytes); };
     }
     return h;
+}
+// After the slots moved or emptied (clear, resize; every fill has finished by then): the table from scratch.
+void table_rebuild(zc_hip_store* s) {
+    if (!s->mirror) return;
+    const uint64_t records = uint64_t(s->layers) * s->experts;
+    for (uint64_t key = 0; key < records; ++key) s->mirror[key] = home_of(s, key);
+    s->shown.assign(s->cache->capacity(), kNone); s->arriving.assign(s->cache->capacity(), kNone); s->in_flight.clear();
+    for (size_t slot = 0; slot < s->cache->capacity(); ++slot)
+        if (const int64_t key = s->cache->key_of(slot); key >= 0) { s->mirror[key] = s->pool + slot * s->stride; s->shown[slot] = uint64_t(key); }
+    s->table_changed = true;
 }
 // Slot storage for `slots` slots; keeps the bytes of the first `keep` slots.
 void provide_pool(zc_hip_store* s, uint64_t slots, uint64_t keep) {
@@ -122,15 +153,17 @@ zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts
     s->ctx = ctx; s->layers = layers; s->experts = experts; s->record_bytes = record_bytes; s->stride = (record_bytes + 255) / 256 * 256;
     s->layer_hits.assign(layers, 0); s->layer_misses.assign(layers, 0);
     const zc_status status = guarded([&] {
-        const uint64_t home = uint64_t(layers) * experts * s->stride;
-        if (ctx) {
-            void* p = nullptr;
-            if (zc_hip_alloc_host(ctx, home, &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
-            s->backing = static_cast<uint8_t*>(p);
-            ZC_STORE_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));   // default priority
-        } else {
-            s->backing = new uint8_t[home]();
+        const uint64_t home = uint64_t(experts) * s->stride;
+        for (uint32_t l = 0; l < layers; ++l) {
+            if (ctx) {
+                void* p = nullptr;
+                if (zc_hip_alloc_host(ctx, home, &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
+                s->homes.push_back(static_cast<uint8_t*>(p));
+            } else {
+                s->homes.push_back(new uint8_t[home]());
+            }
         }
+        if (ctx) ZC_STORE_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));   // default priority
         provide_pool(s.get(), slots, 0);
         s->cache = std::make_unique<zc::SlotCache>(slots, record_bytes, hooks_of(s.get()));
         return ZC_OK;
@@ -147,16 +180,18 @@ zc_status zc_hip_store_destroy(zc_hip_store* s) {
         for (hipEvent_t e : s->released) (void)hipEventDestroy(e);
         if (s->side) (void)hipStreamDestroy(s->side);
         if (s->pool) zc_hip_free(s->ctx, s->pool);
-        if (s->backing) zc_hip_free(s->ctx, s->backing);
+        for (uint8_t* h : s->homes) zc_hip_free(s->ctx, h);
+        if (s->table) zc_hip_free(s->ctx, s->table);
+        if (s->mirror) zc_hip_free(s->ctx, s->mirror);
     } else {
-        delete[] s->pool; delete[] s->backing;
+        delete[] s->pool; for (uint8_t* h : s->homes) delete[] h; delete[] s->mirror;
     }
     delete s;
     return ZC_OK;
 }
 void* zc_hip_store_backing(zc_hip_store* s, uint32_t layer, uint32_t expert) {
     if (!s || layer >= s->layers || expert >= s->experts) return nullptr;
-    return s->backing + key_of(s, layer, expert) * s->stride;
+    return home_of(s, key_of(s, layer, expert));
 }
 uint64_t zc_hip_store_stride(const zc_hip_store* s) { return s ? s->stride : 0; }
 uint64_t zc_hip_store_capacity(const zc_hip_store* s) { return s ? s->cache->capacity() : 0; }
@@ -203,7 +238,7 @@ int zc_hip_store_ready(zc_hip_store* s, uint32_t layer, uint32_t expert) {
 }
 zc_status zc_hip_store_clear(zc_hip_store* s) {
     if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
-    return guarded([&] { s->cache->clear(); return ZC_OK; });
+    return guarded([&] { s->cache->clear(); table_rebuild(s); return ZC_OK; });
 }
 zc_status zc_hip_store_resize(zc_hip_store* s, uint64_t slots) {
     if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
@@ -213,6 +248,7 @@ zc_status zc_hip_store_resize(zc_hip_store* s, uint64_t slots) {
         const uint64_t before = s->cache->capacity();
         if (slots > before) { provide_pool(s, slots, before); s->cache->resize(slots); }   // grow: storage first
         else { s->cache->resize(slots); if (slots < before) provide_pool(s, slots, slots); }   // shrink: survivors are compacted to the front first
+        table_rebuild(s);
         return ZC_OK;
     });
 }
@@ -228,6 +264,88 @@ zc_status zc_hip_store_layer_stats(const zc_hip_store* s, uint32_t layer, uint64
     if (misses) *misses = s->layer_misses[layer];
     return ZC_OK;
 }
+// ---- the device-side view
+zc_status zc_hip_store_table(zc_hip_store* s, const void* const** table) {
+    if (!s || !table) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    return guarded([&] {
+        if (!s->mirror) {
+            if (s->cache->occupancy()) throw std::logic_error("the record table must be created while the store is empty");
+            const uint64_t records = uint64_t(s->layers) * s->experts;
+            if (s->ctx) {
+                void* p = nullptr;
+                if (zc_hip_alloc_host(s->ctx, records * sizeof(void*), &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
+                s->mirror = static_cast<const uint8_t**>(p);
+                if (zc_hip_alloc(s->ctx, records * sizeof(void*), &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
+                s->table = static_cast<const uint8_t**>(p);
+            } else {
+                s->mirror = new const uint8_t*[records];
+                s->table = s->mirror;   // host-memory store: one copy serves both
+            }
+            for (uint64_t key = 0; key < records; ++key) s->mirror[key] = home_of(s, key);
+            s->shown.assign(s->cache->capacity(), kNone); s->arriving.assign(s->cache->capacity(), kNone);
+            s->table_changed = true;
+        }
+        *table = reinterpret_cast<const void* const*>(s->table);
+        return ZC_OK;
+    });
+}
+zc_status zc_hip_store_table_refresh(zc_hip_store* s) {
+    if (!s || !s->mirror) return zc_fail(ZC_LOGIC_ERROR, "the store has no record table");
+    return guarded([&] {
+        size_t kept = 0;
+        for (const size_t slot : s->in_flight) {
+            const uint64_t key = s->arriving[slot];
+            const bool done = s->ctx ? hipEventQuery(s->filled[slot]) == hipSuccess : s->pending[slot] == kNone;
+            if (!done) { s->in_flight[kept++] = slot; continue; }
+            s->arriving[slot] = kNone;
+            if (s->cache->key_of(slot) != int64_t(key)) continue;   // replaced before it was ever shown
+            s->mirror[key] = s->pool + slot * s->stride; s->shown[slot] = key; s->table_changed = true; ++s->seen.switched;
+        }
+        s->in_flight.resize(kept);
+        if (s->table_changed && s->ctx)
+            ZC_STORE_HIP(hipMemcpyAsync(s->table, s->mirror, uint64_t(s->layers) * s->experts * sizeof(void*), hipMemcpyHostToDevice,
+                                        static_cast<hipStream_t>(zc_hip_stream(s->ctx))));
+        s->table_changed = false;
+        return ZC_OK;
+    });
+}
+zc_status zc_hip_store_table_observe(zc_hip_store* s, uint32_t layer, const int32_t* ids, uint32_t count) {
+    if (!s || !s->mirror) return zc_fail(ZC_LOGIC_ERROR, "the store has no record table");
+    if (layer >= s->layers || (!ids && count)) return zc_fail(ZC_OUT_OF_RANGE, "invalid layer");
+    return guarded([&] {
+        std::vector<int32_t> distinct(ids, ids + count);
+        std::sort(distinct.begin(), distinct.end());
+        distinct.erase(std::unique(distinct.begin(), distinct.end()), distinct.end());
+        for (const int32_t e : distinct) {
+            if (e < 0 || uint32_t(e) >= s->experts) throw std::out_of_range("invalid expert id");
+            const uint64_t key = key_of(s, layer, uint32_t(e));
+            const uint8_t* at = s->mirror[key];
+            const bool from_slot = at >= s->pool && at < s->pool + s->cache->capacity() * s->stride;
+            ++s->seen.reads;
+            if (from_slot) ++s->seen.slot_reads; else { ++s->seen.home_reads; s->seen.home_read_bytes += s->record_bytes; }
+            // Touch (a hit) or admit (a miss: the fill starts now, for the launches to come); no lease stays out.
+            zc::SlotCache::Lease lease{};
+            try { lease = s->cache->acquire(key); }
+            catch (const std::runtime_error&) { ++s->seen.not_admitted; continue; }   // every slot is still loading: the record stays at home for now
+            if (lease.acquisition == zc::SlotCache::NewMiss) ++s->layer_misses[layer]; else ++s->layer_hits[layer];
+            s->cache->release(lease.slot);
+        }
+        return ZC_OK;
+    });
+}
+zc_status zc_hip_store_table_stats(const zc_hip_store* s, zc_store_table_stats* out) {
+    if (!s || !out) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    *out = s->seen;
+    return ZC_OK;
+}
+zc_status zc_hip_store_geometry(const zc_hip_store* s, uint32_t* layers, uint32_t* experts, uint64_t* record_bytes) {
+    if (!s) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    if (layers) *layers = s->layers;
+    if (experts) *experts = s->experts;
+    if (record_bytes) *record_bytes = s->record_bytes;
+    return ZC_OK;
+}
+
 zc_status zc_hip_store_hold(zc_hip_store* s, uint32_t layer, uint32_t expert, int hold) {
     if (!s || s->ctx) return zc_fail(ZC_LOGIC_ERROR, "fills can only be held in a store without a context");
     if (layer >= s->layers || expert >= s->experts) return zc_fail(ZC_OUT_OF_RANGE, "invalid expert id");

@@ -68,6 +68,10 @@ class StoreStats(C.Structure):
                                           "prefetches", "prefetch_claims", "prefetch_unclaimed")]
 
 
+class StoreTableStats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("reads", "slot_reads", "home_reads", "home_read_bytes", "switched", "not_admitted")]
+
+
 class StoreLease(C.Structure):
     _fields_ = [("lease", C.c_uint64), ("record", C.c_void_p), ("acquisition", C.c_int32)]
 
@@ -151,6 +155,29 @@ class Store:
         h, m = C.c_uint64(), C.c_uint64()
         self._check(self.lib.zc_hip_store_layer_stats(self.handle, C.c_uint32(layer), C.byref(h), C.byref(m)))
         return h.value, m.value
+
+    # the device-side view: a table of record addresses that kernels read
+    def table(self):
+        """Address of the table (creates it; the store must still be empty)."""
+        t = C.c_void_p()
+        self._check(self.lib.zc_hip_store_table(self.handle, C.byref(t)))
+        return t.value
+
+    def table_entries(self):
+        """Host-memory stores: the table as an array of addresses."""
+        return np.ctypeslib.as_array(C.cast(self.table(), C.POINTER(C.c_uint64)), shape=(self.layers * self.experts,))
+
+    def table_refresh(self):
+        self._check(self.lib.zc_hip_store_table_refresh(self.handle))
+
+    def table_observe(self, layer, ids):
+        ids = np.ascontiguousarray(ids, np.int32)
+        self._check(self.lib.zc_hip_store_table_observe(self.handle, C.c_uint32(layer), ids.ctypes.data_as(C.c_void_p), C.c_uint32(ids.size)))
+
+    def table_stats(self):
+        st = StoreTableStats()
+        self._check(self.lib.zc_hip_store_table_stats(self.handle, C.byref(st)))
+        return st
 
     def slot_bytes(self, lease):
         """Host-memory stores: the slot's current bytes."""
@@ -372,6 +399,12 @@ class Context:
         arr = (Layer * len(layers))(*layers)
         h = C.c_void_p()
         self._call("zc_hip_stack_create", C.byref(cfg), arr, C.c_uint32(len(layers)), C.c_uint32(max_tokens), C.byref(h))
+        return h
+
+    def stack_create_with_store(self, cfg, layers, max_tokens, store):
+        arr = (Layer * len(layers))(*layers)
+        h = C.c_void_p()
+        self._call("zc_hip_stack_create_with_store", C.byref(cfg), arr, C.c_uint32(len(layers)), C.c_uint32(max_tokens), store.handle, C.byref(h))
         return h
 
     def stack_destroy(self, stack):

@@ -103,6 +103,10 @@ class StoreBackedStack:
     def close(self):
         self.store.close()
 
+    def decode_stack(self, max_tokens=8):
+        """The single-launch decode stack over this store (zc_hip_stack_create_with_store)."""
+        return self.ctx.stack_create_with_store(self.cfg, [w.layer for w in self.layers], max_tokens, self.store)
+
     def layer_forward(self, l, x, T):
         ctx, cfg, w = self.ctx, self.cfg, self.layers[l]
         H, E, k, I = cfg.hidden, cfg.experts, cfg.topk, cfg.inter

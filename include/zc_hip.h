@@ -305,6 +305,18 @@ zc_status zc_hip_store_geometry(const zc_hip_store* store, uint32_t* layers, uin
  * refused with ZC_INVALID_ARGUMENT. */
 zc_status zc_hip_stack_create_with_store(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
                                          uint32_t n_layers, uint32_t max_tokens, zc_hip_store* store, zc_hip_stack** out);
+/* ---- Statistics and stage labels (Metal::label, metal.mm:267-270; KernelConfig::profile; Model::stats, model.cpp:706-732)
+ * zc_hip_profile(on != 0) starts a recording: from then on every operator call through the context adds one row -- the
+ * label current at the call, the operator's name, and the GPU time between two events placed around its launches (an
+ * operator that calls other operators counts once).  At most 16384 rows are kept; further calls are counted as dropped.
+ * zc_hip_label names the stage, layer, token count and token offset of the calls that follow; like the reference's it
+ * does nothing unless a recording is on.  zc_hip_stats waits for the context's stream and writes one JSON object:
+ * "memory", "profile" (per (stage, operator) call counts and GPU microseconds, then the rows) and, with a store,
+ * "expert_cache" (the counters of zc_hip_store_stats and zc_hip_store_table_stats, capacity, occupancy).  *needed receives
+ * the text's length including the terminator; ZC_OUT_OF_RANGE with a truncated text if capacity is smaller. */
+zc_status zc_hip_label(zc_hip_ctx* ctx, const char* stage, int32_t layer, uint32_t tokens, uint32_t offset);
+zc_status zc_hip_profile(zc_hip_ctx* ctx, int on);
+zc_status zc_hip_stats(zc_hip_ctx* ctx, const zc_hip_store* store, char* json, uint64_t capacity, uint64_t* needed);
 /* Stores without a context only: fills of this record stay "loading" while held (what a slow read is to the reference's tests). */
 zc_status zc_hip_store_hold(zc_hip_store* store, uint32_t layer, uint32_t expert, int hold);
 

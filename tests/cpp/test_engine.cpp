@@ -215,6 +215,15 @@ static void test_moe_layer() {   // model.cpp:431-557 against the CPU oracle
     CHECK_THROWS(moe(gpu, w, x, 1));            // "invalid router output", model.cpp:459
     CHECK_THROWS(moe_resident(gpu, w, records, stride, x, 1));
     gpu.budget(gpu.allocated() + 16); CHECK_THROWS(gpu.allocate(1 << 20)); gpu.budget(0);   // "engine memory budget exceeded"
+    // Metal::label + KernelConfig::profile (metal.mm:267-270): the layer's calls appear under the stages that moe() names
+    KernelConfig profiled; profiled.profile = true; gpu.configure(profiled);
+    std::fill(x->floats().begin(), x->floats().end(), 0.25f);
+    (void)moe(gpu, w, x, 1); gpu.finish();
+    const std::string stats = gpu.statistics();
+    CHECK(stats.find("\"stage\": \"routed_expert\"") != std::string::npos && stats.find("\"operator\": \"gated_linear\"") != std::string::npos);
+    CHECK(stats.find("\"recording\": true") != std::string::npos && stats.find("\"rows_dropped\": 0") != std::string::npos);
+    gpu.configure(KernelConfig{});
+    CHECK(gpu.statistics().find("\"recording\": false") != std::string::npos);
 }
 static void test_expert_cache() {   // :336-348 on the GPU, and moe() reading its records through leases
     TEST("expert cache: leases pin HBM slots; a layer through a few slots equals the resident layer");

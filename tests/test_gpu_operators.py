@@ -279,3 +279,52 @@ def test_stack_glue_is_max_normalised(ctx):
     want = oracle.bf(y * (f32(1) / m))
     assert got.tobytes() == want.tobytes()
     assert np.nanmax(np.abs(got)) == 1.0
+
+
+def test_profile_rows_carry_the_labels_and_statistics_are_json(ctx):
+    # Metal::label + KernelConfig::profile (metal.mm:267-270) and Model::stats (model.cpp:706-732) through the C ABI.
+    from zerocool_amd import workload
+    cfg = workload.tiny_config(hidden=512, experts=32, topk=4, inter=512)
+    layers = [workload.LayerWeights(ctx, cfg, 60 + l, ("normal", 0.5)) for l in range(2)]
+    stack = ctx.stack_create(cfg, [w.layer for w in layers], 8)
+    x = workload.hidden_rows(ctx, 2, cfg.hidden, 11)
+    out, ws = ctx.alloc(2 * cfg.hidden * 4), ctx.alloc(ctx.moe_workspace_bytes(cfg, 2))
+    ctx.label("ignored", 7, 1, 0)                     # no recording yet: a label is a no-op, as in the reference
+    ctx.moe_forward(cfg, layers[0].layer, x, 2, out, ws)
+    quiet = ctx.stats()
+    assert quiet["profile"] == {"recording": False, "rows_recorded": 0, "rows_dropped": 0, "stages": [], "rows": []}
+    assert quiet["memory"]["allocated_bytes"] == ctx.allocated and quiet["memory"]["peak_bytes"] >= ctx.allocated
+    ctx.profile(True)
+    ctx.moe_forward(cfg, layers[0].layer, x, 2, out, ws)   # before any label
+    ctx.label("router", 3, 2, 5)
+    logits = ctx.router_logits(layers[0].router, x, 2, cfg.hidden, cfg.experts, layers[0].offsets)
+    ctx.label("experts", 3, 2, 5)
+    ctx.moe_forward(cfg, layers[1].layer, x, 2, out, ws)
+    ctx.moe_forward(cfg, layers[1].layer, x, 2, out, ws)
+    ctx.label("decode", -1, 2, 6)
+    ctx.stack_decode(stack, x, 2, out, layered=True)   # calls the layer operator twice inside: one row, its own
+    ctx.stack_decode(stack, x, 2, out)
+    ctx.profile(False)
+    ctx.moe_forward(cfg, layers[0].layer, x, 2, out, ws)   # not recorded
+    s = ctx.stats()
+    rows = s["profile"]["rows"]
+    assert [(r["stage"], r["operator"]) for r in rows] == [("unlabelled", "moe_forward"), ("router", "router_logits"), ("experts", "moe_forward"),
+                                                          ("experts", "moe_forward"), ("decode", "stack_decode"), ("decode", "stack_decode")]
+    assert rows[1]["layer"] == 3 and rows[1]["tokens"] == 2 and rows[1]["offset"] == 5 and rows[4]["layer"] == -1
+    assert all(0 < r["gpu_us"] < 1e5 for r in rows)
+    stages = {(e["stage"], e["operator"]): e for e in s["profile"]["stages"]}
+    assert stages[("experts", "moe_forward")]["calls"] == 2 and stages[("decode", "stack_decode")]["calls"] == 2
+    assert abs(stages[("experts", "moe_forward")]["gpu_us"] - rows[2]["gpu_us"] - rows[3]["gpu_us"]) < 1e-2
+    assert s["profile"]["recording"] is False and s["profile"]["rows_recorded"] == 6
+    ctx.profile(True)                                   # a new recording starts empty
+    assert ctx.stats()["profile"]["rows"] == []
+    ctx.profile(False)
+    store = z.Store(ctx, 1, 8, 4096, 3)
+    lease = store.acquire(0, 2); store.wait(lease); ctx.finish(); store.release(lease)
+    cache = ctx.stats(store)["expert_cache"]
+    assert (cache["capacity"], cache["occupancy"], cache["misses"], cache["hits"], cache["application_read_bytes"]) == (3, 1, 1, 0, 4096)
+    assert cache["record_table"]["reads"] == 0
+    store.close()
+    ctx.stack_destroy(stack)
+    for b in (x, out, ws, logits):
+        ctx.free(b)

@@ -71,7 +71,22 @@ uint64_t MoeShape::expert_bytes(bool shared) const { const auto c = abi(); retur
 Metal::Metal(MoeShape shape, int device) : shape_(shape) { check(zc_hip_create(device, 0, &ctx_)); }
 Metal::~Metal() { if (ctx_) zc_hip_destroy(ctx_); }
 void Metal::budget(uint64_t bytes) { budget_ = bytes; }
-void Metal::configure(KernelConfig config) { config.validate(); check(zc_hip_configure(ctx_, config.policy == "reference" ? 0u : 1u)); }
+void Metal::configure(KernelConfig config) {
+    config.validate();
+    check(zc_hip_configure(ctx_, config.policy == "reference" ? 0u : 1u));
+    check(zc_hip_profile(ctx_, config.profile ? 1 : 0));
+}
+void Metal::label(std::string stage, int layer, uint32_t tokens, uint32_t offset, std::span<const uint32_t>) {
+    check(zc_hip_label(ctx_, stage.c_str(), layer, tokens, offset));
+}
+std::string Metal::statistics(const zc_hip_store* store) const {
+    uint64_t needed = 0;
+    (void)zc_hip_stats(ctx_, store, nullptr, 0, &needed);
+    std::string text(needed, '\0');
+    check(zc_hip_stats(ctx_, store, text.data(), needed, &needed));
+    text.resize(std::strlen(text.c_str()));
+    return text;
+}
 uint64_t Metal::allocated() const { return zc_hip_allocated(ctx_); }
 uint64_t Metal::peak() const { return zc_hip_peak(ctx_); }
 std::string Metal::device_name() const { return zc_hip_version(); }

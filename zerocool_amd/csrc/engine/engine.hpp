@@ -55,6 +55,7 @@ struct Linear {
 // metal.hpp:17-43, the part that concerns this path
 struct KernelConfig {
     std::string policy = "exact-int";   // "reference": literal lane kernels everywhere
+    bool profile = false;               // record one timed row per operator call, tagged by Metal::label
     void validate() const;
 };
 
@@ -87,7 +88,9 @@ public:
     void budget(uint64_t bytes);
     void configure(KernelConfig config);
     bool direct_rows() const { return true; }
-    void label(std::string, int = -1, uint32_t = 0, uint32_t = 0, std::span<const uint32_t> = {}) {}
+    // metal.mm:267-270: names the stage of the calls that follow in the profile rows (nothing unless configure() asked for a profile)
+    void label(std::string stage, int layer = -1, uint32_t tokens = 0, uint32_t offset = 0, std::span<const uint32_t> experts = {});
+    std::string statistics(const zc_hip_store* store = nullptr) const;   // JSON text: memory, profile rows, expert cache counters
     // "moe_sum" and "scatter_experts" are the two kernels the path dispatches by name (model.cpp:555, pipeline.cpp:28)
     void dispatch(const std::string& name, std::initializer_list<Binding> buffers, std::initializer_list<uint32_t> params,
                   uint32_t x, uint32_t y = 1, uint32_t z = 1, uint32_t tx = 32, uint32_t ty = 1, uint32_t tz = 1);

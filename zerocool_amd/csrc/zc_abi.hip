@@ -4,6 +4,8 @@
 // of error before anything reaches the GPU.
 #include "../../include/zc_hip.h"
 #include "zc_kernels.hpp"
+#include <algorithm>
+#include <cstdio>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -56,7 +58,45 @@ struct zc_hip_ctx {
     uint32_t affine_policy = 1;        // 0 literal lane kernels, 1 exact-integer matrix-core kernels where possible
     void* static_scratch = nullptr;    // this device's copy of the static scratch array
     std::mutex mutex;
+    // Profiling (KernelConfig::profile + Metal::label, metal.mm:267-270): while on, every operator call made through this
+    // context records one row: the label current at the call, the operator's name and a pair of events around its launches.
+    struct Row { std::string stage; int32_t layer; uint32_t tokens, offset; const char* op; hipEvent_t begin, end; };
+    bool profile = false; int profile_depth = 0;
+    std::string stage = "unlabelled"; int32_t label_layer = -1; uint32_t label_tokens = 0, label_offset = 0;
+    std::vector<Row> rows; uint64_t rows_dropped = 0;
 };
+
+namespace {
+constexpr size_t kMaxProfileRows = 16384;
+// One row per outermost operator call: operators that call other operators (the layer-by-layer stack, the static-scratch
+// entry point) count once, under their own name.
+struct Timed {
+    zc_hip_ctx* ctx; hipEvent_t end = nullptr;
+    Timed(zc_hip_ctx* c, const char* op) : ctx(c) {
+        if (!ctx || !ctx->profile || ctx->profile_depth++ > 0) return;
+        if (ctx->rows.size() >= kMaxProfileRows) { ++ctx->rows_dropped; return; }
+        hipEvent_t begin = nullptr;
+        if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess || hipEventRecord(begin, ctx->stream) != hipSuccess) {
+            (void)hipGetLastError(); if (begin) (void)hipEventDestroy(begin); if (end) (void)hipEventDestroy(end); end = nullptr; ++ctx->rows_dropped; return;
+        }
+        ctx->rows.push_back({ctx->stage, ctx->label_layer, ctx->label_tokens, ctx->label_offset, op, begin, end});
+    }
+    ~Timed() {
+        if (!ctx || !ctx->profile) return;
+        --ctx->profile_depth;
+        if (end) (void)hipEventRecord(end, ctx->stream);
+    }
+};
+void json_text(std::string& out, const std::string& text) {
+    out += '"';
+    for (const char c : text) {
+        if (c == '"' || c == '\\') { out += '\\'; out += c; }
+        else if (static_cast<unsigned char>(c) < 0x20) { char b[8]; std::snprintf(b, sizeof b, "\\u%04x", c); out += b; }
+        else out += c;
+    }
+    out += '"';
+}
+}  // namespace
 
 extern "C" {
 
@@ -94,6 +134,7 @@ zc_status zc_hip_destroy(zc_hip_ctx* ctx) {
     hipStreamSynchronize(ctx->stream);
     for (auto e : ctx->tickets) hipEventDestroy(e);
     for (auto e : ctx->timer) if (e) hipEventDestroy(e);
+    for (auto& r : ctx->rows) { hipEventDestroy(r.begin); hipEventDestroy(r.end); }
     for (auto& b : ctx->blocks) hipFree(b.first);
     for (auto& b : ctx->host_blocks) hipHostFree(b.first);
     hipFree(ctx->moe_status);
@@ -185,6 +226,78 @@ zc_status zc_hip_timer_stop(zc_hip_ctx* ctx, float* milliseconds) {
     ZC_HIP(hipEventElapsedTime(milliseconds, ctx->timer[0], ctx->timer[1]));
     return ZC_OK;
 }
+zc_status zc_hip_label(zc_hip_ctx* ctx, const char* stage, int32_t layer, uint32_t tokens, uint32_t offset) {
+    ZC_REQUIRE(ctx && stage, "null argument");
+    if (ctx->profile) { ctx->stage = stage; ctx->label_layer = layer; ctx->label_tokens = tokens; ctx->label_offset = offset; }   // metal.mm:267-270: a no-op unless profiling
+    return ZC_OK;
+}
+zc_status zc_hip_profile(zc_hip_ctx* ctx, int on) {
+    ZC_REQUIRE(ctx, "null argument");
+    if (on && !ctx->profile) {   // a new recording: earlier rows go
+        ZC_HIP(hipStreamSynchronize(ctx->stream));
+        for (auto& r : ctx->rows) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
+        ctx->rows.clear(); ctx->rows_dropped = 0; ctx->profile_depth = 0;
+        ctx->stage = "unlabelled"; ctx->label_layer = -1; ctx->label_tokens = ctx->label_offset = 0;
+    }
+    ctx->profile = on != 0;
+    return ZC_OK;
+}
+zc_status zc_hip_stats(zc_hip_ctx* ctx, const zc_hip_store* store, char* json, uint64_t capacity, uint64_t* needed) {
+    ZC_REQUIRE(ctx && (json || !capacity), "null argument");
+    ZC_HIP(hipStreamSynchronize(ctx->stream));   // every recorded event has happened
+    std::string out = "{\"library\": ";
+    json_text(out, zc_hip_version());
+    out += ", \"device\": " + std::to_string(ctx->device);
+    out += ", \"memory\": {\"allocated_bytes\": " + std::to_string(ctx->allocated) + ", \"peak_bytes\": " + std::to_string(ctx->peak) +
+           ", \"budget_bytes\": " + std::to_string(ctx->budget) + "}";
+    // rows by (stage, operator) in order of first appearance, then the rows themselves
+    struct Sum { std::string stage; const char* op; uint64_t calls; double us; };
+    std::vector<Sum> sums; std::string rows;
+    char number[64];
+    for (const auto& r : ctx->rows) {
+        float ms = 0;
+        if (hipEventElapsedTime(&ms, r.begin, r.end) != hipSuccess) { (void)hipGetLastError(); continue; }
+        size_t at = 0;
+        while (at < sums.size() && !(sums[at].stage == r.stage && std::strcmp(sums[at].op, r.op) == 0)) ++at;
+        if (at == sums.size()) sums.push_back({r.stage, r.op, 0, 0.0});
+        ++sums[at].calls; sums[at].us += double(ms) * 1e3;
+        rows += rows.empty() ? "" : ", ";
+        rows += "{\"stage\": "; json_text(rows, r.stage);
+        std::snprintf(number, sizeof number, "%.3f", double(ms) * 1e3);
+        rows += ", \"layer\": " + std::to_string(r.layer) + ", \"tokens\": " + std::to_string(r.tokens) + ", \"offset\": " + std::to_string(r.offset) +
+                ", \"operator\": \"" + r.op + "\", \"gpu_us\": " + number + "}";
+    }
+    out += ", \"profile\": {\"recording\": " + std::string(ctx->profile ? "true" : "false") + ", \"rows_recorded\": " + std::to_string(ctx->rows.size()) +
+           ", \"rows_dropped\": " + std::to_string(ctx->rows_dropped) + ", \"stages\": [";
+    for (size_t i = 0; i < sums.size(); ++i) {
+        out += i ? ", " : "";
+        out += "{\"stage\": "; json_text(out, sums[i].stage);
+        std::snprintf(number, sizeof number, "%.3f", sums[i].us);
+        out += ", \"operator\": \"" + std::string(sums[i].op) + "\", \"calls\": " + std::to_string(sums[i].calls) + ", \"gpu_us\": " + number + "}";
+    }
+    out += "], \"rows\": [" + rows + "]}";
+    if (store) {   // Model::stats' "expert_cache" (model.cpp:706-732)
+        zc_store_stats c{}; zc_store_table_stats t{};
+        if (const zc_status s = zc_hip_store_stats(store, &c)) return s;
+        if (const zc_status s = zc_hip_store_table_stats(store, &t)) return s;
+        out += ", \"expert_cache\": {\"capacity\": " + std::to_string(zc_hip_store_capacity(store)) + ", \"occupancy\": " + std::to_string(zc_hip_store_occupancy(store)) +
+               ", \"hits\": " + std::to_string(c.hits) + ", \"misses\": " + std::to_string(c.misses) + ", \"evictions\": " + std::to_string(c.evictions) +
+               ", \"application_read_bytes\": " + std::to_string(c.bytes) + ", \"ready_hits\": " + std::to_string(c.ready_hits) +
+               ", \"loading_joins\": " + std::to_string(c.loading_joins) + ", \"prefetches\": " + std::to_string(c.prefetches) +
+               ", \"prefetch_claims\": " + std::to_string(c.prefetch_claims) + ", \"prefetch_unclaimed\": " + std::to_string(c.prefetch_unclaimed) +
+               ", \"record_table\": {\"reads\": " + std::to_string(t.reads) + ", \"slot_reads\": " + std::to_string(t.slot_reads) +
+               ", \"home_reads\": " + std::to_string(t.home_reads) + ", \"home_read_bytes\": " + std::to_string(t.home_read_bytes) +
+               ", \"switched\": " + std::to_string(t.switched) + ", \"not_admitted\": " + std::to_string(t.not_admitted) + "}}";
+    }
+    out += "}";
+    if (needed) *needed = out.size() + 1;
+    if (capacity) {
+        const size_t n = std::min<size_t>(out.size(), size_t(capacity) - 1);
+        std::memcpy(json, out.data(), n); json[n] = 0;
+        if (n < out.size()) return fail(ZC_OUT_OF_RANGE, "statistics buffer too small");
+    }
+    return ZC_OK;
+}
 uint64_t zc_hip_allocated(const zc_hip_ctx* ctx) { return ctx ? ctx->allocated : 0; }
 uint64_t zc_hip_peak(const zc_hip_ctx* ctx) { return ctx ? ctx->peak : 0; }
 void* zc_hip_stream(zc_hip_ctx* ctx) { return ctx ? ctx->stream : nullptr; }
@@ -271,6 +384,7 @@ static uint64_t weight_bytes(const zc_linear* l) {
 }
 
 zc_status zc_hip_linear_into(zc_hip_ctx* ctx, const zc_linear* l, const float* x, uint32_t tokens, float* out, int float_output) {
+    Timed timed(ctx, "linear");
     ZC_REQUIRE(ctx && l, "null argument");
     ZC_REQUIRE(tokens && l->input && l->output && x, "linear input shape");
     ZC_REQUIRE(l->weight, "missing linear weights");
@@ -292,6 +406,7 @@ zc_status zc_hip_linear_into(zc_hip_ctx* ctx, const zc_linear* l, const float* x
 }
 zc_status zc_hip_router_logits(zc_hip_ctx* ctx, const void* w, const float* x, uint32_t tokens, uint32_t hidden,
                                uint32_t experts, const float* offsets, float* logits) {
+    Timed timed(ctx, "router_logits");
     ZC_REQUIRE(ctx && w && x && logits && tokens && experts, "linear input shape");
     ZC_REQUIRE(hidden && hidden % 16 == 0, "router needs hidden divisible by 16");
     ZC_REQUIRE(reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0, "router operands must be 16-byte aligned");
@@ -303,6 +418,7 @@ zc_status zc_hip_router_logits(zc_hip_ctx* ctx, const void* w, const float* x, u
 }
 zc_status zc_hip_gated_linear(zc_hip_ctx* ctx, const zc_linear* gate, const zc_linear* up, const float* x, uint32_t x_rows,
                               uint32_t tokens, const int32_t* rows, float* out) {
+    Timed timed(ctx, "gated_linear");
     ZC_REQUIRE(ctx && gate && up, "null argument");
     ZC_REQUIRE(gate->quantized && up->quantized && gate->input == up->input && gate->output == up->output &&
                gate->group == up->group && gate->bits == up->bits, "fused gate/up requires matching affine matrices");
@@ -324,6 +440,7 @@ zc_status zc_hip_gated_linear(zc_hip_ctx* ctx, const zc_linear* gate, const zc_l
     return ZC_OK;
 }
 zc_status zc_hip_route(zc_hip_ctx* ctx, const float* logits, uint32_t tokens, uint32_t experts, uint32_t topk, int32_t* ids, float* weights) {
+    Timed timed(ctx, "route");
     ZC_REQUIRE(ctx && tokens && tokens <= 8192 && logits && ids && weights, "invalid route selection buffers");
     ZC_REQUIRE(experts && experts <= 1024 && topk && topk <= 128 && topk <= experts, "route selection supports at most 1024 experts and top-128");
     zc::launch_route(ctx->stream, logits, tokens, experts, topk, ids, weights);
@@ -332,6 +449,7 @@ zc_status zc_hip_route(zc_hip_ctx* ctx, const float* logits, uint32_t tokens, ui
 }
 zc_status zc_hip_build_dispatch(zc_hip_ctx* ctx, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t experts,
                                 int32_t* offsets, int32_t* slots, int32_t* selected, int32_t* count, int32_t* status) {
+    Timed timed(ctx, "build_dispatch");
     ZC_REQUIRE(ctx && ids && offsets && slots && selected && count && status && tokens && topk && experts, "invalid dispatch buffers");
     ZC_REQUIRE(experts <= 8192, "dispatch supports at most 8192 experts");
     zc::launch_dispatch(ctx->stream, ids, tokens, topk, experts, offsets, slots, nullptr, selected, count, status);
@@ -339,6 +457,7 @@ zc_status zc_hip_build_dispatch(zc_hip_ctx* ctx, const int32_t* ids, uint32_t to
     return ZC_OK;
 }
 zc_status zc_hip_scatter_experts(zc_hip_ctx* ctx, const float* x, const int32_t* positions, uint32_t n, uint32_t hidden, float* out) {
+    Timed timed(ctx, "scatter_experts");
     ZC_REQUIRE(ctx && x && positions && out && hidden, "invalid scatter buffers");
     if (!n) return ZC_OK;
     zc::launch_scatter(ctx->stream, x, positions, n, hidden, out);
@@ -347,36 +466,42 @@ zc_status zc_hip_scatter_experts(zc_hip_ctx* ctx, const float* x, const int32_t*
 }
 zc_status zc_hip_moe_sum(zc_hip_ctx* ctx, const float* experts, const float* weights, const float* shared, const float* gate,
                          uint32_t tokens, uint32_t hidden, uint32_t topk, float* out) {
+    Timed timed(ctx, "moe_sum");
     ZC_REQUIRE(ctx && experts && weights && shared && gate && out && tokens && hidden && topk, "invalid expert reduction buffers");
     zc::launch_moe_sum(ctx->stream, experts, weights, shared, gate, tokens, hidden, topk, out);
     ZC_LAUNCHED();
     return ZC_OK;
 }
 zc_status zc_hip_unary(zc_hip_ctx* ctx, const float* x, uint64_t n, uint32_t op, float* y) {
+    Timed timed(ctx, "unary");
     ZC_REQUIRE(ctx && x && y && n && op <= 4, "invalid unary operator or buffers");
     zc::launch_unary(ctx->stream, x, n, op, y);
     ZC_LAUNCHED();
     return ZC_OK;
 }
 zc_status zc_hip_binary(zc_hip_ctx* ctx, const float* x, const float* y, uint64_t n, uint32_t op, float* out) {
+    Timed timed(ctx, "binary");
     ZC_REQUIRE(ctx && x && y && out && n, "binary shape mismatch");
     zc::launch_binary(ctx->stream, x, y, n, op, out);
     ZC_LAUNCHED();
     return ZC_OK;
 }
 zc_status zc_hip_hc_mix(zc_hip_ctx* ctx, const float* x, const float* w, uint32_t tokens, uint32_t hidden, float* out) {
+    Timed timed(ctx, "hc_mix");
     ZC_REQUIRE(ctx && x && w && out && tokens && hidden && x != out && w != out, "invalid stream mix buffers");
     zc::launch_hc_mix(ctx->stream, x, w, tokens, hidden, out);
     ZC_LAUNCHED();
     return ZC_OK;
 }
 zc_status zc_hip_hc_add(zc_hip_ctx* ctx, const float* hyper, const float* x, const float* inject, uint32_t tokens, uint32_t hidden, float* out) {
+    Timed timed(ctx, "hc_add");
     ZC_REQUIRE(ctx && hyper && x && inject && out && tokens && hidden && x != out && inject != out, "invalid residual injection buffers");
     zc::launch_hc_add(ctx->stream, hyper, x, inject, tokens, hidden, out);
     ZC_LAUNCHED();
     return ZC_OK;
 }
 zc_status zc_hip_norm(zc_hip_ctx* ctx, const float* x, const void* w, uint32_t dtype, uint32_t group, uint32_t width, uint32_t tokens, float* out) {
+    Timed timed(ctx, "norm");
     ZC_REQUIRE(ctx && x && w && out && tokens && group && width && width % group == 0 && group <= 4096 && dtype <= 1, "normalization shape");
     zc::launch_norm(ctx->stream, x, w, dtype, group, width, tokens, out);
     ZC_LAUNCHED();
@@ -384,6 +509,7 @@ zc_status zc_hip_norm(zc_hip_ctx* ctx, const float* x, const void* w, uint32_t d
 }
 zc_status zc_hip_grouped_experts(zc_hip_ctx* ctx, const zc_moe_config* cfg, const void* const* records,
                                  const uint32_t* positions, uint32_t n, const float* x, float* out, float* scratch) {
+    Timed timed(ctx, "grouped_experts");
     if (const zc_status s = validate_config(cfg)) return s;
     ZC_REQUIRE(ctx && n && n <= 8 && records && positions && x && out && scratch && x != out && x != scratch && out != scratch,
                "invalid grouped expert geometry");
@@ -439,6 +565,7 @@ uint64_t zc_hip_moe_static_scratch_bytes(void) { return kStaticScratchBytes; }
 // allocates or frees: no hipMalloc / hipFree / hipHostMalloc, no stream or event creation, no host containers.
 zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
                                     float* out, const zc_moe_trace* trace) {
+    Timed timed(ctx, "moe_forward_static");
     if (const zc_status s = validate_config(c)) return s;
     ZC_REQUIRE(ctx && T, "invalid MoE layer buffers");
     ZC_REQUIRE(ctx->static_scratch, "the static scratch array was not located for this device");
@@ -453,6 +580,7 @@ zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* c, con
 }
 zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
                              float* out, void* workspace, const zc_moe_trace* trace) {
+    Timed timed(ctx, "moe_forward");
     if (const zc_status s = validate_config(c)) return s;
     ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
     ZC_REQUIRE(l->router && l->shared_gate && l->shared_record && l->expert_records, "missing MoE layer weights");
@@ -553,6 +681,7 @@ uint64_t zc_hip_moe_prefill_workspace_bytes(const zc_moe_config* cfg, uint32_t t
 }
 zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
                              float* out, void* workspace, const zc_moe_trace* trace) {
+    Timed timed(ctx, "moe_prefill");
     if (const zc_status s = validate_config(c)) return s;
     ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 group 64 with hidden and intermediate sizes that are multiples of 128");
     ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
@@ -654,6 +783,7 @@ zc_status zc_hip_moe_check(zc_hip_ctx* ctx) {
     return ZC_OK;
 }
 zc_status zc_hip_stack_glue(zc_hip_ctx* ctx, const float* y, uint32_t tokens, uint32_t hidden, float* x_next) {
+    Timed timed(ctx, "stack_glue");
     ZC_REQUIRE(ctx && y && x_next && tokens && hidden, "invalid glue buffers");
     zc::launch_stack_glue(ctx->stream, y, tokens, hidden, x_next);
     ZC_LAUNCHED();
@@ -831,6 +961,7 @@ int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t token
 }
 zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
                               const zc_stack_trace* trace, uint32_t flags) {
+    Timed timed(ctx, "stack_decode");
     ZC_REQUIRE(ctx && st && x && out && tokens && tokens <= st->max_tokens, "invalid stack decode buffers");
     ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && x != out, "invalid or overlapping linear output");
     const zc_moe_config& c = st->cfg;

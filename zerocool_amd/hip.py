@@ -392,6 +392,23 @@ class Context:
     def moe_check(self):
         self._call("zc_hip_moe_check")
 
+    # statistics -----------------------------------------------------------
+    def profile(self, on=True):
+        self._call("zc_hip_profile", C.c_int(int(on)))
+
+    def label(self, stage, layer=-1, tokens=0, offset=0):
+        self._call("zc_hip_label", stage.encode(), C.c_int32(layer), C.c_uint32(tokens), C.c_uint32(offset))
+
+    def stats(self, store=None):
+        """The statistics object of zc_hip_stats (memory, profile rows, expert cache counters) as a dict."""
+        import json
+        needed = C.c_uint64(0)
+        handle = store.handle if store is not None else None
+        self.lib.zc_hip_stats(self.handle, handle, None, C.c_uint64(0), C.byref(needed))
+        buf = C.create_string_buffer(needed.value)
+        self._call("zc_hip_stats", handle, buf, C.c_uint64(needed.value), C.byref(needed))
+        return json.loads(buf.value.decode())
+
     def stack_glue(self, y, tokens, hidden, out):
         self._call("zc_hip_stack_glue", _ptr(y), C.c_uint32(tokens), C.c_uint32(hidden), _ptr(out))
 

@@ -29,13 +29,13 @@ INPUTS = 8   # distinct token batches the timed steps cycle through
 sys.path.insert(0, ROOT)
 
 
-def single_layer(ctx, name, tokens, prefill, reps, warmup=3):
+def single_layer(ctx, name, tokens, prefill, reps, warmup=3, skew=("zipf", 1.1)):
     """One MoE layer of a single-layer configuration (hidden 2048, 512 experts, top-10, intermediate 512), timed with
     weights and inputs resident.  FLOP count: 2 * tokens * hidden * intermediate * 3 projections * (top-k + shared)
     + the router product."""
     from zerocool_amd import workload
     c = workload.config(name)
-    lw = workload.LayerWeights(ctx, c, workload.BASE_SEED + 77, ("zipf", 1.1))
+    lw = workload.LayerWeights(ctx, c, workload.BASE_SEED + 77, skew)
     x = workload.hidden_rows(ctx, tokens, c.hidden, workload.BASE_SEED + 78 + tokens)
     out = ctx.alloc(tokens * c.hidden * 4)
     ws = ctx.alloc(ctx.moe_prefill_workspace_bytes(c, tokens) if prefill else ctx.moe_workspace_bytes(c, tokens))
@@ -51,7 +51,8 @@ def single_layer(ctx, name, tokens, prefill, reps, warmup=3):
         ctx.free(b)
     flops = 2.0 * tokens * c.hidden * c.inter * 3 * (c.topk + 1) + 2.0 * tokens * c.hidden * c.experts
     return {"tokens": tokens, "us_per_layer": ms_layer * 1e3, "tokens_per_s": tokens / (ms_layer * 1e-3),
-            "TFLOPs": flops / (ms_layer * 1e-3) / 1e12, "path": "bf16 matrix-core prefill" if prefill else "exact operator path"}
+            "TFLOPs": flops / (ms_layer * 1e-3) / 1e12, "router_skew": list(skew) if skew else None,
+            "path": "bf16 matrix-core prefill" if prefill else "exact operator path"}
 
 
 def write_traffic_file(fetch_dir, write_dir):
@@ -83,13 +84,13 @@ def write_traffic_file(fetch_dir, write_dir):
 
 
 def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), speculate=True):
-    """The same single-layer configuration through the persistent decode kernel as a stack of one layer: one launch per
-    step, over 8 distinct inputs in rotation."""
+    """The same single-layer configuration through the persistent decode kernels as a stack of one layer: one launch per
+    step up to eight tokens, one launch per eight tokens above that; over 8 distinct inputs in rotation."""
     import numpy as np
     from zerocool_amd import workload
     c = workload.config(name)
     lw = workload.LayerWeights(ctx, c, workload.BASE_SEED + 77, skew)
-    stack = ctx.stack_create(c, [lw.layer], 8)
+    stack = ctx.stack_create(c, [lw.layer], max(8, tokens))
     ctx.stack_set_speculation(stack, speculate)
     xs = [workload.hidden_rows(ctx, tokens, c.hidden, workload.BASE_SEED + 78 + tokens + 97 * i) for i in range(INPUTS)]
     out = ctx.alloc(tokens * c.hidden * 4)
@@ -118,13 +119,17 @@ def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), spec
 
 
 def prefill_workload(ctx, args):
-    r = single_layer(ctx, "S", 2048, True, args.steps, args.warmup)
+    # The configuration names no router skew: the headline is the unskewed layer (every expert is touched, about 40 rows
+    # each); the same layer behind Zipf(1.1) router offsets (a third of the experts, most rows on ten of them) stands beside it.
+    r = single_layer(ctx, "S", args.prefill_tokens, True, args.steps, args.warmup, skew=None)
+    skewed = single_layer(ctx, "S", args.prefill_tokens, True, args.steps, args.warmup)
     print(json.dumps({
         "metric": "moe_prefill_tokens_per_s", "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["us_per_layer"] * 1e-3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u4 codes as bf16 x bf16 inputs, fp32 accumulation", "data": "synthetic (seeded generator)",
         "config": {"workload": "BASELINE configs[3]: one MoE layer, 2048-token prefill batch, hidden 2048, 512 experts, top-10, "
-                               "intermediate 512, affine Q4 group 64", "tokens": 2048},
+                               "intermediate 512, affine Q4 group 64, no router skew", "tokens": args.prefill_tokens,
+                   "with_zipf_1.1_router_offsets": {"us_per_layer": skewed["us_per_layer"], "tokens_per_s": skewed["tokens_per_s"], "TFLOPs": skewed["TFLOPs"]}},
         "roofline": {"bound": "mfma", "achieved": r["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s", "frac": r["TFLOPs"] / 2500.0,
                      "traffic": None, "kernel": "zc::prefill_gemm_kernel (whole-layer rate: router, routing, dispatch, "
                                                 "both grouped products, exact recomputation and combine included)"}}))
@@ -142,6 +147,7 @@ def main():
     ap.add_argument("--workload", choices=("stack", "prefill"), default="stack",
                     help="stack: the 48-layer decode stack (the headline); prefill: one 2048-token batch through one layer of "
                          "hidden 2048 / 512 experts / top-10 / intermediate 512 on the bf16 matrix cores")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="--workload prefill: tokens of the batch")
     ap.add_argument("--capped-layers", type=int, default=12, help="--extra: layers of the capped-HBM run (48 pins 130 GB of host memory)")
     ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
@@ -334,7 +340,7 @@ def main():
         capped.close()
         # Single-layer configurations: decode batches through the exact operator path, and batches through the
         # sorted-token grouped product on the bf16 matrix cores.
-        extra["single_layer_q4_one_launch"] = [one_launch_layer(ctx, "S", t, 200) for t in (1, 8)]
+        extra["single_layer_q4_one_launch"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50) for t in (1, 8, 32, 64)]
         # raw random inputs behind an unskewed router share next to no experts from one step to the next: every guess of
         # the one-token kernel misses, which prices the guessing at its worst
         extra["single_layer_q4_one_launch_all_guesses_miss"] = [one_launch_layer(ctx, "S", 1, 200, skew=None, speculate=on) for on in (True, False)]

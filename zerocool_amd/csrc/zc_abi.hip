@@ -944,34 +944,12 @@ static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, 
     }
     return per_cu >= 1;
 }
-zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t polls) {
-    ZC_REQUIRE(ctx && st, "null argument");
-    st->wait_limit = polls ? polls : 1u << 22;
-    return ZC_OK;
-}
-zc_status zc_hip_stack_set_speculation(zc_hip_ctx* ctx, zc_hip_stack* st, int on) {
-    ZC_REQUIRE(ctx && st, "null argument");
-    st->speculate = on != 0; st->pred_valid = false;
-    return ZC_OK;
-}
-int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
-    if (!ctx || !st) return 0;
-    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt;
-    return persistent_plan(ctx, st, tokens, &plan, &multi, &nt) ? 1 : 0;
-}
-zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
-                              const zc_stack_trace* trace, uint32_t flags) {
-    Timed timed(ctx, "stack_decode");
-    ZC_REQUIRE(ctx && st && x && out && tokens && tokens <= st->max_tokens, "invalid stack decode buffers");
-    ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && x != out, "invalid or overlapping linear output");
+// One launch of the persistent kernels: `tokens` (at most eight) rows starting at token `first` of a batch of `batch`.
+static zc_status launch_piece(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out, const zc_stack_trace* trace,
+                              uint32_t first, uint32_t batch, const zc::DecodeLdsPlan& plan, const zc::MultiLdsPlan& multi, uint32_t nt) {
     const zc_moe_config& c = st->cfg;
     const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
-    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt = 0;
-    if (st->store) {
-        ZC_REQUIRE(!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt), "a stack behind an expert store runs as one launch only");
-        if (const zc_status s = zc_hip_store_table_refresh(st->store)) return s;
-    }
-    if (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt)) {
+    {
         zc::DecodeParams p{};
         p.H = H; p.E = c.experts; p.topk = k; p.I = c.inter; p.T = tokens; p.L = L;
         for (int shared = 0; shared < 2; ++shared)
@@ -989,10 +967,13 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
             p.pred_in = st->pred_valid ? st->pred[st->pred_turn] : nullptr; p.pred_out = st->pred[st->pred_turn ^ 1u];
             st->pred_turn ^= 1u; st->pred_valid = true;
         }
-        p.ids_trace = trace ? trace->ids : nullptr; p.weights_trace = trace ? trace->weights : nullptr; p.out_trace = trace ? trace->outputs : nullptr;
-        if (p.ids_trace) ZC_REQUIRE(p.weights_trace, "a routing trace needs both ids and weights");
-        if (st->store && !p.ids_trace) { p.ids_trace = st->route_ids; p.weights_trace = st->route_weights; }
-        p.clocks = trace ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
+        // trace rows of this piece inside the whole batch's arrays
+        p.trace_tokens = batch;
+        p.ids_trace = trace && trace->ids ? trace->ids + uint64_t(first) * k : nullptr;
+        p.weights_trace = trace && trace->weights ? trace->weights + uint64_t(first) * k : nullptr;
+        p.out_trace = trace && trace->outputs ? trace->outputs + uint64_t(first) * H : nullptr;
+        if (st->store && !p.ids_trace) { p.ids_trace = st->route_ids + uint64_t(first) * k; p.weights_trace = st->route_weights + uint64_t(first) * k; }
+        p.clocks = trace && first == 0 ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
         st->epoch += 4 * L + 16;   // at most four barriers per layer; wraps modulo 2^32, the barrier compares epochs as signed differences
         // The tagged buffers are written by one-token launches only, so their tags advance with those launches only:
@@ -1003,11 +984,56 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         const uint32_t workgroups = uint32_t(st->cus);
         if (nt == 1) ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
         else ZC_HIP(zc::launch_decode_multi(ctx->stream, p, workgroups, multi));
+    }
+    return ZC_OK;
+}
+zc_status zc_hip_stack_set_wait_limit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t polls) {
+    ZC_REQUIRE(ctx && st, "null argument");
+    st->wait_limit = polls ? polls : 1u << 22;
+    return ZC_OK;
+}
+zc_status zc_hip_stack_set_speculation(zc_hip_ctx* ctx, zc_hip_stack* st, int on) {
+    ZC_REQUIRE(ctx && st, "null argument");
+    st->speculate = on != 0; st->pred_valid = false;
+    return ZC_OK;
+}
+int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
+    if (!ctx || !st) return 0;
+    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt;
+    if (tokens > 8)   // pieces of eight and the rest
+        return tokens <= st->max_tokens && !st->store && persistent_plan(ctx, st, 8, &plan, &multi, &nt) &&
+               (tokens % 8 == 0 || persistent_plan(ctx, st, tokens % 8, &plan, &multi, &nt)) ? 1 : 0;
+    return persistent_plan(ctx, st, tokens, &plan, &multi, &nt) ? 1 : 0;
+}
+zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
+                              const zc_stack_trace* trace, uint32_t flags) {
+    Timed timed(ctx, "stack_decode");
+    ZC_REQUIRE(ctx && st && x && out && tokens && tokens <= st->max_tokens, "invalid stack decode buffers");
+    ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && x != out, "invalid or overlapping linear output");
+    const zc_moe_config& c = st->cfg;
+    const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
+    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt = 0;
+    if (st->store) {
+        ZC_REQUIRE(!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt), "a stack behind an expert store runs as one launch only");
+        if (const zc_status s = zc_hip_store_table_refresh(st->store)) return s;
+    }
+    // More than eight tokens go through the single-launch kernels in pieces of eight, one launch per piece (tokens do not
+    // interact inside a layer): every piece streams the weights again, but stays on the device from the first layer to the last.
+    const bool pieces = !(flags & 1u) && tokens > 8 && persistent_plan(ctx, st, 8, &plan, &multi, &nt) &&
+                        (tokens % 8 == 0 || persistent_plan(ctx, st, tokens % 8, &plan, &multi, &nt));
+    if (pieces || (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt))) {
+        if (trace && trace->ids) ZC_REQUIRE(trace->weights, "a routing trace needs both ids and weights");
+        for (uint32_t first = 0; first < tokens; first += 8) {
+            const uint32_t piece = std::min(8u, tokens - first);
+            if (!persistent_plan(ctx, st, piece, &plan, &multi, &nt)) return fail(ZC_LOGIC_ERROR, "no single-launch plan for a piece of the batch");
+            if (const zc_status s = launch_piece(ctx, st, x + uint64_t(first) * H, piece, out + uint64_t(first) * H, trace, first, tokens, plan, multi, nt)) return s;
+        }
         if (st->store) {
             // The launch has read every record through the store's table.  Once it has finished, the store learns which
             // records those were: hits are touched, misses are admitted and their fills start on the side stream.
             const uint64_t per_layer = uint64_t(tokens) * k;
-            ZC_HIP(hipMemcpyAsync(st->route_ids_host, p.ids_trace, L * per_layer * 4, hipMemcpyDeviceToHost, ctx->stream));
+            const int32_t* routes = trace && trace->ids ? trace->ids : st->route_ids;
+            ZC_HIP(hipMemcpyAsync(st->route_ids_host, routes, L * per_layer * 4, hipMemcpyDeviceToHost, ctx->stream));
             ZC_HIP(hipStreamSynchronize(ctx->stream));
             int32_t status = 0;
             ZC_HIP(hipMemcpy(&status, ctx->moe_status, 4, hipMemcpyDeviceToHost));

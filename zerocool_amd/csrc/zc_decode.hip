@@ -516,7 +516,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             const int32_t e = ids[tid];
             if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); if constexpr (NT != 1) next[tid] = -1; }
             else if constexpr (NT != 1) next[tid] = atomicExch(&head[e], int32_t(tid));
-            if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * n + tid, e); st_f32(p.weights_trace + uint64_t(layer) * n + tid, weights[tid]); }
+            if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * p.trace_tokens * k + tid, e); st_f32(p.weights_trace + uint64_t(layer) * p.trace_tokens * k + tid, weights[tid]); }
             if (NT == 1 && wg == 0 && p.pred_out) p.pred_out[uint64_t(layer) * k + tid] = e;   // the next step's guess for this layer
         }
         // One token: slot j belongs to expert ids[j] and no two slots share an expert, so there is nothing to group.
@@ -859,7 +859,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 const uint64_t at = uint64_t(t) * H + rt * 16 + c;
                 if constexpr (NT == 1) ZC_ST(p.tout + (layer & 1u) * H + at, (__float_as_uint(y) & 0xffff0000u) | tag);   // y is BF16-valued
                 else st_f32(p.layer_out + at, y);
-                if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * T * H + at, y);
+                if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * p.trace_tokens * H + at, y);
                 if (layer + 1 == p.L) st_f32(p.out + at, y);
                 if constexpr (NT != 1) {   // one token: the next layer's staging finds the maximum itself
                     uint32_t m = __float_as_uint(y) & 0x7fffffffu;

@@ -239,7 +239,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
             const int32_t e = ids[tid];
             if (e < 0 || e >= int32_t(E)) atomicOr(p.status, 1);
             else { atomicOr(&chosen[e], 1u << (tid / k)); rank_of[uint32_t(e) * MT + tid / k] = uint8_t(tid % k); }
-            if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * n + tid, e); st_f32(p.weights_trace + uint64_t(layer) * n + tid, weights[tid]); }
+            if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * p.trace_tokens * k + tid, e); st_f32(p.weights_trace + uint64_t(layer) * p.trace_tokens * k + tid, weights[tid]); }
         }
         __syncthreads();
         // the distinct experts that own at least one slot, ascending ids
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
             for (uint32_t kk = 1; kk < 8 && kk < k; ++kk) sum += partial[kk];
             const float y = bf(bf(sum) + bf(gatev[t] * shared_out));
             st_f32(p.layer_out + idx, y);
-            if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * T * H + idx, y);
+            if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * p.trace_tokens * H + idx, y);
             if (layer + 1 == p.L) st_f32(p.out + idx, y);
             uint32_t m = __float_as_uint(y) & 0x7fffffffu;
             if (m > 0x7f800000u) m = 0;   // NaN does not take part in the maximum

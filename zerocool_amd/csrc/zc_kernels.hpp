@@ -76,7 +76,8 @@ struct DecodeParams {
     // before this step's ids are known), pred_out [L][topk] receives this step's; tspec [topk + 1][I]: the prediction pass's
     // activations, tagged like tact.
     const int32_t* pred_in; int32_t* pred_out; uint32_t* tspec;
-    int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][T][topk], [L][T][topk], [L][T][H]
+    int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][trace_tokens][topk], [L][trace_tokens][topk], [L][trace_tokens][H],
+    uint32_t trace_tokens;           // each already advanced to this launch's first token: a launch may be one piece of a larger batch
     uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
     uint32_t tag_base;               // one token: layer l exchanges under tag (tag_base + l) % 65535 + 1; advances only with one-token launches
     unsigned long long* clocks;      // optional [L * kDecodeStamps][workgroups] 100 MHz timestamps, one per workgroup

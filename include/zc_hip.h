@@ -251,6 +251,13 @@ typedef struct {
     int32_t acquisition; /* 0 new miss, 1 ready hit, 2 loading join (Lease::acquisition, storage.cpp:600-602) */
 } zc_store_lease;
 zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots, zc_hip_store** out);
+/* The same with the replacement policy by name (parse_cache_policy, storage.cpp:536-540): "clock" (second chance, the
+ * default) or "slru" (segmented LRU, storage.cpp:547-573: probation and protected queues, protected at most three quarters
+ * of the slots; takes no prefetches).  Any other name: ZC_INVALID_ARGUMENT "cache policy must be clock or slru". */
+zc_status zc_hip_store_create_with_policy(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots,
+                                          const char* policy, zc_hip_store** out);
+const char* zc_hip_store_policy(const zc_hip_store* store);                 /* "clock" or "slru" (ExpertCache::json "policy") */
+uint64_t zc_hip_store_protected_entries(const zc_hip_store* store);         /* ExpertCache::json "protected_entries" */
 zc_status zc_hip_store_destroy(zc_hip_store* store);
 void* zc_hip_store_backing(zc_hip_store* store, uint32_t layer, uint32_t expert);   /* HOST pointer: the record's home */
 uint64_t zc_hip_store_stride(const zc_hip_store* store);

@@ -248,3 +248,90 @@ def test_record_table_must_be_created_on_an_empty_store():
     with pytest.raises(z.ZcError):
         s.table_refresh()
     s.close()
+
+
+def make_slru(slots, layers=1, experts=16):
+    return z.Store(None, layers, experts, RECORD, slots, policy="slru")
+
+
+def test_slru_matches_an_independent_probation_protected_replay():   # test_qwen.cpp:334-367
+    with pytest.raises(z.ZcError) as err:
+        z.Store(None, 1, 16, RECORD, 4, policy="adaptive")
+    assert "cache policy must be clock or slru" in str(err.value)
+    assert make(2).policy == "clock"
+    for capacity in range(1, 9):
+        s = make_slru(capacity)
+        assert s.policy == "slru"
+        for e in range(12):
+            put(s, 0, e)
+        probation, protected, random = [], [], 1234
+        for step in range(300):
+            random = (random * 1664525 + 1013904223) & 0xffffffff
+            key = (random >> 16) % 12
+            hit = key in probation or key in protected
+            if hit:
+                (probation if key in probation else protected).remove(key)
+                protected.append(key)
+                if len(protected) > capacity * 3 // 4:
+                    probation.append(protected.pop(0))
+            else:
+                if len(probation) + len(protected) == capacity:
+                    probation.pop(0)
+                probation.append(key)
+            before = s.stats()
+            hits0, misses0 = before.hits, before.misses
+            lease = s.acquire(0, key); s.wait(lease)
+            assert value(s, lease) == key
+            s.release(lease)
+            after = s.stats()
+            assert after.hits - hits0 == int(hit) and after.misses - misses0 == int(not hit), (capacity, step)
+            assert s.protected_entries == len(protected), (capacity, step)
+            for e in range(12):
+                assert s.ready(0, e) == (e in probation or e in protected), (capacity, step, e)
+        assert s.occupancy == min(capacity, 12)
+        s.clear()
+        assert s.protected_entries == 0 and s.occupancy == 0
+        s.close()
+
+
+def test_slru_protects_loading_and_leased_slots_and_survives_resizing():   # test_qwen.cpp:368-391
+    s = make_slru(4)
+    for e in range(10):
+        put(s, 0, e)
+    for e in range(4):
+        use(s, 0, e)
+    for e in range(3):
+        use(s, 0, e)                       # protected: 0, 1, 2; probation: 3
+    s.hold(0, 4)
+    pending = s.acquire(0, 4)              # takes probation's 3; its fill stays in flight
+    assert pending.acquisition == 0 and not s.ready(0, 3)
+    use(s, 0, 5)                           # probation is busy: an eligible protected entry goes
+    assert not s.ready(0, 0)
+    join = s.acquire(0, 4)
+    assert join.acquisition == 2 and s.stats().loading_joins == 1
+    s.release(pending); s.release(join)    # the leases go while the read is still active: loading data cannot be overwritten
+    a, b, c = s.acquire(0, 1), s.acquire(0, 2), s.acquire(0, 5)
+    with pytest.raises(z.ZcError):
+        s.acquire(0, 6)
+    with pytest.raises(z.ZcError):
+        s.resize(2)
+    with pytest.raises(z.ZcError):
+        s.clear()
+    assert not s.prefetch(0, 7)            # segmented LRU takes no prefetches (storage.cpp:679)
+    s.hold(0, 4, False)
+    lease = s.acquire(0, 4); s.wait(lease)
+    assert value(s, lease) == 4
+    for l in (lease, a, b, c):
+        s.release(l)
+    s.resize(2)
+    assert s.occupancy == 2 and s.protected_entries <= 1
+    survivors = [e for e in range(6) if s.ready(0, e)]
+    misses = s.stats().misses
+    s.resize(8)
+    for e in survivors:
+        assert use(s, 0, e) == e
+    assert s.stats().misses == misses
+    s.clear()
+    use(s, 0, 9)
+    assert s.occupancy == 1
+    s.close()

@@ -148,7 +148,13 @@ void provide_pool(zc_hip_store* s, uint64_t slots, uint64_t keep) {
 extern "C" {
 
 zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots, zc_hip_store** out) {
+    return zc_hip_store_create_with_policy(ctx, layers, experts, record_bytes, slots, "clock", out);
+}
+zc_status zc_hip_store_create_with_policy(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots,
+                                          const char* policy, zc_hip_store** out) {
     if (!out || !layers || !experts || !record_bytes || !slots) return zc_fail(ZC_INVALID_ARGUMENT, "empty expert cache");
+    const std::string name = policy ? policy : "";
+    if (name != "clock" && name != "slru") return zc_fail(ZC_INVALID_ARGUMENT, "cache policy must be clock or slru");   // parse_cache_policy, storage.cpp:536-540
     auto s = std::make_unique<zc_hip_store>();
     s->ctx = ctx; s->layers = layers; s->experts = experts; s->record_bytes = record_bytes; s->stride = (record_bytes + 255) / 256 * 256;
     s->layer_hits.assign(layers, 0); s->layer_misses.assign(layers, 0);
@@ -165,7 +171,7 @@ zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts
         }
         if (ctx) ZC_STORE_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));   // default priority
         provide_pool(s.get(), slots, 0);
-        s->cache = std::make_unique<zc::SlotCache>(slots, record_bytes, hooks_of(s.get()));
+        s->cache = std::make_unique<zc::SlotCache>(slots, record_bytes, hooks_of(s.get()), name == "slru" ? zc::SlotCache::SegmentedLRU : zc::SlotCache::Clock);
         return ZC_OK;
     });
     if (status != ZC_OK) { zc_hip_store_destroy(s.release()); return status; }
@@ -258,6 +264,8 @@ zc_status zc_hip_store_stats(const zc_hip_store* s, zc_store_stats* out) {
     *out = zc_store_stats{c.hits, c.misses, c.evictions, c.bytes, c.ready_hits, c.loading_joins, c.prefetches, c.prefetch_claims, c.prefetch_unclaimed};
     return ZC_OK;
 }
+const char* zc_hip_store_policy(const zc_hip_store* s) { return s && s->cache->policy() == zc::SlotCache::SegmentedLRU ? "slru" : "clock"; }
+uint64_t zc_hip_store_protected_entries(const zc_hip_store* s) { return s ? s->cache->protected_entries() : 0; }
 zc_status zc_hip_store_layer_stats(const zc_hip_store* s, uint32_t layer, uint64_t* hits, uint64_t* misses) {
     if (!s || layer >= s->layers) return zc_fail(ZC_OUT_OF_RANGE, "invalid layer");
     if (hits) *hits = s->layer_hits[layer];

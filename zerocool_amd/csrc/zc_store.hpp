@@ -10,6 +10,11 @@
 //     unclaimed guess is the next victim; it never evicts a pinned or loading slot
 //   * counters: hits, misses, evictions, bytes, ready_hits, loading_joins, prefetches, prefetch_claims,
 //     prefetch_unclaimed (storage.hpp:183-192)
+//   * two replacement policies (storage.cpp:536-573): CLOCK second chance (the default), and segmented LRU -- a new
+//     record enters a probation queue, a hit moves it to the newest end of a protected queue that holds at most three
+//     quarters of the slots (its oldest entry drops back to probation's newest end), the victim is the oldest
+//     unpinned, finished entry of probation, then of protected ("a preference, never a pin").  Segmented LRU takes
+//     no prefetches, as in the reference.
 // One coordinator thread owns the object (storage.hpp:194-197); nothing here is thread safe.
 #pragma once
 #include <cstdint>
@@ -34,11 +39,17 @@ public:
         std::function<void(size_t from, size_t to)> move;          // copy a finished slot's bytes (resize compaction)
     };
     enum Acquisition { NewMiss = 0, ReadyHit = 1, LoadingJoin = 2 };
+    enum Policy { Clock = 0, SegmentedLRU = 1 };
     struct Lease { size_t slot; Acquisition acquisition; };
 
-    SlotCache(size_t slots, uint64_t record_bytes, Hooks hooks) : slots_(slots), record_bytes_(record_bytes), hooks_(std::move(hooks)) {
+    SlotCache(size_t slots, uint64_t record_bytes, Hooks hooks, Policy policy = Clock)
+        : slots_(slots), record_bytes_(record_bytes), hooks_(std::move(hooks)), policy_(policy) {
         if (!slots || !record_bytes) throw std::invalid_argument("empty expert cache");
+        if (policy != Clock && policy != SegmentedLRU) throw std::invalid_argument("cache policy must be clock or slru");
     }
+    Policy policy() const { return policy_; }
+    size_t protected_entries() const { return queue_[1].count; }
+    size_t probation_entries() const { return policy_ == SegmentedLRU ? queue_[0].count : 0; }
     size_t capacity() const { return slots_.size(); }
     size_t occupancy() const { return lookup_.size(); }
     const SlotCacheStats& stats() const { return stats_; }
@@ -49,15 +60,22 @@ public:
     Lease acquire(uint64_t key) {
         if (auto it = lookup_.find(key); it != lookup_.end()) {
             Entry& e = slots_[it->second];
-            e.referenced = true; ++stats_.hits;
+            touch(it->second); ++stats_.hits;
             const bool ready = hooks_.done(it->second);
             if (ready) ++stats_.ready_hits; else ++stats_.loading_joins;
             if (e.prefetched) { e.prefetched = false; ++stats_.prefetch_claims; }
             ++e.pins;
             return {it->second, ready ? ReadyHit : LoadingJoin};
         }
-        size_t selected = clock_victim();
-        while (selected == slots_.size()) {
+        size_t selected = slots_.size();
+        if (policy_ == SegmentedLRU) {
+            if (occupancy() == capacity()) selected = slru_victim();
+            else for (size_t trial = 0; trial < slots_.size() && selected == slots_.size(); ++trial) {   // free capacity first
+                const size_t slot = hand_; hand_ = (hand_ + 1) % slots_.size();
+                if (!slots_[slot].used) selected = slot;
+            }
+        } else selected = clock_victim();
+        while (selected == slots_.size() && policy_ == Clock) {
             // Unclaimed guesses load without a lease.  Wait for one to finish rather than failing an admission
             // that would fit once it does (storage.cpp:650-658).
             size_t guess = slots_.size();
@@ -72,6 +90,7 @@ public:
         place(selected, key);
         Entry& e = slots_[selected];
         e.referenced = true; e.prefetched = false; e.pins = 1;
+        if (policy_ == SegmentedLRU) link(selected, 0);
         hooks_.start(selected, key);
         ++stats_.misses; stats_.bytes += record_bytes_;
         return {selected, NewMiss};
@@ -82,7 +101,7 @@ public:
     }
     // storage.cpp:677-692
     bool prefetch(uint64_t key) {
-        if (lookup_.count(key)) return false;
+        if (policy_ != Clock || lookup_.count(key)) return false;
         const size_t selected = clock_victim();
         if (selected == slots_.size()) return false;
         place(selected, key);
@@ -102,7 +121,7 @@ public:
         drain();
         lookup_.clear();
         for (Entry& e : slots_) e = Entry{};
-        hand_ = 0;
+        hand_ = 0; queue_[0] = queue_[1] = Queue{};
     }
     // storage.cpp:708-725: a coordinator boundary; never invalidates a lease or a fill in flight; survivors keep their bytes
     void resize(size_t slots) {
@@ -112,32 +131,72 @@ public:
         if (slots >= slots_.size()) { slots_.resize(slots); return; }
         size_t occupied = lookup_.size();
         while (occupied > slots) {
-            const size_t victim = hand_; hand_ = (hand_ + 1) % slots_.size();
+            size_t victim = hand_; hand_ = (hand_ + 1) % slots_.size();
+            if (policy_ == SegmentedLRU) victim = slru_victim();   // nothing is pinned or loading here: there always is one
             Entry& e = slots_[victim];
             if (!e.used) continue;
-            if (e.referenced) { e.referenced = false; continue; }
+            if (policy_ == Clock && e.referenced) { e.referenced = false; continue; }
             if (e.prefetched) ++stats_.prefetch_unclaimed;
-            lookup_.erase(e.key); e = Entry{}; --occupied; ++stats_.evictions;
+            unlink(victim); lookup_.erase(e.key); e = Entry{}; --occupied; ++stats_.evictions;
         }
         size_t to = 0;
         lookup_.clear();
         for (size_t from = 0; from < slots_.size(); ++from) if (slots_[from].used) {
-            if (from != to) { hooks_.move(from, to); slots_[to] = slots_[from]; slots_[from] = Entry{}; }
+            if (from != to) { hooks_.move(from, to); relabel(from, to); slots_[to] = slots_[from]; slots_[from] = Entry{}; }
             lookup_[slots_[to].key] = to; ++to;
         }
         drain();
         slots_.resize(slots); hand_ = 0;
+        if (policy_ == SegmentedLRU) demote();
     }
     int64_t key_of(size_t slot) const { return slots_[slot].used ? int64_t(slots_[slot].key) : -1; }
 
 private:
-    struct Entry { uint64_t key = 0; unsigned pins = 0; bool used = false, referenced = false, prefetched = false; };
+    static constexpr size_t kNoSlot = ~size_t(0);
+    // A slot's place in the probation (0) or protected (1) queue: links are slot numbers, oldest first.
+    struct Entry {
+        uint64_t key = 0; unsigned pins = 0; bool used = false, referenced = false, prefetched = false;
+        int listed = -1; size_t older = kNoSlot, newer = kNoSlot;
+    };
+    struct Queue { size_t oldest = kNoSlot, newest = kNoSlot, count = 0; };
+    void unlink(size_t slot) {
+        Entry& e = slots_[slot];
+        if (e.listed < 0) return;
+        Queue& q = queue_[e.listed];
+        if (e.older != kNoSlot) slots_[e.older].newer = e.newer; else q.oldest = e.newer;
+        if (e.newer != kNoSlot) slots_[e.newer].older = e.older; else q.newest = e.older;
+        --q.count; e.listed = -1; e.older = e.newer = kNoSlot;
+    }
+    void link(size_t slot, int which) {
+        Entry& e = slots_[slot]; Queue& q = queue_[which];
+        e.listed = which; e.older = q.newest; e.newer = kNoSlot;
+        if (q.newest != kNoSlot) slots_[q.newest].newer = slot; else q.oldest = slot;
+        q.newest = slot; ++q.count;
+    }
+    void demote() { while (queue_[1].count > 3 * capacity() / 4) { const size_t slot = queue_[1].oldest; unlink(slot); link(slot, 0); } }
+    void touch(size_t slot) {   // storage.cpp:563-566
+        if (policy_ == Clock) { slots_[slot].referenced = true; return; }
+        unlink(slot); link(slot, 1); demote();
+    }
+    size_t slru_victim() const {   // storage.cpp:567-572
+        for (const Queue& q : queue_)
+            for (size_t slot = q.oldest; slot != kNoSlot; slot = slots_[slot].newer)
+                if (!slots_[slot].pins && hooks_.done(slot)) return slot;
+        return slots_.size();
+    }
+    void relabel(size_t from, size_t to) {   // the entry of slot `from` is about to live in slot `to`: its neighbours and queue ends follow
+        const Entry& e = slots_[from];
+        if (e.listed < 0) return;
+        Queue& q = queue_[e.listed];
+        if (e.older != kNoSlot) slots_[e.older].newer = to; else q.oldest = to;
+        if (e.newer != kNoSlot) slots_[e.newer].older = to; else q.newest = to;
+    }
     void drain() { for (size_t i = 0; i < slots_.size(); ++i) if (slots_[i].used) hooks_.wait(i); }
     void place(size_t slot, uint64_t key) {   // storage.cpp:606-613
         Entry& old = slots_[slot];
         if (old.used) {
             if (old.prefetched) ++stats_.prefetch_unclaimed;
-            lookup_.erase(old.key); ++stats_.evictions;
+            unlink(slot); lookup_.erase(old.key); ++stats_.evictions;
         }
         old = Entry{}; old.used = true; old.key = key;
         lookup_[key] = slot;
@@ -160,6 +219,8 @@ private:
     size_t hand_ = 0;
     uint64_t record_bytes_;
     Hooks hooks_;
+    Policy policy_ = Clock;
+    Queue queue_[2];
     SlotCacheStats stats_;
 };
 

@@ -52,8 +52,12 @@ def load_library():
     lib.zc_hip_last_error.restype = C.c_char_p
     lib.zc_hip_version.restype = C.c_char_p
     for name in ("zc_hip_allocated", "zc_hip_peak", "zc_hip_moe_workspace_bytes", "zc_hip_moe_prefill_workspace_bytes", "zc_hip_projection_bytes",
-                 "zc_hip_record_bytes", "zc_hip_moe_static_scratch_bytes", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy"):
+                 "zc_hip_record_bytes", "zc_hip_moe_static_scratch_bytes", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy",
+                 "zc_hip_store_protected_entries"):
         getattr(lib, name).restype = C.c_uint64
+    lib.zc_hip_store_policy.restype = C.c_char_p
+    lib.zc_hip_store_policy.argtypes = [C.c_void_p]
+    lib.zc_hip_store_protected_entries.argtypes = [C.c_void_p]
     lib.zc_hip_stream.restype = C.c_void_p
     lib.zc_hip_store_backing.restype = C.c_void_p
     for name in ("zc_hip_store_backing", "zc_hip_store_stride", "zc_hip_store_capacity", "zc_hip_store_occupancy"):
@@ -82,12 +86,12 @@ class Store:
 
     ACQUISITIONS = ("new_miss", "ready_hit", "loading_join")
 
-    def __init__(self, ctx, layers, experts, record_bytes, slots):
+    def __init__(self, ctx, layers, experts, record_bytes, slots, policy="clock"):
         self.lib = load_library()
         self.ctx, self.layers, self.experts, self.record_bytes = ctx, layers, experts, record_bytes
         self.handle = C.c_void_p()
-        self._check(self.lib.zc_hip_store_create(ctx.handle if ctx else None, C.c_uint32(layers), C.c_uint32(experts),
-                                                 C.c_uint64(record_bytes), C.c_uint64(slots), C.byref(self.handle)))
+        self._check(self.lib.zc_hip_store_create_with_policy(ctx.handle if ctx else None, C.c_uint32(layers), C.c_uint32(experts),
+                                                             C.c_uint64(record_bytes), C.c_uint64(slots), policy.encode(), C.byref(self.handle)))
 
     def _check(self, status):
         if status:
@@ -137,6 +141,14 @@ class Store:
     @property
     def capacity(self):
         return self.lib.zc_hip_store_capacity(self.handle)
+
+    @property
+    def policy(self):
+        return self.lib.zc_hip_store_policy(self.handle).decode()
+
+    @property
+    def protected_entries(self):
+        return self.lib.zc_hip_store_protected_entries(self.handle)
 
     @property
     def occupancy(self):

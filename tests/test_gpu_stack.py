@@ -65,7 +65,7 @@ def _check_stack(ctx, cfg, L, tokens, seed, skew, persistent, mutate=None):
         x_dev = workload.hidden_rows(ctx, T, cfg.hidden, seed * 131 + T)
         x = x_dev.numpy(f32)
         want = oracle_stack(cfg, hosts, x, T)
-        assert ctx.stack_is_persistent(stack, T) == persistent   # above eight tokens: launches of eight and the rest
+        assert ctx.stack_is_persistent(stack, T) == (persistent(T) if callable(persistent) else persistent)   # above eight tokens: launches of eight and the rest
         for layered in (True, False):
             got = run_stack(ctx, cfg, stack, x_dev, T, L, layered)
             name = "layered" if layered else "persistent"
@@ -92,6 +92,16 @@ def test_few_experts_stack(ctx):  # the single-layer shape (hidden 2048 / interm
 
 def test_single_layer_shape_stack(ctx):
     check_stack(ctx, workload.tiny_config(hidden=2048, experts=128, topk=10, inter=512), 3, [1, 8, 20])
+
+
+def test_mixed_artifact_stack(ctx):
+    # Affine Q8 down projection and shared expert (BASELINE config 4's artifact): one token runs the single-launch kernel
+    # with those projections on literal lanes; several tokens take the layer-by-layer path.  Both against the oracle.
+    one_token = lambda T: T == 1
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512, bits=(4, 8, 8, 8)), 3, [1, 3], persistent=one_token)
+    check_stack(ctx, workload.tiny_config(hidden=2048, experts=128, topk=10, inter=512, bits=(4, 8, 8, 8)), 2, [1], seed=37, persistent=one_token)
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 8, 4, 8)), 2, [1], seed=41, persistent=one_token)
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 4, 8, 4)), 2, [1], seed=43, persistent=one_token)
 
 
 def test_small_hidden_stack(ctx):

@@ -817,8 +817,12 @@ struct zc_hip_stack {
 };
 
 namespace {
+bool all_q4(const zc_moe_config& c) { return c.bits_down == 4 && c.shared_bits_gate_up == 4 && c.shared_bits_down == 4; }
+// Routed gate/up is affine Q4 (the exact-integer tiles); the down projection and the shared expert may be affine Q8, which
+// the one-token kernel runs on literal lanes (the kernel for several tokens takes Q4 only).
 bool persistent_shape(const zc_moe_config& c) {
-    return c.bits_gate_up == 4 && c.bits_down == 4 && c.shared_bits_gate_up == 4 && c.shared_bits_down == 4 && c.group == 64 &&
+    return c.bits_gate_up == 4 && (c.bits_down == 4 || c.bits_down == 8) && (c.shared_bits_gate_up == 4 || c.shared_bits_gate_up == 8) &&
+           (c.shared_bits_down == 4 || c.shared_bits_down == 8) && c.group == 64 &&
            c.hidden % 512 == 0 && c.inter % 512 == 0 && c.hidden <= 3072 && c.inter <= 1024 && c.experts <= 1024 && c.topk <= 64;
 }
 uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : 8; }   // kernel variant; LDS is sized by the real token count
@@ -929,6 +933,7 @@ zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* st) {
 static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, zc::DecodeLdsPlan* plan, zc::MultiLdsPlan* multi, uint32_t* nt) {
     if (!st->persistent_ok || tokens > 8 || tokens > st->max_tokens) return false;
     const zc_moe_config& c = st->cfg;
+    if (tokens > 1 && !all_q4(c)) return false;
     *nt = token_tile(tokens);
     if (tokens * c.topk > 256) return false;
     int per_cu = 0;
@@ -952,6 +957,7 @@ static zc_status launch_piece(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
     {
         zc::DecodeParams p{};
         p.H = H; p.E = c.experts; p.topk = k; p.I = c.inter; p.T = tokens; p.L = L;
+        p.bits_down = c.bits_down; p.shared_bits_gate_up = c.shared_bits_gate_up; p.shared_bits_down = c.shared_bits_down;
         for (int shared = 0; shared < 2; ++shared)
             for (int pr = 0; pr < 3; ++pr) {
                 zc_linear l; zc_hip_expert_linear(&c, shared, reinterpret_cast<const void*>(uintptr_t(4096)), pr, &l);

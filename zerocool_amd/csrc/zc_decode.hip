@@ -31,7 +31,10 @@ constexpr int kRing = 8;         // sixteen-byte pieces of a router partition in
 #define ZC_RUN_TILE(SPANS, ...) do { if (NT != 1 && (SPANS) % 8 == 0) xint_run_tile<PT, 8>(__VA_ARGS__); else xint_run_tile<PT, 4>(__VA_ARGS__); } while (0)
 
 // NT = 1: single-token decode.  NT = 8: up to eight tokens, tiles take four at a time.
-template <int NT>
+// MIXED: the down projection and/or the shared expert are affine Q8 and run on literal lanes; that variant leaves out the
+// wave-local down phase (whose tile engine is the largest single piece of the kernel), so that both variants fit the
+// register file without scratch memory and the all-Q4 variant is exactly what it was.
+template <int NT, bool MIXED>
 __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
     constexpr int PT = NT < 4 ? NT : 4;   // tokens per tile pass
     constexpr uint32_t kDecodeThreads = decode_threads(NT), kDecodeWaves = kDecodeThreads / 64;
@@ -551,6 +554,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             // runs once the ids are final: the tiles of the slots whose expert was not predicted.  Both passes compute a slot
             // with the same arithmetic, so a guess can only cost time, never change a bit.
             const uint32_t tiles = I / 8;
+            const bool q8_shared = MIXED && p.shared_bits_gate_up == 8;
+            const uint32_t shared_cut = q8_shared ? 4u : 1u;   // pieces a shared gate/up tile is cut into in the first pass
             for (int pass = 0; pass < 2; ++pass) {
                 uint32_t first, stride, units;
                 bool far_end = false;
@@ -558,8 +563,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     // With whole rounds of routed tiles the shared tiles (one more round, not a full one) go to the workgroups counted
                     // from the far end: the near end owns the router units and comes to the tiles last.
                     if (!pred || wave == 0) continue;
-                    far_end = (k * tiles) % nwg == 0 && tiles <= nwg;
-                    first = wg + nwg * (wave - 1); stride = nwg * (kDecodeWaves - 1); units = far_end ? k * tiles + nwg : (k + 1) * tiles;
+                    far_end = !q8_shared && (k * tiles) % nwg == 0 && tiles <= nwg;
+                    first = wg + nwg * (wave - 1); stride = nwg * (kDecodeWaves - 1);
+                    units = far_end ? k * tiles + nwg : k * tiles + tiles * shared_cut;
                 } else {
                     if (wave != 0) {
                         for (uint32_t i = 0; uint32_t(__hip_atomic_load(misc + 11, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != tag && i < (1u << 22); ++i)
@@ -570,7 +576,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     first = wg + nwg * turn; stride = nwg * kDecodeWaves; units = uint32_t(uniform(spec[2 * (k + 1)])) * tiles;
                 }
                 for (uint32_t u = first; u < units; u += stride) {
-                    uint32_t slot = u / tiles, tile = u % tiles;
+                    uint32_t slot = u / tiles, tile = u % tiles, piece = 0, pieces = shared_cut;
+                    if (pass == 0 && q8_shared && u >= k * tiles) { slot = k; tile = (u - k * tiles) / shared_cut; piece = (u - k * tiles) % shared_cut; pieces = piece + 1; }
                     if (far_end && u >= k * tiles) {
                         const uint32_t s = nwg - 1 - wg;   // the shared tile of this workgroup, if it has one
                         if (s >= tiles) continue;
@@ -579,6 +586,25 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     if (pass == 1) slot = uint32_t(uniform(spec[(k + 1) + slot]));   // the miss list
                     const int32_t e = slot < k ? (pass == 0 ? uniform(pred[slot]) : uniform(ids[slot])) : 0;
                     if (e < 0 || e >= int32_t(E)) continue;   // no guess for the slot, or an id reported above (the combine drops the slot)
+                    uint32_t* out_row = (pass == 0 ? p.tspec : p.tact) + uint64_t(slot) * I;
+                    if (MIXED && slot == k && p.shared_bits_gate_up == 8) {
+                        // the shared expert's gate/up rows as affine Q8: the lower half of the wave takes gate row tile * 8 + i,
+                        // the upper half the up row of the same index
+                        // (a row pair is several memory latencies long, so in the first pass a tile is cut into pieces of two
+                        // row pairs that different waves take; the second pass, which sees the shared expert only when there was
+                        // no guess at all, runs a tile's pieces one after the other)
+                        const uint32_t side = lane >> 5, per_piece = 8 / shared_cut;
+                        const uint8_t* rec = L.shared_record;
+                        for (; piece < pieces; ++piece)
+                            q8_rows<false>(rec + p.so[side * 3], reinterpret_cast<const uint16_t*>(rec + p.so[side * 3 + 1]),
+                                    reinterpret_cast<const uint16_t*>(rec + p.so[side * 3 + 2]), H, xh_all, per_piece,
+                                    [&](uint32_t i) { return tile * 8 + piece * per_piece + i; },
+                                    [&](uint32_t i, float v) {
+                                        const float up = __shfl(v, 32);
+                                        if (lane == 0) ZC_ST(out_row + tile * 8 + piece * per_piece + i, (__float_as_uint(swiglu_bf(v, up)) & 0xffff0000u) | tag);
+                                    });
+                        continue;
+                    }
                     const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                     const uint8_t* rec = slot < k ? record_of(L, e) : L.shared_record;
                     const uint64_t* off = slot < k ? p.ro : p.so;
@@ -586,7 +612,6 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
                     const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 2]) + uint64_t(row) * (H / 64);
                     const uint8_t* img[PT] = {lds + lp.img_rg}; LdsBf16 src[PT] = {LdsBf16{xh_all}};
-                    uint32_t* out_row = (pass == 0 ? p.tspec : p.tact) + uint64_t(slot) * I;
                     // SwiGLU of the finished tile as tagged words, one per activation: row `slot` of the tagged buffer (row k: shared)
                     auto emit = [&](int, float v) {
                         const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
@@ -636,7 +661,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         if constexpr (NT == 1) { if (wg >= H / 16) bar.arrive(); }
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
             const uint32_t row = rt * 16 + col;
-            if (NT == 1 && SB >= slots_total && I == 1024) {
+            if (!MIXED && NT == 1 && SB >= slots_total && I == 1024) {
                 // One token, all slots' images resident, tiles of two bodies (intermediate 1024): every wave works alone.  It requests the first weights of its slot's
                 // tile, then polls that slot's activations (one 16-element block per lane), builds the slot's image and the
                 // BF16 copy under the latency of those loads, and runs the tile; no workgroup barrier until the combine, and
@@ -785,6 +810,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                             if (e < 0 || e >= int32_t(E)) continue;
                             rec = record_of(L, e); off = p.ro;
                         }
+                        if (MIXED && (slot < k ? p.bits_down : p.shared_bits_down) == 8) {   // affine Q8 down rows: row 2 i of the tile on the lower half of the wave, 2 i + 1 on the upper
+                            q8_rows<true>(rec + off[6], reinterpret_cast<const uint16_t*>(rec + off[7]), reinterpret_cast<const uint16_t*>(rec + off[8]), I,
+                                    ah + (slot - s0) * I, 8, [&](uint32_t i) { return rt * 16 + 2 * i + (lane >> 5); },
+                                    [&](uint32_t i, float v) { if ((lane & 31u) == 0) otile[slot * 16 + 2 * i + (lane >> 5)] = bf(v); });
+                            continue;
+                        }
                         const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
                         const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
                         const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
@@ -823,7 +854,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
             __syncthreads();
-            if (NT == 1 && SB >= slots_total && I == 1024 && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
+            if (!MIXED && NT == 1 && SB >= slots_total && I == 1024 && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
             clock();
             // weighted combine of the tile (reference: qwen.metal:804-816)
             if (tid < T * 16) {
@@ -831,7 +862,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 float partial[8];
 #pragma unroll
                 for (int q = 0; q < 8; ++q) partial[q] = 0;
-                const bool products = NT == 1 && SB >= slots_total && I == 1024;   // the waves left products, not outputs
+                const bool products = !MIXED && NT == 1 && SB >= slots_total && I == 1024;   // the waves left products, not outputs
                 if (products) {
                     for (uint32_t base = 0; base < k; base += 8) {
                         float value[8];
@@ -908,23 +939,31 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
 }
 
 hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp) {
-#define ZC_DECODE(NT)                                                                                              \
-    do {                                                                                                           \
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<NT>),                  \
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));             \
-        if (e != hipSuccess) return e;                                                                             \
-        hipLaunchKernelGGL((decode_stack_kernel<NT>), dim3(workgroups), dim3(decode_threads(NT)), lp.total, s, p, lp);  \
+#define ZC_DECODE(MIXED)                                                                                               \
+    do {                                                                                                               \
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1, MIXED>),                \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));                 \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL((decode_stack_kernel<1, MIXED>), dim3(workgroups), dim3(decode_threads(1)), lp.total, s, p, lp);  \
     } while (0)
     (void)nt;   // two to eight tokens run decode_multi_kernel (zc_decode_multi.hip)
-    ZC_DECODE(1);
+    if (p.bits_down == 4 && p.shared_bits_gate_up == 4 && p.shared_bits_down == 4) ZC_DECODE(false); else ZC_DECODE(true);
 #undef ZC_DECODE
     return hipGetLastError();
 }
 hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu) {
     (void)nt;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    // both variants have the same launch bounds and dynamic LDS; the mixed one uses no more registers than the other
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1, false>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_stack_kernel<1>, decode_threads(1), lds_bytes);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1, true>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (e != hipSuccess) return e;
+    int plain = 0, mixed = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, decode_stack_kernel<1, false>, decode_threads(1), lds_bytes);
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&mixed, decode_stack_kernel<1, true>, decode_threads(1), lds_bytes);
+    *blocks_per_cu = plain < mixed ? plain : mixed;
+    return e;
 }
 
 }  // namespace zc

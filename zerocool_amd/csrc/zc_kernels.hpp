@@ -62,6 +62,7 @@ struct DecodeLayer {
 };
 struct DecodeParams {
     uint32_t H, E, topk, I, T, L;
+    uint32_t bits_down, shared_bits_gate_up, shared_bits_down;   // 4 or 8 (routed gate/up is always 4 in these kernels); 8: literal lanes, one token only
     uint64_t ro[9], so[9];           // byte offsets [projection*3 + {codes, scales, biases}] in a routed / shared record
     const DecodeLayer* layers;       // device array [L]
     const float* x_in; float* out;   // [T][H]

@@ -200,9 +200,11 @@ zc_status zc_hip_moe_check(zc_hip_ctx* ctx);
  * between the reference's MoE layers (attention / GDN / hyper-connections) is outside
  * this path; the stack stands in for it with a glue that keeps activations bounded and
  * BF16-valued: x_next = bf(y * (1 / max|y|)) per token (zc_hip_stack_glue).
- * Up to 8 tokens run as ONE persistent kernel launch for the whole stack (routing,
- * dispatch and combine stay on the device, no host synchronisation between layers);
- * larger batches run layer by layer through zc_hip_moe_forward.  Both give identical bytes.
+ * Up to 64 tokens run as ONE persistent kernel launch for the whole stack (routing,
+ * dispatch and combine stay on the device, no host synchronisation between layers; one
+ * kernel each for one token, two to eight, and nine to sixty-four), larger batches as
+ * one such launch per 64 tokens; shapes those kernels do not take run layer by layer
+ * through zc_hip_moe_forward.  All give identical bytes.
  * out: [tokens][hidden], the last layer's output.  flags bit 0: force the layer-by-layer path. */
 typedef struct zc_hip_stack zc_hip_stack;
 typedef struct {       /* optional device buffers, any may be NULL */

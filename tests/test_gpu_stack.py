@@ -104,6 +104,14 @@ def test_mixed_artifact_stack(ctx):
     check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 4, 8, 4)), 2, [1], seed=43, persistent=one_token)
 
 
+def test_nine_to_sixty_four_tokens_in_one_launch(ctx):
+    # The kernel for nine to sixty-four tokens: entries of up to eight tokens per expert (a skewed router sends dozens of
+    # tokens to one expert, so its tokens fill several entries), a full launch of 64, and 64 + 6 as two launches.
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512), 2, [9, 64, 70], seed=47)
+    check_stack(ctx, workload.tiny_config(hidden=2048, experts=512, topk=10, inter=512), 1, [33], seed=53)
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=16, topk=4, inter=1024), 2, [40], seed=59, skew=None)
+
+
 def test_small_hidden_stack(ctx):
     check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512), 2, [1, 4, 17, 32])
 

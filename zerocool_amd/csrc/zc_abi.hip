@@ -801,6 +801,7 @@ struct zc_hip_stack {
     float *logits = nullptr, *gate = nullptr, *shared_act = nullptr, *act = nullptr, *layer_out = nullptr, *eout = nullptr;
     uint32_t* maxabs = nullptr; uint32_t* sync = nullptr;
     unsigned long long* tlogits = nullptr; uint32_t *tact = nullptr, *tout = nullptr;   // tagged exchange buffers of the one-token kernel
+    int32_t* wide_ids = nullptr; float* wide_weights = nullptr;   // routes of the nine-to-sixty-four-token kernel
     uint32_t* tspec = nullptr; int32_t* pred[2] = {nullptr, nullptr};   // prediction pass: its activations, the previous / this step's ids per layer
     uint32_t pred_turn = 0; bool pred_valid = false, speculate = true;
     uint32_t epoch = 1u << 12;
@@ -825,7 +826,6 @@ bool persistent_shape(const zc_moe_config& c) {
            (c.shared_bits_down == 4 || c.shared_bits_down == 8) && c.group == 64 &&
            c.hidden % 512 == 0 && c.inter % 512 == 0 && c.hidden <= 3072 && c.inter <= 1024 && c.experts <= 1024 && c.topk <= 64;
 }
-uint32_t token_tile(uint32_t tokens) { return tokens <= 1 ? 1 : 8; }   // kernel variant; LDS is sized by the real token count
 }  // namespace
 
 extern "C" {
@@ -868,14 +868,15 @@ static zc_status create_stack(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
     // persistent path arena
     st->persistent_ok = persistent_shape(*c) && n_layers <= 16384;   // the 16-bit exchange tags tell at most 65535 layers apart
     if (st->persistent_ok) {
-        const uint32_t Tp = T < 8 ? T : 8;
+        const uint32_t Tp = T < 64 ? T : 64;   // tokens of the largest single launch
         uint64_t at = 0;
         auto take = [&](uint64_t bytes) { const uint64_t o = at; at += align_up(bytes, 256); return o; };
         const uint64_t o_layers = take(sizeof(zc::DecodeLayer) * n_layers), o_logits = take(uint64_t(Tp) * E * 4), o_gate = take(Tp * 4),
                        o_sact = take(uint64_t(Tp) * I * 4), o_act = take(uint64_t(Tp) * k * I * 4), o_lout = take(uint64_t(Tp) * H * 4),
                        o_max = take(std::max<uint64_t>(uint64_t(n_layers) * Tp * 4, uint64_t(Tp) * (H / 64 + 1) * 4)), o_sync = take(zc::kDecodeSyncBytes), o_eout = take(uint64_t(Tp) * (k + 1) * H * 4),
                        o_tlogits = take(uint64_t(E + 1) * 8), o_tact = take(uint64_t(k + 1) * I * 4), o_tout = take(uint64_t(2) * H * 4),
-                       o_tspec = take(uint64_t(k + 1) * I * 4), o_pred0 = take(uint64_t(n_layers) * k * 4), o_pred1 = take(uint64_t(n_layers) * k * 4);
+                       o_tspec = take(uint64_t(k + 1) * I * 4), o_pred0 = take(uint64_t(n_layers) * k * 4), o_pred1 = take(uint64_t(n_layers) * k * 4),
+                       o_wids = take(uint64_t(Tp) * k * 4), o_wweights = take(uint64_t(Tp) * k * 4);
         if (zc_hip_alloc(ctx, at, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
         st->arena = static_cast<uint8_t*>(p); st->arena_bytes = at;
         st->dev_layers = reinterpret_cast<zc::DecodeLayer*>(st->arena + o_layers);
@@ -887,6 +888,7 @@ static zc_status create_stack(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         st->tout = reinterpret_cast<uint32_t*>(st->arena + o_tout);
         st->tspec = reinterpret_cast<uint32_t*>(st->arena + o_tspec);
         st->pred[0] = reinterpret_cast<int32_t*>(st->arena + o_pred0); st->pred[1] = reinterpret_cast<int32_t*>(st->arena + o_pred1);
+        st->wide_ids = reinterpret_cast<int32_t*>(st->arena + o_wids); st->wide_weights = reinterpret_cast<float*>(st->arena + o_wweights);
         std::vector<zc::DecodeLayer> host(n_layers);
         for (uint32_t l = 0; l < n_layers; ++l) {
             const zc_moe_layer& y = host_layers[l];
@@ -930,28 +932,51 @@ zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* st) {
     delete st;
     return ZC_OK;
 }
-static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, zc::DecodeLdsPlan* plan, zc::MultiLdsPlan* multi, uint32_t* nt) {
-    if (!st->persistent_ok || tokens > 8 || tokens > st->max_tokens) return false;
+// Which single-launch kernel takes `tokens` rows in one launch, and its LDS plan: nt = 1 (one token), 8 (two to eight) or 64
+// (nine to sixty-four); false if none does.
+struct LaunchPlan { zc::DecodeLdsPlan one; zc::MultiLdsPlan multi; zc::WideLdsPlan wide; uint32_t nt = 0; };
+static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, LaunchPlan* plan) {
+    if (!st->persistent_ok || !tokens || tokens > 64 || tokens > st->max_tokens) return false;
     const zc_moe_config& c = st->cfg;
     if (tokens > 1 && !all_q4(c)) return false;
-    *nt = token_tile(tokens);
-    if (tokens * c.topk > 256) return false;
     int per_cu = 0;
     (void)ctx;
-    if (*nt == 1) {
-        *plan = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
-        if (plan->total > st->lds_limit || plan->slots_per_batch == 0) return false;
-        if (zc::decode_stack_occupancy(*nt, plan->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+    if (tokens == 1) {
+        plan->nt = 1;
+        plan->one = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
+        if (plan->one.total > st->lds_limit || plan->one.slots_per_batch == 0) return false;
+        if (zc::decode_stack_occupancy(1, plan->one.total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+    } else if (tokens <= 8) {
+        plan->nt = 8;
+        if (tokens * c.topk > 256) return false;
+        plan->multi = zc::decode_multi_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
+        if (plan->multi.total > st->lds_limit) return false;
+        if (zc::decode_multi_occupancy(plan->multi.total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
     } else {
-        *multi = zc::decode_multi_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
-        if (multi->total > st->lds_limit) return false;
-        if (zc::decode_multi_occupancy(multi->total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
+        plan->nt = 64;
+        plan->wide = zc::decode_wide_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
+        if (plan->wide.total > st->lds_limit) return false;
+        if (zc::decode_wide_occupancy(plan->wide.total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
     }
     return per_cu >= 1;
 }
+// How a batch is cut into launches: up to eight tokens are one launch; more go sixty-four at a time through the kernel for
+// nine to sixty-four tokens where its plan fits, eight at a time otherwise.  0: no single-launch path for this batch.
+static uint32_t launch_unit(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
+    LaunchPlan plan;
+    if (tokens > st->max_tokens) return 0;
+    if (tokens <= 8) return persistent_plan(ctx, st, tokens, &plan) ? 8u : 0u;
+    for (const uint32_t unit : {64u, 8u}) {
+        bool fits = true;
+        for (uint32_t first = 0; first < tokens && fits; first += unit) fits = persistent_plan(ctx, st, std::min(unit, tokens - first), &plan);
+        if (fits) return unit;
+    }
+    return 0;
+}
 // One launch of the persistent kernels: `tokens` (at most eight) rows starting at token `first` of a batch of `batch`.
 static zc_status launch_piece(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out, const zc_stack_trace* trace,
-                              uint32_t first, uint32_t batch, const zc::DecodeLdsPlan& plan, const zc::MultiLdsPlan& multi, uint32_t nt) {
+                              uint32_t first, uint32_t batch, const LaunchPlan& plan) {
+    const uint32_t nt = plan.nt;
     const zc_moe_config& c = st->cfg;
     const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
     {
@@ -969,6 +994,7 @@ static zc_status launch_piece(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.logits = st->logits; p.gate = st->gate; p.shared_act = st->shared_act; p.act = st->act; p.layer_out = st->layer_out;
         p.maxabs = st->maxabs; p.eout = st->eout;
         p.tlogits = st->tlogits; p.tact = st->tact; p.tout = st->tout; p.tspec = st->tspec;
+        p.route_ids = st->wide_ids; p.route_weights = st->wide_weights;
         if (nt == 1 && st->speculate) {   // this step reads the ids the previous one-token step left, and leaves its own
             p.pred_in = st->pred_valid ? st->pred[st->pred_turn] : nullptr; p.pred_out = st->pred[st->pred_turn ^ 1u];
             st->pred_turn ^= 1u; st->pred_valid = true;
@@ -981,15 +1007,16 @@ static zc_status launch_piece(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         if (st->store && !p.ids_trace) { p.ids_trace = st->route_ids + uint64_t(first) * k; p.weights_trace = st->route_weights + uint64_t(first) * k; }
         p.clocks = trace && first == 0 ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
-        st->epoch += 4 * L + 16;   // at most four barriers per layer; wraps modulo 2^32, the barrier compares epochs as signed differences
+        st->epoch += 5 * L + 16;   // at most five barriers per layer; wraps modulo 2^32, the barrier compares epochs as signed differences
         // The tagged buffers are written by one-token launches only, so their tags advance with those launches only:
         // a launch's layer 0 then expects the tag right after the one its predecessor's last layer left, however many
         // launches of the other kernel ran in between.
         p.tag_base = st->tag_base;
         if (nt == 1) st->tag_base = (st->tag_base + L) % 65535u;
         const uint32_t workgroups = uint32_t(st->cus);
-        if (nt == 1) ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan));
-        else ZC_HIP(zc::launch_decode_multi(ctx->stream, p, workgroups, multi));
+        if (nt == 1) ZC_HIP(zc::launch_decode_stack(ctx->stream, p, nt, workgroups, plan.one));
+        else if (nt == 8) ZC_HIP(zc::launch_decode_multi(ctx->stream, p, workgroups, plan.multi));
+        else ZC_HIP(zc::launch_decode_wide(ctx->stream, p, workgroups, plan.wide));
     }
     return ZC_OK;
 }
@@ -1004,12 +1031,9 @@ zc_status zc_hip_stack_set_speculation(zc_hip_ctx* ctx, zc_hip_stack* st, int on
     return ZC_OK;
 }
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
-    if (!ctx || !st) return 0;
-    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt;
-    if (tokens > 8)   // pieces of eight and the rest
-        return tokens <= st->max_tokens && !st->store && persistent_plan(ctx, st, 8, &plan, &multi, &nt) &&
-               (tokens % 8 == 0 || persistent_plan(ctx, st, tokens % 8, &plan, &multi, &nt)) ? 1 : 0;
-    return persistent_plan(ctx, st, tokens, &plan, &multi, &nt) ? 1 : 0;
+    if (!ctx || !st || !tokens) return 0;
+    if (st->store && tokens > 8) return 0;
+    return launch_unit(ctx, st, tokens) ? 1 : 0;
 }
 zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
                               const zc_stack_trace* trace, uint32_t flags) {
@@ -1018,21 +1042,20 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
     ZC_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && x != out, "invalid or overlapping linear output");
     const zc_moe_config& c = st->cfg;
     const uint32_t L = uint32_t(st->layers.size()), H = c.hidden, k = c.topk;
-    zc::DecodeLdsPlan plan; zc::MultiLdsPlan multi; uint32_t nt = 0;
+    LaunchPlan plan;
+    const uint32_t unit = (flags & 1u) ? 0u : launch_unit(ctx, st, tokens);
     if (st->store) {
-        ZC_REQUIRE(!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt), "a stack behind an expert store runs as one launch only");
+        ZC_REQUIRE(unit && tokens <= 8, "a stack behind an expert store runs as one launch only");
         if (const zc_status s = zc_hip_store_table_refresh(st->store)) return s;
     }
-    // More than eight tokens go through the single-launch kernels in pieces of eight, one launch per piece (tokens do not
-    // interact inside a layer): every piece streams the weights again, but stays on the device from the first layer to the last.
-    const bool pieces = !(flags & 1u) && tokens > 8 && persistent_plan(ctx, st, 8, &plan, &multi, &nt) &&
-                        (tokens % 8 == 0 || persistent_plan(ctx, st, tokens % 8, &plan, &multi, &nt));
-    if (pieces || (!(flags & 1u) && persistent_plan(ctx, st, tokens, &plan, &multi, &nt))) {
+    // More than eight tokens go through the single-launch kernels sixty-four (or eight) at a time, one launch per piece (tokens
+    // do not interact inside a layer); every piece stays on the device from the first layer to the last.
+    if (unit) {
         if (trace && trace->ids) ZC_REQUIRE(trace->weights, "a routing trace needs both ids and weights");
-        for (uint32_t first = 0; first < tokens; first += 8) {
-            const uint32_t piece = std::min(8u, tokens - first);
-            if (!persistent_plan(ctx, st, piece, &plan, &multi, &nt)) return fail(ZC_LOGIC_ERROR, "no single-launch plan for a piece of the batch");
-            if (const zc_status s = launch_piece(ctx, st, x + uint64_t(first) * H, piece, out + uint64_t(first) * H, trace, first, tokens, plan, multi, nt)) return s;
+        for (uint32_t first = 0; first < tokens; first += unit) {
+            const uint32_t piece = std::min(unit, tokens - first);
+            if (!persistent_plan(ctx, st, piece, &plan)) return fail(ZC_LOGIC_ERROR, "no single-launch plan for a piece of the batch");
+            if (const zc_status s = launch_piece(ctx, st, x + uint64_t(first) * H, piece, out + uint64_t(first) * H, trace, first, tokens, plan)) return s;
         }
         if (st->store) {
             // The launch has read every record through the store's table.  Once it has finished, the store learns which

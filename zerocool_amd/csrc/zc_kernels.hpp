@@ -77,6 +77,7 @@ struct DecodeParams {
     // before this step's ids are known), pred_out [L][topk] receives this step's; tspec [topk + 1][I]: the prediction pass's
     // activations, tagged like tact.
     const int32_t* pred_in; int32_t* pred_out; uint32_t* tspec;
+    int32_t* route_ids; float* route_weights;   // nine to sixty-four tokens: [T][topk] routes, written by the routing waves, read by every workgroup
     int32_t* ids_trace; float* weights_trace; float* out_trace;   // optional [L][trace_tokens][topk], [L][trace_tokens][topk], [L][trace_tokens][H],
     uint32_t trace_tokens;           // each already advanced to this launch's first token: a launch may be one piece of a larger batch
     uint32_t* sync; uint32_t epoch; int32_t* status; uint32_t spin_limit;
@@ -100,6 +101,15 @@ struct MultiLdsPlan {
 MultiLdsPlan decode_multi_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t T, uint32_t lds_limit);
 hipError_t launch_decode_multi(hipStream_t s, const DecodeParams& p, uint32_t workgroups, const MultiLdsPlan& lp);
 hipError_t decode_multi_occupancy(uint32_t lds_bytes, int* blocks_per_cu);
+
+// Nine to sixty-four tokens (zc_decode_wide.hip)
+struct WideLdsPlan {
+    uint32_t ids, weights, gatev, gscale, chosen, entries, cum, misc, gatew, region, total;
+    uint32_t img_x, xh, img_d, ah;
+};
+WideLdsPlan decode_wide_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t T, uint32_t lds_limit);
+hipError_t launch_decode_wide(hipStream_t s, const DecodeParams& p, uint32_t workgroups, const WideLdsPlan& lp);
+hipError_t decode_wide_occupancy(uint32_t lds_bytes, int* blocks_per_cu);
 
 // ---- prefill: sorted-token grouped GEMM on the bf16 matrix cores (zc_prefill.hip)
 struct PrefillGemm {

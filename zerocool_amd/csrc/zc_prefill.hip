@@ -137,14 +137,19 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     const uint32_t x_row = p.a_rows ? uint32_t(p.a_rows[x_pos]) / p.a_div : x_pos;
     const float* x_src = p.asum + uint64_t(x_row) * groups;
 
-    uint4 a_next, b_next; uint16_t s_next = 0, o_next = 0; float x_next = 0;
-    auto fetch = [&](uint32_t g) {
-        a_next = *reinterpret_cast<const uint4*>(a_src + g * 64);
-        b_next = ldg_u4(b_src + g * 32);
-        if (tid < 128) { s_next = ldg_u16(s_src, g); o_next = ldg_u16(o_src, g); }
-        else if (tid < 160) x_next = x_src[g];
+    // What a step needs is requested two steps ahead and waits in registers (two sets, taken in turn): with one step of
+    // lead the loads' latency, several times a step's arithmetic, was paid at every step.
+    struct Fetched { uint4 a, b; uint16_t s, o; float x; };
+    Fetched ahead[2];
+    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), 0, 0, 0.0f};
+    auto fetch = [&](uint32_t g, Fetched& f) {
+        f.a = *reinterpret_cast<const uint4*>(a_src + g * 64);
+        f.b = ldg_u4(b_src + g * 32);
+        if (tid < 128) { f.s = ldg_u16(s_src, g); f.o = ldg_u16(o_src, g); }
+        else if (tid < 160) f.x = x_src[g];
     };
-    auto stash = [&](uint32_t buf) {
+    auto stash = [&](uint32_t buf, const Fetched& f) {
+        const uint4 a_next = f.a, b_next = f.b; const uint16_t s_next = f.s, o_next = f.o; const float x_next = f.x;
         *reinterpret_cast<uint4*>(&a_s[buf][a_r * kPitch + a_c * 8]) = a_next;
         // 32 codes -> 32 bf16: nibble i of a word is element 8w+i
         const uint32_t words[4] = {b_next.x, b_next.y, b_next.z, b_next.w};
@@ -177,12 +182,15 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) total[q] = mag[q] = f32x4{0, 0, 0, 0};
 
-    fetch(0);
-    stash(0);
+    fetch(0, ahead[0]);
+    if (groups > 1) fetch(1, ahead[1]);
+    stash(0, ahead[0]);
     __syncthreads();
-    for (uint32_t g = 0; g < groups; ++g) {
+    // two steps per trip, so that the register sets are named at compile time: step g computes from LDS buffer g & 1, requests
+    // step g + 2 into the set that step g's data has just left, and stashes step g + 1 from the other set
+    auto step = [&](uint32_t g, Fetched& mine, Fetched& next) {
         const uint32_t buf = g & 1u;
-        if (g + 1 < groups) fetch(g + 1);
+        if (g + 2 < groups) fetch(g + 2, mine);
         f32x4 dot[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) dot[q] = f32x4{0, 0, 0, 0};
@@ -207,8 +215,12 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
                 mag[q][r] = __builtin_fmaf(fabsf(scale), fabsf(dot[q][r]), __builtin_fmaf(fabsf(bias), fabsf(sums[r]), mag[q][r]));
             }
         }
-        if (g + 1 < groups) stash(buf ^ 1u);
+        if (g + 1 < groups) stash(buf ^ 1u, next);
         __syncthreads();
+    };
+    for (uint32_t g = 0; g < groups; g += 2) {
+        step(g, ahead[0], ahead[1]);
+        if (g + 1 < groups) step(g + 1, ahead[1], ahead[0]);
     }
     // epilogue: row m of the tile is sorted position first + m.  A sum close to a BF16 rounding boundary could round
     // the other way under the reference's order of additions: such elements are listed for exact recomputation.

@@ -25,13 +25,19 @@
 namespace zc {
 
 constexpr int kWideBatch = 8;                // tokens whose rows and images a workgroup holds at a time
-constexpr int kWidePass = 2;                 // tokens one tile pass holds
-constexpr uint32_t kWideThreads = 512, kWideWaves = kWideThreads / 64;
+// Tokens one tile pass holds, chosen at build time: 2 with 512 threads (two waves per SIMD cover each other's latencies), or
+// up to 8 with 256 threads (one wave per SIMD with the whole register file; a tile's codes are expanded once for the entry).
+#ifndef ZC_WIDE_PASS_TOKENS
+#define ZC_WIDE_PASS_TOKENS 2
+#endif
+constexpr int kWidePass = ZC_WIDE_PASS_TOKENS;
+constexpr uint32_t kWideThreads = kWidePass <= 2 ? 512 : 256, kWideWaves = kWideThreads / 64;
 
 template <class Emit>
 __device__ __forceinline__ void run_tile_wide(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans, const uint8_t* const* img,
                                               const LdsBf16* src, const XintLayout L, uint32_t lane, int nt, Emit emit) {
-    if (nt <= 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    if constexpr (kWidePass == 8) xint_run_tile_upto8(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    else if (nt <= 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     else xint_run_tile_tokens_piped<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
 }
 

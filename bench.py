@@ -171,7 +171,7 @@ def main():
     L, T = args.layers, args.batch
     layers = [workload.LayerWeights(ctx, cfg, workload.BASE_SEED + 4 * 1000 + l, ("zipf", 1.1)) for l in range(L)]
     ctx.finish()
-    stack = ctx.stack_create(cfg, [l.layer for l in layers], max(T, 8))
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], max(T, 64 if args.extra else 8))
 
     def run(stack, cfg, n_layers, tokens, steps, warmup, speculate=True, inputs=INPUTS, seed=workload.BASE_SEED + 4 * 7):
         """Times `steps` launches that cycle through `inputs` distinct token batches (a decode loop never sees the same
@@ -277,6 +277,10 @@ def main():
         extra["stack_batch8"] = {"tokens_per_s": 8 / (r8["ms"] * 1e-3), "ms_per_step": r8["ms"], "GBps": r8["bytes"] / (r8["ms"] * 1e-3) / 1e9,
                                  "frac_of_hbm_peak": r8["bytes"] / (r8["ms"] * 1e-3) / 8e12, "distinct_experts_per_layer": r8["unique"],
                                  "kernel": "zc::decode_multi_kernel"}
+        for tokens in (32, 64):   # one launch of the kernel for nine to sixty-four tokens
+            rw = run(stack, cfg, L, tokens, max(4, quick // 4), 1, inputs=2)
+            extra[f"stack_batch{tokens}"] = {"tokens_per_s": tokens / (rw["ms"] * 1e-3), "ms_per_step": rw["ms"], "GBps": rw["bytes"] / (rw["ms"] * 1e-3) / 1e9,
+                                             "distinct_experts_per_layer": rw["unique"], "kernel": "zc::decode_wide_kernel"}
         # The same records behind routers with a milder popularity skew (Zipf exponent 0.5: the offsets span 3.1 instead
         # of 6.9) and with none at all, so that consecutive tokens share fewer experts and a batch of eight touches
         # several times more records.

@@ -223,14 +223,14 @@ def test_a_wait_that_runs_out_is_reported_and_the_stack_stays_usable(ctx):
     # default bound back, the same stack gives the right answer again.
     cfg = workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512)
     layers = [workload.LayerWeights(ctx, cfg, 501 + l, ("zipf", 1.1)) for l in range(4)]
-    stack = ctx.stack_create(cfg, [l.layer for l in layers], 2)
-    out = {T: ctx.alloc(T * cfg.hidden * 4) for T in (1, 2)}
-    xs = {T: workload.hidden_rows(ctx, T, cfg.hidden, 30 + T) for T in (1, 2)}
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], 12)
+    out = {T: ctx.alloc(T * cfg.hidden * 4) for T in (1, 2, 12)}
+    xs = {T: workload.hidden_rows(ctx, T, cfg.hidden, 30 + T) for T in (1, 2, 12)}
     want = {}
-    for T in (1, 2):
+    for T in (1, 2, 12):
         ctx.stack_decode(stack, xs[T], T, out[T]); ctx.moe_check()
         want[T] = out[T].numpy(f32).tobytes()
-    for T in (1, 2):
+    for T in (1, 2, 12):
         ctx.stack_set_wait_limit(stack, 1)
         reported = 0
         for _ in range(5):
@@ -248,7 +248,7 @@ def test_a_wait_that_runs_out_is_reported_and_the_stack_stays_usable(ctx):
     for l in layers:
         for b in (l.router, l.shared_gate, l.shared_record, l.records):
             ctx.free(b)
-    for T in (1, 2):
+    for T in (1, 2, 12):
         ctx.free(out[T]); ctx.free(xs[T])
 
 

@@ -349,8 +349,8 @@ def main():
         # the one-token kernel misses, which prices the guessing at its worst
         extra["single_layer_q4_one_launch_all_guesses_miss"] = [one_launch_layer(ctx, "S", 1, 200, skew=None, speculate=on) for on in (True, False)]
         extra["single_layer_q4"] = [single_layer(ctx, "S", t, False, 50) for t in (1, 8, 32, 64)]
-        extra["single_layer_mixed_one_launch"] = [one_launch_layer(ctx, "S-mixed", 1, 200)]
-        extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8)]
+        extra["single_layer_mixed_one_launch"] = [one_launch_layer(ctx, "S-mixed", t, 100) for t in (1, 8, 16)]
+        extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8, 16)]
         extra["prefill_q4"] = [single_layer(ctx, "S", t, True, 20) for t in (32, 64, 256, 2048)]
         result["extra"] = extra
 

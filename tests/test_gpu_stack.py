@@ -95,13 +95,12 @@ def test_single_layer_shape_stack(ctx):
 
 
 def test_mixed_artifact_stack(ctx):
-    # Affine Q8 down projection and shared expert (BASELINE config 4's artifact): one token runs the single-launch kernel
-    # with those projections on literal lanes; several tokens take the layer-by-layer path.  Both against the oracle.
-    one_token = lambda T: T == 1
-    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512, bits=(4, 8, 8, 8)), 3, [1, 3], persistent=one_token)
-    check_stack(ctx, workload.tiny_config(hidden=2048, experts=128, topk=10, inter=512, bits=(4, 8, 8, 8)), 2, [1], seed=37, persistent=one_token)
-    check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 8, 4, 8)), 2, [1], seed=41, persistent=one_token)
-    check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 4, 8, 4)), 2, [1], seed=43, persistent=one_token)
+    # Affine Q8 down projection and shared expert (BASELINE config 4's artifact): one token runs the one-token kernel with
+    # those projections on literal lanes, more tokens the kernel for nine to sixty-four tokens.  All against the oracle.
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=64, topk=10, inter=512, bits=(4, 8, 8, 8)), 3, [1, 3, 16, 21])
+    check_stack(ctx, workload.tiny_config(hidden=2048, experts=128, topk=10, inter=512, bits=(4, 8, 8, 8)), 2, [1, 16], seed=37)
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 8, 4, 8)), 2, [1, 5], seed=41)
+    check_stack(ctx, workload.tiny_config(hidden=1024, experts=32, topk=4, inter=1024, bits=(4, 4, 8, 4)), 2, [1, 9], seed=43)
 
 
 def test_nine_to_sixty_four_tokens_in_one_launch(ctx):

@@ -820,7 +820,8 @@ struct zc_hip_stack {
 namespace {
 bool all_q4(const zc_moe_config& c) { return c.bits_down == 4 && c.shared_bits_gate_up == 4 && c.shared_bits_down == 4; }
 // Routed gate/up is affine Q4 (the exact-integer tiles); the down projection and the shared expert may be affine Q8, which
-// the one-token kernel runs on literal lanes (the kernel for several tokens takes Q4 only).
+// the one-token kernel and the kernel for nine to sixty-four tokens run on literal lanes (two to eight tokens of such an
+// artifact go through the latter as well; the kernel for two to eight tokens takes Q4 only).
 bool persistent_shape(const zc_moe_config& c) {
     return c.bits_gate_up == 4 && (c.bits_down == 4 || c.bits_down == 8) && (c.shared_bits_gate_up == 4 || c.shared_bits_gate_up == 8) &&
            (c.shared_bits_down == 4 || c.shared_bits_down == 8) && c.group == 64 &&
@@ -938,7 +939,6 @@ struct LaunchPlan { zc::DecodeLdsPlan one; zc::MultiLdsPlan multi; zc::WideLdsPl
 static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, LaunchPlan* plan) {
     if (!st->persistent_ok || !tokens || tokens > 64 || tokens > st->max_tokens) return false;
     const zc_moe_config& c = st->cfg;
-    if (tokens > 1 && !all_q4(c)) return false;
     int per_cu = 0;
     (void)ctx;
     if (tokens == 1) {
@@ -946,7 +946,7 @@ static bool persistent_plan(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens, 
         plan->one = zc::decode_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);
         if (plan->one.total > st->lds_limit || plan->one.slots_per_batch == 0) return false;
         if (zc::decode_stack_occupancy(1, plan->one.total, &per_cu) != hipSuccess) { (void)hipGetLastError(); return false; }
-    } else if (tokens <= 8) {
+    } else if (tokens <= 8 && all_q4(c)) {
         plan->nt = 8;
         if (tokens * c.topk > 256) return false;
         plan->multi = zc::decode_multi_lds_plan(c.hidden, c.experts, c.topk, c.inter, tokens, st->lds_limit);

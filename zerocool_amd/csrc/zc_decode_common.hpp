@@ -28,20 +28,23 @@ __device__ __forceinline__ void st_i32(int32_t* p, int32_t v) { ZC_ST(reinterpre
 constexpr uint32_t decode_threads(int nt) { return nt == 1 ? 512u : 256u; }
 constexpr uint32_t kFlagStride = 32, kReleaseBase = 32 * 1024, kReleaseStride = 64, kAbortWord = kReleaseBase + 8 * kReleaseStride;
 
-// Literal affine Q8 rows (reference: qwen.metal:112-125) against ONE input row held in LDS as BF16.  Each 32-lane half of
-// the wave plays the reference's 32 lanes for one output row at a time: lane l takes the eight-element blocks l, l + 32, ...
-// (K is a multiple of 512 here, so the lane width is eight and a row of codes is K bytes); per block the plain fp32 sum of
-// the inputs and the multiply-add chain of inputs times codes, result += scale * dot + sum * bias, then the xor butterfly.
-// `codes`, `scales`, `biases` are per-lane bases (the two halves may read different matrices); row_of(i) is the half's i-th
-// row, emit(i, value) runs in every lane with that row's value.  Two rows per half are fetched together, CH blocks each.
-template <int CH, int ROWS, class RowOf, class Emit>
+// Literal affine Q8 rows (reference: qwen.metal:112-125) against NTOK input rows held in LDS as BF16 (the tokens of one tile
+// pass: a row's codes are fetched once and serve all of them).  Each 32-lane half of the wave plays the reference's 32 lanes
+// for one output row at a time: lane l takes the eight-element blocks l, l + 32, ... (K is a multiple of 512 here, so the lane
+// width is eight and a row of codes is K bytes); per block the plain fp32 sum of the inputs and the multiply-add chain of
+// inputs times codes, result += scale * dot + sum * bias, then the xor butterfly.  `codes`, `scales`, `biases` are per-lane
+// bases (the two halves may read different matrices); row_of(i) is the half's i-th row, emit(i, t, value) runs in every lane
+// with that row's value for token t.  ROWS rows per half are fetched together, CH blocks each.
+template <int CH, int ROWS, int NTOK, class RowOf, class Emit>
 __device__ __forceinline__ void q8_rows_chunked(const uint8_t* codes, const uint16_t* scales, const uint16_t* biases, uint32_t K,
-                                                const uint16_t* x, uint32_t rows, RowOf row_of, Emit emit) {
+                                                const uint16_t* const* x, uint32_t rows, RowOf row_of, Emit emit) {
     const uint32_t l32 = threadIdx.x & 31u, per = K / 256u, groups = K / 64u;
     for (uint32_t i0 = 0; i0 < rows; i0 += ROWS) {
-        float result[ROWS];
+        float result[NTOK][ROWS];
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) result[r] = 0.0f;
+        for (int t = 0; t < NTOK; ++t)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) result[t][r] = 0.0f;
         for (uint32_t j0 = 0; j0 < per; j0 += CH) {
             uint2 q[ROWS][CH]; uint16_t sb[ROWS][CH], bb[ROWS][CH];
 #pragma unroll
@@ -57,37 +60,44 @@ __device__ __forceinline__ void q8_rows_chunked(const uint8_t* codes, const uint
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
                 const uint32_t b = l32 + 32u * (j0 + c);
-                const uint4 raw = *reinterpret_cast<const uint4*>(x + b * 8u);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-                float xb[8];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { xb[2 * e] = __uint_as_float(w[e] << 16); xb[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u); }
-                float sum = 0;
+                for (int t = 0; t < NTOK; ++t) {
+                    const uint4 raw = *reinterpret_cast<const uint4*>(x[t] + b * 8u);
+                    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+                    float xb[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) sum += xb[e];
+                    for (int e = 0; e < 4; ++e) { xb[2 * e] = __uint_as_float(w[e] << 16); xb[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u); }
+                    float sum = 0;
 #pragma unroll
-                for (int r = 0; r < ROWS; ++r) {
-                    const uint32_t words[2] = {q[r][c].x, q[r][c].y};
-                    float dot = 0;
+                    for (int e = 0; e < 8; ++e) sum += xb[e];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) dot += xb[e] * float((words[e / 4] >> (8 * (e % 4))) & 255u);
-                    result[r] += b16(sb[r][c]) * dot + sum * b16(bb[r][c]);
+                    for (int r = 0; r < ROWS; ++r) {
+                        const uint32_t words[2] = {q[r][c].x, q[r][c].y};
+                        float dot = 0;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) dot += xb[e] * float((words[e / 4] >> (8 * (e % 4))) & 255u);
+                        result[t][r] += b16(sb[r][c]) * dot + sum * b16(bb[r][c]);
+                    }
                 }
             }
         }
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            const float v = lane_sum32(result[r]);
-            if (i0 + r < rows) emit(i0 + r, v);
-        }
+        for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+            for (int t = 0; t < NTOK; ++t) {
+                const float v = lane_sum32(result[t][r]);
+                if (i0 + r < rows) emit(i0 + r, t, v);
+            }
     }
 }
-// DEEP: four rows per half in flight (short rows: the down projection); otherwise two.
+// One token.  DEEP: four rows per half in flight (short rows: the down projection); otherwise two.
 template <bool DEEP, class RowOf, class Emit>
 __device__ __forceinline__ void q8_rows(const uint8_t* codes, const uint16_t* scales, const uint16_t* biases, uint32_t K,
                                         const uint16_t* x, uint32_t rows, RowOf row_of, Emit emit) {
-    if constexpr (DEEP) q8_rows_chunked<2, 4>(codes, scales, biases, K, x, rows, row_of, emit);
-    else q8_rows_chunked<2, 2>(codes, scales, biases, K, x, rows, row_of, emit);
+    const uint16_t* const rows_in[1] = {x};
+    auto emit_one = [&](uint32_t i, int, float v) { emit(i, v); };
+    if constexpr (DEEP) q8_rows_chunked<2, 4, 1>(codes, scales, biases, K, rows_in, rows, row_of, emit_one);
+    else q8_rows_chunked<2, 2, 1>(codes, scales, biases, K, rows_in, rows, row_of, emit_one);
 }
 
 struct Barrier {

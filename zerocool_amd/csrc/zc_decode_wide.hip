@@ -41,6 +41,9 @@ __device__ __forceinline__ void run_tile_wide(const uint8_t* w_row, const uint16
     else xint_run_tile_tokens_piped<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
 }
 
+// MIXED: the down projection and/or the shared expert are affine Q8 and run on literal lanes (q8_rows_chunked); a variant of
+// its own, so that the all-Q4 kernel is exactly what it was.  It also serves two to eight tokens of such artifacts.
+template <bool MIXED>
 __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams p, WideLdsPlan lp) {
     constexpr int PT = kWidePass, MT = kWideBatch;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -307,12 +310,17 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
         clock();
         // ---------------- phase G: gate/up tiles; items (entry, tile, pass), one contiguous range per workgroup ----------------
         {
-            const uint32_t tiles = I / 8, total = tiles * uint32_t(cum[NE]);
+            // A Q8 gate/up tile of the shared expert is several memory latencies long: its items are cut into `cut` pieces of
+            // 8 / cut row pairs, i.e. the shared entries (the last ones of the list) count `cut` times their passes here.
+            const bool q8_shared = MIXED && p.shared_bits_gate_up == 8;
+            const uint32_t cut = q8_shared ? 4u : 1u, routed_passes = uint32_t(cum[U]);
+            auto gcum = [&](uint32_t i) { const uint32_t c = uint32_t(uniform(cum[i])); return i <= U ? c : routed_passes + cut * (c - routed_passes); };
+            const uint32_t tiles = I / 8, total = tiles * gcum(NE);
             const uint32_t i0 = uint32_t(uint64_t(wg) * total / nwg), i1 = uint32_t(uint64_t(wg + 1) * total / nwg);
             uint32_t ei = 0;
-            while (ei + 1 < NE && tiles * uint32_t(uniform(cum[ei + 1])) <= i0) ++ei;
+            while (ei + 1 < NE && tiles * gcum(ei + 1) <= i0) ++ei;
             for (uint32_t at = i0; at < i1; ++ei) {
-                const uint32_t first = tiles * uint32_t(uniform(cum[ei])), seg_end = min(i1, tiles * uint32_t(uniform(cum[ei + 1])));
+                const uint32_t first = tiles * gcum(ei), seg_end = min(i1, tiles * gcum(ei + 1));
                 int32_t all[MT], token[MT]; bool routed; uint32_t e;
                 const int na = slots_of(ei, all, token, routed, e);
                 __syncthreads();   // the previous entry's tiles have read their rows and images
@@ -327,6 +335,25 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
                 const uint64_t* off = routed ? p.ro : p.so;
                 const uint32_t passes = uint32_t(na + PT - 1) / PT;
                 for (uint32_t item = at + wave; item < seg_end; item += kWideWaves) {
+                    if (MIXED && !routed && q8_shared) {
+                        // affine Q8 rows: the lower half of the wave takes gate rows, the upper half the up rows of the same indices
+                        const uint32_t local = item - first, piece = local % cut, pass = (local / cut) % passes, tile = local / (cut * passes);
+                        int32_t slot[PT]; uint32_t index[PT];
+                        const int nt = pass_of(all, na, pass, slot, index);
+                        const uint32_t side = lane >> 5, per_piece = 8 / cut, row0 = tile * 8 + piece * per_piece;
+                        const uint16_t* const rows_in[PT] = {xh + index[0] * H, xh + index[PT - 1] * H};
+                        q8_rows_chunked<2, 2, PT>(rec + p.so[side * 3], reinterpret_cast<const uint16_t*>(rec + p.so[side * 3 + 1]),
+                                reinterpret_cast<const uint16_t*>(rec + p.so[side * 3 + 2]), H, rows_in, per_piece,
+                                [&](uint32_t i) { return row0 + i; },
+                                [&](uint32_t i, int t, float v) {
+                                    const float up = __shfl(v, 32);
+                                    const uint32_t a = __float_as_uint(swiglu_bf(v, up)) >> 16;   // BF16 bits
+                                    if (lane == 0 && t < nt)
+                                        __hip_atomic_store(reinterpret_cast<uint16_t*>(p.shared_act) + uint64_t(uint32_t(slot[t]) - n) * I + row0 + i, uint16_t(a),
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                });
+                        continue;
+                    }
                     const uint32_t tile = (item - first) / passes, pass = (item - first) % passes;
                     const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                     const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
@@ -382,6 +409,16 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
                     const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
                     int32_t slot[PT]; uint32_t index[PT];
                     const int nt = pass_of(all, na, pass, slot, index);
+                    if (MIXED && (routed ? p.bits_down : p.shared_bits_down) == 8) {   // affine Q8 down rows: row 2 i of the tile on the lower half, 2 i + 1 on the upper
+                        const uint32_t row0 = ((item - first) / passes) * 16;
+                        const uint16_t* const rows_in[PT] = {ah + index[0] * I, ah + index[PT - 1] * I};
+                        q8_rows_chunked<2, 4, PT>(rec + off[6], reinterpret_cast<const uint16_t*>(rec + off[7]), reinterpret_cast<const uint16_t*>(rec + off[8]), I,
+                                rows_in, 8, [&](uint32_t i) { return row0 + 2 * i + (lane >> 5); },
+                                [&](uint32_t i, int t, float v) {
+                                    if ((lane & 31u) == 0 && t < nt) st_f32(p.eout + uint64_t(slot[t]) * H + row0 + 2 * i + (lane >> 5), bf(v));
+                                });
+                        continue;
+                    }
                     const uint8_t* img[PT]; LdsBf16 src[PT];
 #pragma unroll
                     for (int t = 0; t < PT; ++t) { img[t] = lds + lp.img_d + index[t] * LI.bytes(); src[t] = LdsBf16{ah + index[t] * I}; }
@@ -464,16 +501,26 @@ WideLdsPlan decode_wide_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t
     return lp;
 }
 
+static bool wide_mixed(const DecodeParams& p) { return !(p.bits_down == 4 && p.shared_bits_gate_up == 4 && p.shared_bits_down == 4); }
 hipError_t launch_decode_wide(hipStream_t s, const DecodeParams& p, uint32_t workgroups, const WideLdsPlan& lp) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));
+    const void* kernel = wide_mixed(p) ? reinterpret_cast<const void*>(decode_wide_kernel<true>) : reinterpret_cast<const void*>(decode_wide_kernel<false>);
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(decode_wide_kernel, dim3(workgroups), dim3(kWideThreads), lp.total, s, p, lp);
+    if (wide_mixed(p)) hipLaunchKernelGGL(decode_wide_kernel<true>, dim3(workgroups), dim3(kWideThreads), lp.total, s, p, lp);
+    else hipLaunchKernelGGL(decode_wide_kernel<false>, dim3(workgroups), dim3(kWideThreads), lp.total, s, p, lp);
     return hipGetLastError();
 }
 hipError_t decode_wide_occupancy(uint32_t lds_bytes, int* blocks_per_cu) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    int plain = 0, mixed = 0;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_wide_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, decode_wide_kernel, kWideThreads, lds_bytes);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_wide_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, decode_wide_kernel<false>, kWideThreads, lds_bytes);
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&mixed, decode_wide_kernel<true>, kWideThreads, lds_bytes);
+    *blocks_per_cu = plain < mixed ? plain : mixed;
+    return e;
 }
 
 }  // namespace zc

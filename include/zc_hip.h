@@ -307,7 +307,7 @@ zc_status zc_hip_store_table_stats(const zc_hip_store* store, zc_store_table_sta
 zc_status zc_hip_store_geometry(const zc_hip_store* store, uint32_t* layers, uint32_t* experts, uint64_t* record_bytes);
 /* A decode stack whose routed records live in an expert store (the capped-HBM run: model.cpp:431-557 with the cache of
  * storage.cpp:525-725 in the loop).  host_layers[l].expert_records is ignored; the store must have n_layers layers of
- * cfg's records, and max_tokens <= 8.  zc_hip_stack_decode on such a stack is ONE launch that reads every record
+ * cfg's records, and max_tokens <= 64.  zc_hip_stack_decode on such a stack is ONE launch that reads every record
  * through the store's table (zc_hip_store_table), then waits for the launch on the host, copies the routes back and
  * hands them to zc_hip_store_table_observe, so that the records this step read from their homes are in HBM slots for
  * the steps to come.  Output bytes are those of a stack with all records resident.  flags bit 0 (layer by layer) is

@@ -114,7 +114,7 @@ def _stack_pair(ctx, cfg, seeds, skew, slots):
     """The same layers twice: records resident in HBM, and records behind an expert store with `slots` HBM slots."""
     resident = [workload.LayerWeights(ctx, cfg, seed, skew) for seed in seeds]
     capped = workload.StoreBackedStack(ctx, cfg, seeds, skew, slots)
-    return resident, ctx.stack_create(cfg, [w.layer for w in resident], 8), capped, capped.decode_stack(8)
+    return resident, ctx.stack_create(cfg, [w.layer for w in resident], 24), capped, capped.decode_stack(24)
 
 
 def test_decode_stack_behind_a_store_equals_the_resident_stack(ctx):
@@ -124,9 +124,9 @@ def test_decode_stack_behind_a_store_equals_the_resident_stack(ctx):
     cfg = workload.tiny_config(hidden=512, experts=32, topk=4, inter=512)
     resident, full, capped, stack = _stack_pair(ctx, cfg, [51, 52, 53], ("normal", 0.5), slots=10)
     assert ctx.stack_is_persistent(stack, 1) and ctx.stack_is_persistent(stack, 8)
-    n = 3 * 8 * cfg.topk
+    n = 3 * 24 * cfg.topk
     ids_a, w_a, ids_b, w_b = (ctx.alloc(n * 4) for _ in range(4))
-    for step, tokens in enumerate((1, 1, 3, 1, 8, 1, 1, 2, 1, 1, 5, 1, 1, 1)):
+    for step, tokens in enumerate((1, 1, 3, 1, 8, 1, 1, 2, 1, 24, 1, 5, 1, 13, 1)):
         x = workload.hidden_rows(ctx, tokens, cfg.hidden, 7000 + step)
         want, got = ctx.alloc(tokens * cfg.hidden * 4), ctx.alloc(tokens * cfg.hidden * 4)
         traced = step % 2 == 0   # with the caller's trace buffers and with the stack's own

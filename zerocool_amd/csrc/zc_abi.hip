@@ -840,7 +840,7 @@ static zc_status create_stack(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         if (const zc_status s = zc_hip_store_geometry(store, &store_layers, &store_experts, &store_record)) return s;
         ZC_REQUIRE(store_layers == n_layers && store_experts == c->experts && store_record == zc_hip_record_bytes(c, 0),
                    "the expert store does not hold this stack's records");
-        ZC_REQUIRE(max_tokens <= 8, "a stack behind an expert store decodes at most 8 tokens a launch");
+        ZC_REQUIRE(max_tokens <= 64, "a stack behind an expert store decodes at most 64 tokens a call (one launch)");
         if (const zc_status s = zc_hip_store_table(store, &table)) return s;
     }
     for (uint32_t l = 0; l < n_layers; ++l) {
@@ -1032,7 +1032,7 @@ zc_status zc_hip_stack_set_speculation(zc_hip_ctx* ctx, zc_hip_stack* st, int on
 }
 int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t tokens) {
     if (!ctx || !st || !tokens) return 0;
-    if (st->store && tokens > 8) return 0;
+    if (st->store && tokens > 64) return 0;
     return launch_unit(ctx, st, tokens) ? 1 : 0;
 }
 zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
@@ -1045,7 +1045,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
     LaunchPlan plan;
     const uint32_t unit = (flags & 1u) ? 0u : launch_unit(ctx, st, tokens);
     if (st->store) {
-        ZC_REQUIRE(unit && tokens <= 8, "a stack behind an expert store runs as one launch only");
+        ZC_REQUIRE(unit && tokens <= unit, "a stack behind an expert store runs as one launch only");
         if (const zc_status s = zc_hip_store_table_refresh(st->store)) return s;
     }
     // More than eight tokens go through the single-launch kernels sixty-four (or eight) at a time, one launch per piece (tokens

@@ -13,10 +13,13 @@
 // specified by a tolerance (max relative error 2e-3 of the layer output), not as bit-exact.  Routing, dispatch and the
 // combine use the exact kernels.
 //
-// Tiling.  One workgroup (4 waves) owns 32 sorted token rows of ONE expert and 128 weight rows (gate/up: 64 gate rows
+// Tiling.  One workgroup (4 waves) owns up to 48 sorted token rows of ONE expert and 128 weight rows (gate/up: 64 gate rows
 // and the 64 up rows of the same indices, so SwiGLU is fused in registers), and walks K in steps of 64 = one scale
 // group: the 4-bit codes of the step are expanded to bf16 once per workgroup into LDS, the token rows are gathered into
-// LDS as bf16, both double-buffered.  Each wave multiplies a 16-row half of the tokens by 4 of the 8 column tiles.
+// LDS as bf16, both double-buffered.  Each wave multiplies all (two or three) 16-row blocks of the tokens by 2 of the 8
+// column tiles.  An expert's rows are cut into tiles of 32, except that a run of up to 48 rows (a whole expert with few
+// rows, or the last rows of a longer run) is ONE tile: with about forty rows per expert -- an unskewed router at 2048
+// tokens -- every expert's codes are then expanded once, not twice.
 #include "zc_kernels.hpp"
 #include "zc_device.hpp"
 
@@ -27,7 +30,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kTileRows = 32, kTileCols = 128, kPitch = 72;   // LDS row pitch in bf16 elements (144 bytes)
+constexpr uint32_t kTileRows = 32, kTileRowsMax = 48, kTileCols = 128, kPitch = 72;   // LDS row pitch in bf16 elements (144 bytes)
 
 // fp32 rows holding BF16 values -> bf16 rows, plus per (row, group of 64) the sum of the four blocks' BF16-rounded
 // sum-of-four chains.  One thread per (row, group).  status bit 4: a value was not BF16-valued.
@@ -91,7 +94,9 @@ __global__ __launch_bounds__(1024) void prefill_tiles_kernel(const int32_t* offs
     __shared__ int32_t scan[1024];
     const uint32_t e = threadIdx.x;
     const int32_t first = offsets ? (e < experts ? offsets[e] : 0) : 0, count = offsets ? (e < experts ? offsets[e + 1] - offsets[e] : 0) : (e == 0 ? int32_t(rows) : 0);
-    const int32_t tiles = (count + int32_t(kTileRows) - 1) / int32_t(kTileRows);
+    // whole tiles of 32 rows; what is left joins the last of them when that gives at most 48 rows, else it is a tile of its own
+    const int32_t whole = count / int32_t(kTileRows), left = count % int32_t(kTileRows);
+    const int32_t tiles = count == 0 ? 0 : (whole == 0 ? 1 : whole + (left > int32_t(kTileRowsMax - kTileRows) ? 1 : 0));
     scan[e] = tiles;
     __syncthreads();
     for (uint32_t step = 1; step < 1024; step <<= 1) {
@@ -103,16 +108,16 @@ __global__ __launch_bounds__(1024) void prefill_tiles_kernel(const int32_t* offs
     const int32_t begin = scan[e] - tiles;
     for (int32_t t = 0; t < tiles; ++t) {
         tile_expert[begin + t] = int32_t(e); tile_first[begin + t] = first + t * int32_t(kTileRows);
-        tile_rows[begin + t] = min(int32_t(kTileRows), count - t * int32_t(kTileRows));
+        tile_rows[begin + t] = t + 1 < tiles ? int32_t(kTileRows) : count - t * int32_t(kTileRows);   // the last tile takes what is left (at most 48)
     }
     if (e == 1023) *tile_count = scan[1023];
 }
 
 template <bool GATED>
 __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
-    __shared__ __align__(16) uint16_t a_s[2][kTileRows * kPitch];
+    __shared__ __align__(16) uint16_t a_s[2][kTileRowsMax * kPitch];
     __shared__ __align__(16) uint16_t b_s[2][kTileCols * kPitch];
-    __shared__ float scale_s[2][kTileCols], bias_s[2][kTileCols], sum_s[2][kTileRows];
+    __shared__ float scale_s[2][kTileCols], bias_s[2][kTileCols], sum_s[2][kTileRowsMax];
     const uint32_t tile = blockIdx.y;
     if (tile >= uint32_t(*p.tile_count)) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, j = lane & 15u, g4 = lane >> 4;
@@ -126,6 +131,10 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     const uint32_t a_pos = first + min(a_r, rows - 1);                   // rows past the end repeat the last one (never stored)
     const uint32_t a_row = p.a_rows ? uint32_t(p.a_rows[a_pos]) / p.a_div : a_pos;
     const uint16_t* a_src = p.a + uint64_t(a_row) * K + a_c * 8;
+    const bool tall = rows > kTileRows;                                  // a third block of sixteen rows: threads 0..127 fetch it too
+    const uint32_t a_pos2 = first + min(32u + (a_r & 15u), rows - 1);
+    const uint32_t a_row2 = p.a_rows ? uint32_t(p.a_rows[a_pos2]) / p.a_div : a_pos2;
+    const uint16_t* a_src2 = p.a + uint64_t(a_row2) * K + a_c * 8;
     const uint32_t b_r = tid >> 1, b_h = tid & 1u;                       // weight row of the tile, half of the step (32 codes)
     const uint32_t b_proj = GATED ? b_r >> 6 : 0u, b_n = n0 + (GATED ? (b_r & 63u) : b_r);
     const uint8_t* b_src = record + p.off[b_proj * 3] + uint64_t(b_n) * (K / 2) + b_h * 16;
@@ -133,24 +142,25 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     const uint32_t m_proj = GATED ? m_r >> 6 : 0u, m_n = n0 + (GATED ? (m_r & 63u) : m_r);
     const uint16_t* s_src = reinterpret_cast<const uint16_t*>(record + p.off[m_proj * 3 + 1]) + uint64_t(m_n) * groups;
     const uint16_t* o_src = reinterpret_cast<const uint16_t*>(record + p.off[m_proj * 3 + 2]) + uint64_t(m_n) * groups;
-    const uint32_t x_pos = first + min(tid & 31u, rows - 1);
+    const uint32_t x_pos = first + min(tid - 128u < kTileRowsMax ? tid - 128u : 0u, rows - 1);   // threads 128..175: one row's group sums each
     const uint32_t x_row = p.a_rows ? uint32_t(p.a_rows[x_pos]) / p.a_div : x_pos;
     const float* x_src = p.asum + uint64_t(x_row) * groups;
 
     // What a step needs is requested two steps ahead and waits in registers (two sets, taken in turn): with one step of
     // lead the loads' latency, several times a step's arithmetic, was paid at every step.
-    struct Fetched { uint4 a, b; uint16_t s, o; float x; };
+    struct Fetched { uint4 a, a2, b; uint16_t s, o; float x; };
     Fetched ahead[2];
-    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), 0, 0, 0.0f};
+    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), 0, 0, 0.0f};
     auto fetch = [&](uint32_t g, Fetched& f) {
         f.a = *reinterpret_cast<const uint4*>(a_src + g * 64);
         f.b = ldg_u4(b_src + g * 32);
-        if (tid < 128) { f.s = ldg_u16(s_src, g); f.o = ldg_u16(o_src, g); }
-        else if (tid < 160) f.x = x_src[g];
+        if (tid < 128) { f.s = ldg_u16(s_src, g); f.o = ldg_u16(o_src, g); if (tall) f.a2 = *reinterpret_cast<const uint4*>(a_src2 + g * 64); }
+        else if (tid < 128 + kTileRowsMax) f.x = x_src[g];
     };
     auto stash = [&](uint32_t buf, const Fetched& f) {
         const uint4 a_next = f.a, b_next = f.b; const uint16_t s_next = f.s, o_next = f.o; const float x_next = f.x;
         *reinterpret_cast<uint4*>(&a_s[buf][a_r * kPitch + a_c * 8]) = a_next;
+        if (tall && tid < 128) *reinterpret_cast<uint4*>(&a_s[buf][(32 + a_r) * kPitch + a_c * 8]) = f.a2;
         // 32 codes -> 32 bf16: nibble i of a word is element 8w+i
         const uint32_t words[4] = {b_next.x, b_next.y, b_next.z, b_next.w};
         uint32_t out[16];
@@ -170,17 +180,21 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) dst[q] = make_uint4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
         if (tid < 128) { scale_s[buf][m_r] = b16(s_next); bias_s[buf][m_r] = b16(o_next); }
-        else if (tid < 160) sum_s[buf][tid & 31u] = x_next;
+        else if (tid < 128 + kTileRowsMax) sum_s[buf][tid - 128u] = x_next;
     };
 
-    const uint32_t wm = wave & 1u, wn = wave >> 1;
-    // the wave's four column tiles (rows of b_s): gate/up: two gate tiles and the up tiles of the same rows
-    uint32_t col_row[4];
+    // the wave's two column tiles (rows of b_s) for every block of sixteen token rows; gate/up: a gate tile and the up tile of
+    // the same rows
+    uint32_t col_row[2];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) col_row[q] = (GATED ? ((q >> 1) * 64u + (2 * wn + (q & 1)) * 16u) : (4 * wn + q) * 16u) + j;
-    f32x4 total[4], mag[4];                  // mag: sum of the magnitudes of the folded terms, the scale of the rounding error
+    for (int q = 0; q < 2; ++q) col_row[q] = (GATED ? (uint32_t(q) * 64u + wave * 16u) : (2 * wave + uint32_t(q)) * 16u) + j;
+    constexpr int kBlocks = int(kTileRowsMax / 16);
+    const int blocks = tall ? kBlocks : 2;
+    f32x4 total[kBlocks][2], mag[kBlocks][2];   // mag: sum of the magnitudes of the folded terms, the scale of the rounding error
 #pragma unroll
-    for (int q = 0; q < 4; ++q) total[q] = mag[q] = f32x4{0, 0, 0, 0};
+    for (int rb = 0; rb < kBlocks; ++rb)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) total[rb][q] = mag[rb][q] = f32x4{0, 0, 0, 0};
 
     fetch(0, ahead[0]);
     if (groups > 1) fetch(1, ahead[1]);
@@ -191,29 +205,40 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     auto step = [&](uint32_t g, Fetched& mine, Fetched& next) {
         const uint32_t buf = g & 1u;
         if (g + 2 < groups) fetch(g + 2, mine);
-        f32x4 dot[4];
+        f32x4 dot[kBlocks][2];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) dot[q] = f32x4{0, 0, 0, 0};
+        for (int rb = 0; rb < kBlocks; ++rb)
+#pragma unroll
+            for (int q = 0; q < 2; ++q) dot[rb][q] = f32x4{0, 0, 0, 0};
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&a_s[buf][(16 * wm + j) * kPitch + kk * 32 + g4 * 8]));
+            bf16x8 b[2];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&b_s[buf][col_row[q] * kPitch + kk * 32 + g4 * 8]));
-                dot[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, dot[q], 0, 0, 0);
+            for (int q = 0; q < 2; ++q) b[q] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&b_s[buf][col_row[q] * kPitch + kk * 32 + g4 * 8]));
+#pragma unroll
+            for (int rb = 0; rb < kBlocks; ++rb) {
+                if (rb >= blocks) break;
+                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&a_s[buf][(16 * rb + j) * kPitch + kk * 32 + g4 * 8]));
+#pragma unroll
+                for (int q = 0; q < 2; ++q) dot[rb][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[q], dot[rb][q], 0, 0, 0);
             }
         }
-        float sums[4];
+        float scale[2], bias[2];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sums[r] = sum_s[buf][16 * wm + 4 * g4 + r];
+        for (int q = 0; q < 2; ++q) { scale[q] = scale_s[buf][col_row[q]]; bias[q] = bias_s[buf][col_row[q]]; }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float scale = scale_s[buf][col_row[q]], bias = bias_s[buf][col_row[q]];
+        for (int rb = 0; rb < kBlocks; ++rb) {
+            if (rb >= blocks) break;
+            float sums[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                total[q][r] = __builtin_fmaf(scale, dot[q][r], __builtin_fmaf(bias, sums[r], total[q][r]));
-                mag[q][r] = __builtin_fmaf(fabsf(scale), fabsf(dot[q][r]), __builtin_fmaf(fabsf(bias), fabsf(sums[r]), mag[q][r]));
-            }
+            for (int r = 0; r < 4; ++r) sums[r] = sum_s[buf][16 * rb + 4 * g4 + r];
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    total[rb][q][r] = __builtin_fmaf(scale[q], dot[rb][q][r], __builtin_fmaf(bias[q], sums[r], total[rb][q][r]));
+                    mag[rb][q][r] = __builtin_fmaf(fabsf(scale[q]), fabsf(dot[rb][q][r]), __builtin_fmaf(fabsf(bias[q]), fabsf(sums[r]), mag[rb][q][r]));
+                }
         }
         if (g + 1 < groups) stash(buf ^ 1u, next);
         __syncthreads();
@@ -230,26 +255,27 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     // lanes that share a token row hold sixteen neighbouring weight rows.
     uint16_t* bits = reinterpret_cast<uint16_t*>(p.near_bits);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const uint32_t m = 16 * wm + 4 * g4 + r;
-        const bool live = m < rows;
-        const uint32_t pos = first + (live ? m : 0u);
-        if constexpr (GATED) {
+    for (int rb = 0; rb < kBlocks; ++rb) {
+        if (rb >= blocks) break;
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const uint32_t n = n0 + (2 * wn + q) * 16 + j;
-                if (live) p.out_b[uint64_t(pos) * N + n] = uint16_t(__float_as_uint(swiglu_bf(total[q][r], total[2 + q][r])) >> 16);
-                const uint64_t marks = __ballot(near_boundary(total[q][r], mag[q][r]) || near_boundary(total[2 + q][r], mag[2 + q][r]));
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t m = 16 * uint32_t(rb) + 4 * g4 + uint32_t(r);
+            const bool live = m < rows;
+            const uint32_t pos = first + (live ? m : 0u);
+            if constexpr (GATED) {
+                const uint32_t n = n0 + wave * 16 + j;
+                if (live) p.out_b[uint64_t(pos) * N + n] = uint16_t(__float_as_uint(swiglu_bf(total[rb][0][r], total[rb][1][r])) >> 16);
+                const uint64_t marks = __ballot(near_boundary(total[rb][0][r], mag[rb][0][r]) || near_boundary(total[rb][1][r], mag[rb][1][r]));
                 if (live && j == 0) bits[(uint64_t(pos) * N + n) / 16] = uint16_t(marks >> (16 * g4));
-            }
-        } else {
-            const uint32_t out_row = p.out_rows ? uint32_t(p.out_rows[pos]) : pos;
+            } else {
+                const uint32_t out_row = p.out_rows ? uint32_t(p.out_rows[pos]) : pos;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t n = n0 + (4 * wn + q) * 16 + j;
-                if (live) p.out_f[uint64_t(out_row) * N + n] = bf(total[q][r]);
-                const uint64_t marks = __ballot(near_boundary(total[q][r], mag[q][r]));
-                if (live && j == 0) bits[(uint64_t(pos) * N + n) / 16] = uint16_t(marks >> (16 * g4));
+                for (int q = 0; q < 2; ++q) {
+                    const uint32_t n = n0 + (2 * wave + uint32_t(q)) * 16 + j;
+                    if (live) p.out_f[uint64_t(out_row) * N + n] = bf(total[rb][q][r]);
+                    const uint64_t marks = __ballot(near_boundary(total[rb][q][r], mag[rb][q][r]));
+                    if (live && j == 0) bits[(uint64_t(pos) * N + n) / 16] = uint16_t(marks >> (16 * g4));
+                }
             }
         }
     }

@@ -87,6 +87,7 @@ def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), spec
     """The same single-layer configuration through the persistent decode kernels as a stack of one layer: one launch per
     step up to eight tokens, one launch per eight tokens above that; over 8 distinct inputs in rotation."""
     import numpy as np
+    import zerocool_amd as z
     from zerocool_amd import workload
     c = workload.config(name)
     lw = workload.LayerWeights(ctx, c, workload.BASE_SEED + 77, skew)
@@ -96,12 +97,16 @@ def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), spec
     out = ctx.alloc(tokens * c.hidden * 4)
     ws = ctx.alloc(ctx.moe_workspace_bytes(c, tokens))
     ref = ctx.alloc(tokens * c.hidden * 4)
+    ids, wts = ctx.alloc(tokens * c.topk * 4), ctx.alloc(tokens * c.topk * 4)
+    unique = []
     for x in xs:   # parity gate: the operator path's bytes (glue of layer 0 is the identity on the input)
-        ctx.stack_decode(stack, x, tokens, out)
+        ctx.stack_decode(stack, x, tokens, out, z.StackTrace(ids.ptr, wts.ptr, None, None))
         ctx.moe_forward(c, lw.layer, x, tokens, ref, ws)
         ctx.moe_check()
         if out.numpy(np.float32).tobytes() != ref.numpy(np.float32).tobytes():
             raise SystemExit("bench.py: one-launch layer and operator path disagree; refusing to time")
+        unique.append(len(np.unique(ids.numpy(np.int32))))
+    nbytes = float(np.mean([workload.layer_bytes(c, u, tokens, ctx) for u in unique]))
     for i in range(warmup):
         ctx.stack_decode(stack, xs[i % INPUTS], tokens, out)
     ctx.finish()
@@ -112,9 +117,11 @@ def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), spec
     ctx.moe_check()
     persistent = ctx.stack_is_persistent(stack, tokens)
     ctx.stack_destroy(stack)
-    for b in xs + [out, ws, ref, lw.router, lw.shared_gate, lw.shared_record, lw.records]:
+    for b in xs + [out, ws, ref, ids, wts, lw.router, lw.shared_gate, lw.shared_record, lw.records]:
         ctx.free(b)
     return {"tokens": tokens, "us_per_layer": ms * 1e3, "tokens_per_s": tokens / (ms * 1e-3), "router_skew": list(skew) if skew else None,
+            "distinct_experts": float(np.mean(unique)), "slots_per_distinct_expert": tokens * c.topk / float(np.mean(unique)),
+            "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 8e12,
             "guessing": bool(speculate), "path": "persistent single-launch kernel" if persistent else "layer by layer"}
 
 
@@ -344,10 +351,14 @@ def main():
         capped.close()
         # Single-layer configurations: decode batches through the exact operator path, and batches through the
         # sorted-token grouped product on the bf16 matrix cores.
+        # BASELINE configs[1]: continuous-batching decode of the single-layer shape behind N(0, 0.5) router offsets: GEMV
+        # bandwidth over the distinct records of a step, and the expert dedup across its tokens (slots per distinct expert)
+        extra["single_layer_q4_one_launch_normal_0.5"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50, skew=("normal", 0.5)) for t in (1, 8, 32, 64)]
         extra["single_layer_q4_one_launch"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50) for t in (1, 8, 32, 64)]
         # raw random inputs behind an unskewed router share next to no experts from one step to the next: every guess of
         # the one-token kernel misses, which prices the guessing at its worst
         extra["single_layer_q4_one_launch_all_guesses_miss"] = [one_launch_layer(ctx, "S", 1, 200, skew=None, speculate=on) for on in (True, False)]
+        extra["single_layer_q4_normal_0.5"] = [single_layer(ctx, "S", t, False, 30, skew=("normal", 0.5)) for t in (1, 8, 32, 64)]
         extra["single_layer_q4"] = [single_layer(ctx, "S", t, False, 50) for t in (1, 8, 32, 64)]
         extra["single_layer_mixed_one_launch"] = [one_launch_layer(ctx, "S-mixed", t, 100) for t in (1, 8, 16)]
         extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8, 16)]

@@ -155,7 +155,10 @@ def main():
                     help="stack: the 48-layer decode stack (the headline); prefill: one 2048-token batch through one layer of "
                          "hidden 2048 / 512 experts / top-10 / intermediate 512 on the bf16 matrix cores")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="--workload prefill: tokens of the batch")
-    ap.add_argument("--capped-layers", type=int, default=12, help="--extra: layers of the capped-HBM run (48 pins 130 GB of host memory)")
+    ap.add_argument("--capped-layers", type=int, default=48, help="--extra: layers of the capped-HBM run")
+    ap.add_argument("--capped-homes", type=int, default=12,
+                    help="--extra: pinned-host homes of the capped-HBM run's records; layer l shares the home of layer l mod this number "
+                         "(48 distinct homes would pin 130 GB of host memory, more than this pool's boxes grant; 24 are 65 GB)")
     ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: rewrite the tracked traffic file from the output folders of the two counter runs")
@@ -306,49 +309,56 @@ def main():
             for o in offsets:
                 if o: ctx.free(o)
         # The capped-HBM run of the same configuration: the records' home is pinned host memory and 2000 of the 24576
-        # records fit in HBM slots (the same fraction on --capped-layers layers, so that the pinned home stays modest by
-        # default).  Each step is one launch of the same persistent kernels, which take every record's address from the
-        # store's table: an HBM slot, or the record's home over the host link; after the launch the store admits what was
-        # read from home (fills on its side stream).  Timed by the host clock: the step includes the wait for the launch,
-        # the readback of the routes and the store's bookkeeping.
+        # records fit in HBM slots.  The host cannot pin all 130 GB, so the 48 layers share --capped-homes pinned homes
+        # (layer l holds the records of layer l mod that number; routers, shared experts and offsets are every layer's
+        # own, and the slot cache keys every (layer, expert) separately, so the slot traffic is that of 48 distinct layers).
+        # Each step is one launch of the same persistent kernels, which take every record's address from the store's
+        # table: an HBM slot, or the record's home over the host link; after the launch the store admits what was read
+        # from home (fills on its side stream).  Timed by the host clock: the step includes the wait for the launch, the
+        # readback of the routes and the store's bookkeeping.
         ctx.stack_destroy(stack)
         for l in layers:
             for b in (l.router, l.shared_gate, l.shared_record, l.records):
                 ctx.free(b)
         CL = args.capped_layers
-        slots = max(cfg.topk + 2, 2000 * CL // 48)
-        capped = workload.StoreBackedStack(ctx, cfg, [workload.BASE_SEED + 4 * 1000 + l for l in range(CL)], ("zipf", 1.1), slots)
-        cstack = capped.decode_stack(8)
-        extra["capped_hbm"] = {"layers": CL, "hbm_slots": int(slots), "records": CL * cfg.experts,
-                               "pinned_home_bytes": CL * cfg.experts * int(capped.store.stride)}
-        for tokens in (1, 8):
-            xs = [workload.hidden_rows(ctx, tokens, cfg.hidden, workload.BASE_SEED + 4 * 7 + tokens + 97 * i) for i in range(INPUTS)]
-            out = ctx.alloc(tokens * cfg.hidden * 4)
-            t0 = time.perf_counter()
-            ctx.stack_decode(cstack, xs[0], tokens, out)      # cold: every record comes over the host link
-            cold = time.perf_counter() - t0
-            for i in range(2 * INPUTS):
-                ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
-            ctx.finish(); ctx.moe_check()
-            seen0, st0 = capped.store.table_stats(), capped.store.stats()
-            reads0, slot0, home0, fill0 = seen0.reads, seen0.slot_reads, seen0.home_read_bytes, st0.bytes
-            n_steps = max(16, args.steps)
-            t0 = time.perf_counter()
-            for i in range(n_steps):
-                ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
-            dt = (time.perf_counter() - t0) / n_steps
-            ctx.moe_check()
-            seen, st = capped.store.table_stats(), capped.store.stats()
-            extra["capped_hbm"][f"batch{tokens}"] = {
-                "ms_per_step": dt * 1e3, "us_per_layer": dt / CL * 1e6, "tokens_per_s_at_48_layers": tokens / (dt / CL * 48),
-                "first_step_ms": cold * 1e3, "slot_hit_rate": (seen.slot_reads - slot0) / max(1, seen.reads - reads0),
-                "bytes_read_from_home_per_token": (seen.home_read_bytes - home0) / n_steps / tokens * 48 / CL,
-                "bytes_filled_into_slots_per_token": (st.bytes - fill0) / n_steps / tokens * 48 / CL}
-            for b in xs + [out]:
-                ctx.free(b)
-        extra["capped_hbm"]["evictions"] = int(capped.store.stats().evictions)
-        ctx.stack_destroy(cstack)
-        capped.close()
+        homes = min(CL, args.capped_homes)
+        extra["capped_hbm"] = {}
+        # 2000 slots (the configuration), and as many slots as one token selects experts per step (48 x top-10 = 480): fewer than
+        # the eight rotating inputs touch, so every step misses and the slots turn over
+        for slots, batches in ((max(cfg.topk + 2, 2000 * CL // 48), (1, 8)), (CL * cfg.topk, (1,))):
+            capped = workload.StoreBackedStack(ctx, cfg, [workload.BASE_SEED + 4 * 1000 + l for l in range(CL)], ("zipf", 1.1), slots, home_layers=homes)
+            cstack = capped.decode_stack(8)
+            report = {"layers": CL, "hbm_slots": int(slots), "records": CL * cfg.experts,
+                      "record_homes": homes, "pinned_home_bytes": homes * cfg.experts * int(capped.store.stride)}
+            for tokens in batches:
+                xs = [workload.hidden_rows(ctx, tokens, cfg.hidden, workload.BASE_SEED + 4 * 7 + tokens + 97 * i) for i in range(INPUTS)]
+                out = ctx.alloc(tokens * cfg.hidden * 4)
+                t0 = time.perf_counter()
+                ctx.stack_decode(cstack, xs[0], tokens, out)      # cold: every record comes over the host link
+                cold = time.perf_counter() - t0
+                for i in range(2 * INPUTS):
+                    ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
+                ctx.finish(); ctx.moe_check()
+                seen0, st0 = capped.store.table_stats(), capped.store.stats()
+                reads0, slot0, home0, fill0, evict0 = seen0.reads, seen0.slot_reads, seen0.home_read_bytes, st0.bytes, st0.evictions
+                n_steps = max(16, args.steps)
+                t0 = time.perf_counter()
+                for i in range(n_steps):
+                    ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
+                dt = (time.perf_counter() - t0) / n_steps
+                ctx.moe_check()
+                seen, st = capped.store.table_stats(), capped.store.stats()
+                report[f"batch{tokens}"] = {
+                    "ms_per_step": dt * 1e3, "us_per_layer": dt / CL * 1e6, "tokens_per_s": tokens / dt * CL / 48 * 48 / CL,
+                    "first_step_ms": cold * 1e3, "slot_hit_rate": (seen.slot_reads - slot0) / max(1, seen.reads - reads0),
+                    "bytes_read_from_home_per_token": (seen.home_read_bytes - home0) / n_steps / tokens,
+                    "bytes_filled_into_slots_per_token": (st.bytes - fill0) / n_steps / tokens,
+                    "evictions_per_step": (st.evictions - evict0) / n_steps}
+                for b in xs + [out]:
+                    ctx.free(b)
+            extra["capped_hbm"][f"{slots}_slots"] = report
+            ctx.stack_destroy(cstack)
+            capped.close()
         # Single-layer configurations: decode batches through the exact operator path, and batches through the
         # sorted-token grouped product on the bf16 matrix cores.
         # BASELINE configs[1]: continuous-batching decode of the single-layer shape behind N(0, 0.5) router offsets: GEMV

@@ -258,6 +258,11 @@ zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts
  * of the slots; takes no prefetches).  Any other name: ZC_INVALID_ARGUMENT "cache policy must be clock or slru". */
 zc_status zc_hip_store_create_with_policy(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots,
                                           const char* policy, zc_hip_store** out);
+/* The same with fewer homes than layers: layer l's records live in home (l mod home_layers), i.e. layers l and l + home_layers
+ * hold the same bytes, while the slot cache still keys every (layer, expert) separately.  For measuring the capped-HBM run
+ * of a model whose records exceed what the host can pin (no counterpart in the reference, which reads from SSD). */
+zc_status zc_hip_store_create_shared_homes(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots,
+                                           const char* policy, uint32_t home_layers, zc_hip_store** out);
 const char* zc_hip_store_policy(const zc_hip_store* store);                 /* "clock" or "slru" (ExpertCache::json "policy") */
 uint64_t zc_hip_store_protected_entries(const zc_hip_store* store);         /* ExpertCache::json "protected_entries" */
 zc_status zc_hip_store_destroy(zc_hip_store* store);
@@ -287,9 +292,9 @@ zc_status zc_hip_store_layer_stats(const zc_hip_store* store, uint32_t layer, ui
  *   zc_hip_store_table_refresh  before a launch: entries of fills that have finished switch to their slots; the changed
  *                               table is copied to the device on the context's stream.
  *   zc_hip_store_table_observe  after the launch has FINISHED (the host has synchronised): the expert ids one layer chose.
- *                               Records read from a slot are touched (ExpertCache::acquire's hit), records read from home
- *                               are admitted (its miss: a victim by CLOCK, the fill starts on the side stream and serves
- *                               later launches); no lease stays out.  A fill never starts while a launch that may read
+ *                               First the records read from a slot are touched (ExpertCache::acquire's hit), then the records
+ *                               read from home are admitted (its miss: a victim by the store's policy that this call did not
+ *                               touch, the fill starts on the side stream and serves later launches); no lease stays out.  A fill never starts while a launch that may read
  *                               its slot is in flight, because fills start here only.
  * Leases and the table may not be mixed on one store while launches are in flight. */
 typedef struct {
@@ -303,6 +308,10 @@ typedef struct {
 zc_status zc_hip_store_table(zc_hip_store* store, const void* const** table);
 zc_status zc_hip_store_table_refresh(zc_hip_store* store);
 zc_status zc_hip_store_table_observe(zc_hip_store* store, uint32_t layer, const int32_t* ids, uint32_t count);
+/* The same for a launch that ran every layer: ids [layers][per_layer].  All records that the launch read from slots are touched
+ * before any record read from home is admitted, whatever their layers, so a miss never takes the slot of a record the same
+ * launch used. */
+zc_status zc_hip_store_table_observe_layers(zc_hip_store* store, const int32_t* ids, uint32_t per_layer);
 zc_status zc_hip_store_table_stats(const zc_hip_store* store, zc_store_table_stats* out);
 zc_status zc_hip_store_geometry(const zc_hip_store* store, uint32_t* layers, uint32_t* experts, uint64_t* record_bytes);
 /* A decode stack whose routed records live in an expert store (the capped-HBM run: model.cpp:431-557 with the cache of

@@ -335,3 +335,43 @@ def test_slru_protects_loading_and_leased_slots_and_survives_resizing():   # tes
     use(s, 0, 9)
     assert s.occupancy == 1
     s.close()
+
+
+def test_layers_can_share_their_records_homes():
+    # Fewer homes than layers: layer l's records live in home l mod home_layers, the cache still tells the layers apart.
+    s = z.Store(None, 4, 8, RECORD, 3, home_layers=2)
+    home = lambda l, e: s.lib.zc_hip_store_backing(s.handle, l, e)
+    assert home(0, 5) == home(2, 5) and home(1, 5) == home(3, 5) and home(0, 5) != home(1, 5)
+    put(s, 0, 5)                                   # also what layer 2 reads
+    assert use(s, 0, 5) == 5.0
+    lease = s.acquire(2, 5); s.wait(lease)
+    assert lease.acquisition == 0 and value(s, lease) == 5.0   # a miss of its own, the same bytes
+    s.release(lease)
+    assert s.stats().misses == 2 and s.occupancy == 2
+    with pytest.raises(z.ZcError):
+        z.Store(None, 4, 8, RECORD, 3, home_layers=5)
+    s.close()
+
+
+def test_a_launch_never_loses_a_record_it_used_to_its_own_misses():
+    # Twelve slots that hold a launch's twelve records; the next launch uses eleven of them and one new record.  The records
+    # read from slots are touched before the new one is admitted, so the victim is the one record this launch did not use --
+    # whatever the order of the ids, and across layers when a launch reports all its layers at once.
+    s = z.Store(None, 2, 32, RECORD, 12)
+    for l in range(2):
+        for e in range(32):
+            put(s, l, e)
+    s.table()
+    first = np.array([[0, 1, 2, 3, 4, 5], [10, 11, 12, 13, 14, 15]], np.int32)
+    s.table_observe_layers(first); s.table_refresh()
+    assert s.table_stats().home_reads == 12
+    second = np.array([[20, 0, 1, 2, 3, 4], [10, 11, 12, 13, 14, 15]], np.int32)   # the new record comes FIRST in the list
+    s.table_observe_layers(second); s.table_refresh()
+    st = s.table_stats()
+    assert (st.slot_reads, st.home_reads) == (11, 13)
+    assert not s.ready(0, 5) and all(s.ready(0, e) for e in (20, 0, 1, 2, 3, 4)) and all(s.ready(1, e) for e in range(10, 16))
+    s.table_observe_layers(second)
+    assert s.table_stats().slot_reads == 23 and s.stats().evictions == 1
+    with pytest.raises(z.ZcError):
+        s.table_observe_layers(np.array([[0], [32]], np.int32))
+    s.close()

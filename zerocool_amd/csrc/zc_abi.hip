@@ -1067,8 +1067,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
             int32_t status = 0;
             ZC_HIP(hipMemcpy(&status, ctx->moe_status, 4, hipMemcpyDeviceToHost));
             if (!status)   // ids of a launch that gave up are not routes
-                for (uint32_t l = 0; l < L; ++l)
-                    if (const zc_status s = zc_hip_store_table_observe(st->store, l, st->route_ids_host + l * per_layer, uint32_t(per_layer))) return s;
+                if (const zc_status s = zc_hip_store_table_observe_layers(st->store, st->route_ids_host, uint32_t(per_layer))) return s;
         }
         return ZC_OK;
     }

@@ -21,6 +21,7 @@ struct zc_hip_store {
     zc_hip_ctx* ctx = nullptr;          // nullptr: host-memory slots
     uint32_t layers = 0, experts = 0;
     uint64_t record_bytes = 0, stride = 0;
+    std::vector<uint8_t*> owned_homes;  // the allocations behind `homes` (fewer than layers when layers share their records' homes)
     std::vector<uint8_t*> homes;        // per layer: [experts] records, pinned host memory (or plain, without a context); one allocation
                                         // per layer, because a single pinned block for a large model can exceed what the driver grants
     uint8_t* pool = nullptr;            // [capacity] slots, HBM (or plain host memory)
@@ -152,7 +153,12 @@ zc_status zc_hip_store_create(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts
 }
 zc_status zc_hip_store_create_with_policy(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots,
                                           const char* policy, zc_hip_store** out) {
+    return zc_hip_store_create_shared_homes(ctx, layers, experts, record_bytes, slots, policy, layers, out);
+}
+zc_status zc_hip_store_create_shared_homes(zc_hip_ctx* ctx, uint32_t layers, uint32_t experts, uint64_t record_bytes, uint64_t slots,
+                                           const char* policy, uint32_t home_layers, zc_hip_store** out) {
     if (!out || !layers || !experts || !record_bytes || !slots) return zc_fail(ZC_INVALID_ARGUMENT, "empty expert cache");
+    if (!home_layers || home_layers > layers) return zc_fail(ZC_INVALID_ARGUMENT, "invalid number of record homes");
     const std::string name = policy ? policy : "";
     if (name != "clock" && name != "slru") return zc_fail(ZC_INVALID_ARGUMENT, "cache policy must be clock or slru");   // parse_cache_policy, storage.cpp:536-540
     auto s = std::make_unique<zc_hip_store>();
@@ -160,15 +166,16 @@ zc_status zc_hip_store_create_with_policy(zc_hip_ctx* ctx, uint32_t layers, uint
     s->layer_hits.assign(layers, 0); s->layer_misses.assign(layers, 0);
     const zc_status status = guarded([&] {
         const uint64_t home = uint64_t(experts) * s->stride;
-        for (uint32_t l = 0; l < layers; ++l) {
+        for (uint32_t l = 0; l < home_layers; ++l) {
             if (ctx) {
                 void* p = nullptr;
                 if (zc_hip_alloc_host(ctx, home, &p) != ZC_OK) throw std::runtime_error(zc_hip_last_error());
-                s->homes.push_back(static_cast<uint8_t*>(p));
+                s->owned_homes.push_back(static_cast<uint8_t*>(p));
             } else {
-                s->homes.push_back(new uint8_t[home]());
+                s->owned_homes.push_back(new uint8_t[home]());
             }
         }
+        for (uint32_t l = 0; l < layers; ++l) s->homes.push_back(s->owned_homes[l % home_layers]);   // layer l's records live in home l mod home_layers
         if (ctx) ZC_STORE_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));   // default priority
         provide_pool(s.get(), slots, 0);
         s->cache = std::make_unique<zc::SlotCache>(slots, record_bytes, hooks_of(s.get()), name == "slru" ? zc::SlotCache::SegmentedLRU : zc::SlotCache::Clock);
@@ -186,11 +193,11 @@ zc_status zc_hip_store_destroy(zc_hip_store* s) {
         for (hipEvent_t e : s->released) (void)hipEventDestroy(e);
         if (s->side) (void)hipStreamDestroy(s->side);
         if (s->pool) zc_hip_free(s->ctx, s->pool);
-        for (uint8_t* h : s->homes) zc_hip_free(s->ctx, h);
+        for (uint8_t* h : s->owned_homes) zc_hip_free(s->ctx, h);
         if (s->table) zc_hip_free(s->ctx, s->table);
         if (s->mirror) zc_hip_free(s->ctx, s->mirror);
     } else {
-        delete[] s->pool; for (uint8_t* h : s->homes) delete[] h; delete[] s->mirror;
+        delete[] s->pool; for (uint8_t* h : s->owned_homes) delete[] h; delete[] s->mirror;
     }
     delete s;
     return ZC_OK;
@@ -317,29 +324,59 @@ zc_status zc_hip_store_table_refresh(zc_hip_store* s) {
         return ZC_OK;
     });
 }
-zc_status zc_hip_store_table_observe(zc_hip_store* s, uint32_t layer, const int32_t* ids, uint32_t count) {
-    if (!s || !s->mirror) return zc_fail(ZC_LOGIC_ERROR, "the store has no record table");
-    if (layer >= s->layers || (!ids && count)) return zc_fail(ZC_OUT_OF_RANGE, "invalid layer");
+// What one finished launch read: per layer the distinct valid experts, each classified by what the table showed AT THE LAUNCH
+// (nothing below has changed it yet).  First every record that was read from a slot is leased, then the records read from
+// home are admitted, then all leases go: a miss can only take the slot of a record that this launch did not use.
+static zc_status observe_layers(zc_hip_store* s, uint32_t first_layer, uint32_t layers, const int32_t* ids, uint32_t per_layer) {
     return guarded([&] {
-        std::vector<int32_t> distinct(ids, ids + count);
-        std::sort(distinct.begin(), distinct.end());
-        distinct.erase(std::unique(distinct.begin(), distinct.end()), distinct.end());
-        for (const int32_t e : distinct) {
-            if (e < 0 || uint32_t(e) >= s->experts) throw std::out_of_range("invalid expert id");
-            const uint64_t key = key_of(s, layer, uint32_t(e));
-            const uint8_t* at = s->mirror[key];
-            const bool from_slot = at >= s->pool && at < s->pool + s->cache->capacity() * s->stride;
-            ++s->seen.reads;
-            if (from_slot) ++s->seen.slot_reads; else { ++s->seen.home_reads; s->seen.home_read_bytes += s->record_bytes; }
-            // Touch (a hit) or admit (a miss: the fill starts now, for the launches to come); no lease stays out.
+        std::vector<std::pair<uint64_t, uint32_t>> from_slots, from_home;   // (key, layer)
+        std::vector<int32_t> distinct;
+        for (uint32_t l = 0; l < layers; ++l) {
+            distinct.assign(ids + uint64_t(l) * per_layer, ids + uint64_t(l + 1) * per_layer);
+            std::sort(distinct.begin(), distinct.end());
+            distinct.erase(std::unique(distinct.begin(), distinct.end()), distinct.end());
+            for (const int32_t e : distinct) {
+                if (e < 0 || uint32_t(e) >= s->experts) throw std::out_of_range("invalid expert id");
+                const uint64_t key = key_of(s, first_layer + l, uint32_t(e));
+                const uint8_t* at = s->mirror[key];
+                const bool slot = at >= s->pool && at < s->pool + s->cache->capacity() * s->stride;
+                (slot ? from_slots : from_home).push_back({key, first_layer + l});
+            }
+        }
+        s->seen.reads += from_slots.size() + from_home.size();
+        s->seen.slot_reads += from_slots.size();
+        s->seen.home_reads += from_home.size(); s->seen.home_read_bytes += from_home.size() * s->record_bytes;
+        // ExpertCache::acquire's hit for everything that was read from a slot; the leases stay out while the misses are admitted, so
+        // that a victim is never a record this launch used, whatever the policy's own preferences
+        struct Held {   // whatever happens below, no lease stays out
+            zc::SlotCache* cache; std::vector<size_t> slots;
+            ~Held() { for (const size_t slot : slots) { try { cache->release(slot); } catch (...) {} } }
+        } leases{s->cache.get(), {}};
+        std::vector<size_t>& held = leases.slots;
+        held.reserve(from_slots.size() + from_home.size());
+        for (const auto& [key, layer] : from_slots) {
+            held.push_back(s->cache->acquire(key).slot);
+            ++s->layer_hits[layer];
+        }
+        for (const auto& [key, layer] : from_home) {   // acquire's miss (or a join to a fill still in flight): the fill serves later launches
             zc::SlotCache::Lease lease{};
             try { lease = s->cache->acquire(key); }
-            catch (const std::runtime_error&) { ++s->seen.not_admitted; continue; }   // every slot is still loading: the record stays at home for now
+            catch (const std::runtime_error&) { ++s->seen.not_admitted; continue; }   // no slot to take (all used by this launch, or loading): the record stays at home
             if (lease.acquisition == zc::SlotCache::NewMiss) ++s->layer_misses[layer]; else ++s->layer_hits[layer];
-            s->cache->release(lease.slot);
+            held.push_back(lease.slot);
         }
         return ZC_OK;
     });
+}
+zc_status zc_hip_store_table_observe(zc_hip_store* s, uint32_t layer, const int32_t* ids, uint32_t count) {
+    if (!s || !s->mirror) return zc_fail(ZC_LOGIC_ERROR, "the store has no record table");
+    if (layer >= s->layers || (!ids && count)) return zc_fail(ZC_OUT_OF_RANGE, "invalid layer");
+    return observe_layers(s, layer, 1, ids, count);
+}
+zc_status zc_hip_store_table_observe_layers(zc_hip_store* s, const int32_t* ids, uint32_t per_layer) {
+    if (!s || !s->mirror) return zc_fail(ZC_LOGIC_ERROR, "the store has no record table");
+    if (!ids && per_layer) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");
+    return observe_layers(s, 0, s->layers, ids, per_layer);
 }
 zc_status zc_hip_store_table_stats(const zc_hip_store* s, zc_store_table_stats* out) {
     if (!s || !out) return zc_fail(ZC_INVALID_ARGUMENT, "null argument");

@@ -86,12 +86,13 @@ class Store:
 
     ACQUISITIONS = ("new_miss", "ready_hit", "loading_join")
 
-    def __init__(self, ctx, layers, experts, record_bytes, slots, policy="clock"):
+    def __init__(self, ctx, layers, experts, record_bytes, slots, policy="clock", home_layers=None):
         self.lib = load_library()
         self.ctx, self.layers, self.experts, self.record_bytes = ctx, layers, experts, record_bytes
         self.handle = C.c_void_p()
-        self._check(self.lib.zc_hip_store_create_with_policy(ctx.handle if ctx else None, C.c_uint32(layers), C.c_uint32(experts),
-                                                             C.c_uint64(record_bytes), C.c_uint64(slots), policy.encode(), C.byref(self.handle)))
+        self._check(self.lib.zc_hip_store_create_shared_homes(ctx.handle if ctx else None, C.c_uint32(layers), C.c_uint32(experts),
+                                                              C.c_uint64(record_bytes), C.c_uint64(slots), policy.encode(),
+                                                              C.c_uint32(home_layers or layers), C.byref(self.handle)))
 
     def _check(self, status):
         if status:
@@ -185,6 +186,11 @@ class Store:
     def table_observe(self, layer, ids):
         ids = np.ascontiguousarray(ids, np.int32)
         self._check(self.lib.zc_hip_store_table_observe(self.handle, C.c_uint32(layer), ids.ctypes.data_as(C.c_void_p), C.c_uint32(ids.size)))
+
+    def table_observe_layers(self, ids):
+        """ids [layers][per_layer]: what one launch through all layers chose."""
+        ids = np.ascontiguousarray(ids, np.int32).reshape(self.layers, -1)
+        self._check(self.lib.zc_hip_store_table_observe_layers(self.handle, ids.ctypes.data_as(C.c_void_p), C.c_uint32(ids.shape[1])))
 
     def table_stats(self):
         st = StoreTableStats()

@@ -37,7 +37,7 @@ def record_stride(ctx, cfg):
 class LayerWeights:
     """Device buffers of one layer plus the zc_moe_layer that points at them."""
 
-    def __init__(self, ctx, cfg, seed, skew=None, records=None):
+    def __init__(self, ctx, cfg, seed, skew=None, records=None, keep_records=False):
         H, E = cfg.hidden, cfg.experts
         self.ctx, self.cfg, self.seed = ctx, cfg, seed
         self.stride = record_stride(ctx, cfg)
@@ -49,7 +49,8 @@ class LayerWeights:
         ctx.synth_normal_bf16(self.router, E * H, seed * 16 + 1, sigma)
         ctx.synth_normal_bf16(self.shared_gate, H, seed * 16 + 2, sigma)
         ctx.synth_records(cfg, self.shared_record, self.shared_record.nbytes, 1, seed * 16 + 3, shared=True)
-        ctx.synth_records(cfg, self.records, self.stride, E, (seed * 16 + 4) * 4096)
+        if not keep_records:   # (keep_records: the buffer already holds another layer's records, which this layer shares)
+            ctx.synth_records(cfg, self.records, self.stride, E, (seed * 16 + 4) * 4096)
         self.offsets_host = None
         if skew is not None:
             kind, value = skew
@@ -87,17 +88,20 @@ class StoreBackedStack:
     leases for the selected experts (fills on the store's side stream), per-expert gate/up + down into the expert's
     slots, shared expert, weighted combine; leases are released once the step's GPU work has finished."""
 
-    def __init__(self, ctx, cfg, seeds, skew, slots):
+    def __init__(self, ctx, cfg, seeds, skew, slots, home_layers=None):
+        """home_layers < len(seeds): layer l shares its records' home with layer l - home_layers (routers, shared experts
+        and router offsets stay every layer's own), for hosts that cannot pin all records."""
         from .hip import Store, DevBuf
         self.ctx, self.cfg = ctx, cfg
-        self.store = Store(ctx, len(seeds), cfg.experts, ctx.record_bytes(cfg), slots)
+        home_layers = home_layers or len(seeds)
+        self.store = Store(ctx, len(seeds), cfg.experts, ctx.record_bytes(cfg), slots, home_layers=home_layers)
         assert self.store.stride == record_stride(ctx, cfg)
         self.layers = []
         for l, seed in enumerate(seeds):
             home = self.store.lib.zc_hip_store_backing(self.store.handle, l, 0)
             # the generator kernel writes the records straight into their pinned-host home (mapped into the GPU)
             records = DevBuf(ctx, home, cfg.experts * self.store.stride)
-            self.layers.append(LayerWeights(ctx, cfg, seed, skew, records=records))
+            self.layers.append(LayerWeights(ctx, cfg, seed, skew, records=records, keep_records=l >= home_layers))
         ctx.finish()
 
     def close(self):

@@ -317,4 +317,51 @@ __device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t to
     if (lane < topk) weights[lane] = v * inverse;
 }
 
+// The same for up to N rows that lie apart (rows[t], t < count; `words` 8-byte words each) into consecutive LDS rows
+// of `words` words: the loads of all rows are in flight together, so an entry's rows cost one latency, not one each.
+template <int N>
+__device__ __forceinline__ void stage_copy_rows(const uint64_t* const (&rows)[N], int count, uint32_t words, uint64_t* dst) {
+    for (uint32_t j = threadIdx.x; j < words; j += blockDim.x) {
+        uint64_t v[N];
+#pragma unroll
+        for (int t = 0; t < N; ++t) v[t] = t < count ? __hip_atomic_load(rows[t] + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+#pragma unroll
+        for (int t = 0; t < N; ++t)
+            if (t < count) dst[uint32_t(t) * words + j] = v[t];
+    }
+}
+// Rows of fp32 values that lie apart (rows[t], t < count; `pairs` pairs of values each) as BF16 into consecutive LDS
+// rows of `pairs` dwords, all rows' loads in flight together; transform(t, a, b) may rescale a pair of row t first.
+// Returns nonzero if any value had low mantissa bits (see stage_bf16).
+template <int N, class Transform>
+__device__ __forceinline__ int stage_bf16_rows(const float* const (&rows)[N], int count, uint32_t pairs, uint32_t* dst, Transform transform) {
+    int inexact = 0;
+    for (uint32_t j = threadIdx.x; j < pairs; j += blockDim.x) {
+        uint64_t v[N];
+#pragma unroll
+        for (int t = 0; t < N; ++t)
+            v[t] = t < count ? __hip_atomic_load(reinterpret_cast<const uint64_t*>(rows[t]) + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+#pragma unroll
+        for (int t = 0; t < N; ++t)
+            if (t < count) {
+                float a = __uint_as_float(uint32_t(v[t])), b = __uint_as_float(uint32_t(v[t] >> 32));
+                transform(t, a, b);
+                const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+                inexact |= ((ua | ub) & 0xffffu) != 0;
+                dst[uint32_t(t) * pairs + j] = (ua >> 16) | (ub & 0xffff0000u);
+            }
+    }
+    return inexact;
+}
+
+// Which pass of its tile item q of an entry is (tile = q / passes).  The waves of a workgroup take every waves-th item, so
+// with a pass count that divides the wave count a wave would meet the same pass -- the same tokens -- in all its items, and
+// the wave that holds a token with many unsafe blocks would do all of that token's literal chains while the others wait
+// for it at the end of the phase; the pass index is therefore rotated from tile to tile.
+__device__ __forceinline__ uint32_t pass_of_item(uint32_t q, uint32_t passes, uint32_t waves) {
+    const uint32_t tile = q / passes, base = q % passes;
+    if (passes == 1 || waves % passes != 0) return base;
+    return (base + tile / (waves / passes)) % passes;
+}
+
 }  // namespace zc

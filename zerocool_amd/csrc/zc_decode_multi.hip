@@ -329,7 +329,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                 const uint64_t* off = routed ? p.ro : p.so;
                 const uint32_t passes = uint32_t(na + PT - 1) / PT;
                 for (uint32_t item = at + wave; item < seg_end; item += kMultiWaves) {
-                    const uint32_t tile = (item - first) / passes, pass = (item - first) % passes;
+                    const uint32_t tile = (item - first) / passes, pass = pass_of_item(item - first, passes, kMultiWaves);
                     const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
                     const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
@@ -367,13 +367,15 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                 const int na = slots_of(ei, all, routed, e);
                 __syncthreads();   // the previous segment's tiles have read their images
                 // the slots' activations (packed BF16 rows of I elements) into LDS, then their images
+                {
+                    const uint64_t* rows[MT];
 #pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    if (t >= na) break;
-                    const uint32_t sl = uint32_t(all[t]);
-                    const uint64_t* from = sl < n ? reinterpret_cast<const uint64_t*>(p.act) + uint64_t(sl) * I / 4
-                                                  : reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(sl - n) * I / 4;
-                    stage_copy<2>(from, I / 4, reinterpret_cast<uint64_t*>(ah + uint32_t(t) * I));
+                    for (int t = 0; t < MT; ++t) {
+                        const uint32_t sl = uint32_t(all[t]);
+                        rows[t] = sl < n ? reinterpret_cast<const uint64_t*>(p.act) + uint64_t(sl) * I / 4
+                                         : reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(sl - n) * I / 4;
+                    }
+                    stage_copy_rows(rows, na, I / 4, reinterpret_cast<uint64_t*>(ah));
                 }
                 __syncthreads();
                 xint_prepare_batch([&](uint32_t t) { return LdsBf16{ah + t * I}; }, uint32_t(na), LI, lds + lp.img_d);
@@ -381,7 +383,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                 const uint64_t* off = routed ? p.ro : p.so;
                 const uint32_t passes = uint32_t(na + PT - 1) / PT;
                 for (uint32_t item = at + wave; item < seg_end; item += kMultiWaves) {
-                    const uint32_t pass = (item - first) % passes;
+                    const uint32_t pass = pass_of_item(item - first, passes, kMultiWaves);
                     const uint32_t row = ((item - first) / passes) * 16 + col;
                     const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);

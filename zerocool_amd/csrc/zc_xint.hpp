@@ -35,6 +35,18 @@ struct XintLayout {
     __host__ __device__ uint32_t bytes() const { return (planes_bytes() + info_bytes() + mask_bytes() + 15) / 16 * 16; }
 };
 
+// The three digit sums of a block recombined, d0 + 2^7 d1 + 2^14 d2, by Horner's rule in two shift-and-add instructions.
+// (The empty statement keeps the compiler from regrouping the sum into two shifts and a three-operand add; the instructions
+// themselves are the compiler's, so it still places the wait states a read of matrix-core results needs.)
+__device__ __forceinline__ int xint_digits(const v4i r) {
+    int t = int((uint32_t(r[2]) << 7) + uint32_t(r[1]));
+    asm("" : "+v"(t));
+    return int((uint32_t(t) << 7) + uint32_t(r[0]));
+}
+
+// One of a dword's two BF16 values as fp32, in one byte-permute: select 0x03020c0c takes the upper one, 0x01000c0c the lower.
+__device__ __forceinline__ float xint_bf16_of(uint32_t pair, uint32_t select) { return __uint_as_float(__builtin_amdgcn_perm(pair, pair, select)); }
+
 // Byte t of a lane's 16-byte operand holds block element kOrder[t]: the order in which
 // (w & 0x0f0f0f0f), ((w >> 4) & 0x0f0f0f0f) of the block's two code words lay nibbles out.
 __device__ __forceinline__ uint32_t xint_element_of_byte(uint32_t t) {
@@ -251,7 +263,7 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
     for (int t = 0; t < PT; ++t)
 #pragma unroll
         for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
-    const uint32_t shamt = (lane & 32u) ? 0u : 16u;   // group 2d + (G >> 1): low half for G < 2
+    const uint32_t half = (lane & 32u) ? 0x03020c0cu : 0x01000c0cu;   // group 2d + (G >> 1): the low BF16 of a dword for G < 2
     // A operand: row (c,p) of lane group G holds digit plane p of block 2c (+1) when c == G, zeros otherwise
     const bool live = (c_a == G) && p_a < 3;
     const uint32_t a_first = live ? 2 * G * 48 + p_a * 16 : L.blocks() * 48, a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
@@ -279,8 +291,8 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
                     const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
                     const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, zero, 0, 0, 0);
                     const float4 fi = *reinterpret_cast<const float4*>(info + 8 * d + 2 * G);   // {2^e, sum} of blocks 2G, 2G+1
-                    dot[j][0] = float(r0[0] + (r0[1] << 7) + (r0[2] << 14)) * fi.x; bsum[j][0] = fi.y;
-                    dot[j][1] = float(r1[0] + (r1[1] << 7) + (r1[2] << 14)) * fi.z; bsum[j][1] = fi.w;
+                    dot[j][0] = float(xint_digits(r0)) * fi.x; bsum[j][0] = fi.y;
+                    dot[j][1] = float(xint_digits(r1)) * fi.z; bsum[j][1] = fi.w;
                 }
             }
             // pass 2: blocks 8d + 2G + h of spans d0 .. d0+7 sit in mask words d0/4, d0/4 + 1
@@ -301,7 +313,7 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
 #pragma unroll
             for (int j = 0; j < R; ++j) {
                 {
-                    const float scale = __uint_as_float((sd[j] << shamt) & 0xffff0000u), bias = __uint_as_float((bd[j] << shamt) & 0xffff0000u);
+                    const float scale = xint_bf16_of(sd[j], half), bias = xint_bf16_of(bd[j], half);
                     acc[t][j & 3][0] += scale * dot[j][0] + bsum[j][0] * bias;
                     acc[t][j & 3][1] += scale * dot[j][1] + bsum[j][1] * bias;
                 }
@@ -366,19 +378,26 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
 #define ZC_TILE_LOAD(p, i) ldg_u4(p, i)
 #endif
 // The literal fp32 chain of one block (reference: qwen.metal:52-57) from the block's two raw code words (nibble i of word w
-// is element 8 w + i) and the block's sixteen BF16 inputs in LDS.  Written as a loop over the four quads so that it is
-// small in code and registers: it runs inside the tile engines, whose registers are full.
+// is element 8 w + i) and the block's sixteen BF16 inputs in LDS.  The four quads' nested sums do not depend on each other:
+// all sixteen inputs are read at once and the four chains run side by side, then the quad sums are added in order -- one
+// LDS latency and a chain of eight dependent operations instead of four latencies and twenty.
 __device__ __forceinline__ float xint_literal_block(const uint16_t* x_block, uint32_t w_lo, uint32_t w_hi) {
-    float dot = 0;
-#pragma unroll 1
-    for (int quad = 0; quad < 4; ++quad) {
-        const uint2 xv = *reinterpret_cast<const uint2*>(x_block + 4 * quad);
-        const uint32_t nib = ((quad & 2 ? w_hi : w_lo) >> (16 * (quad & 1))) & 0xffffu;
-        const float a = __uint_as_float(xv.x << 16), c = __uint_as_float(xv.x & 0xffff0000u);
-        const float d = __uint_as_float(xv.y << 16), e = __uint_as_float(xv.y & 0xffff0000u);
+    const uint4 xa = *reinterpret_cast<const uint4*>(x_block), xb = *reinterpret_cast<const uint4*>(x_block + 8);
+    const uint32_t xw[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+    float quad[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t w = q & 2 ? w_hi : w_lo, x0 = xw[2 * q], x1 = xw[2 * q + 1];
+        const int at = 16 * (q & 1);
+        const float a = __uint_as_float(x0 << 16), c = __uint_as_float(x0 & 0xffff0000u);
+        const float d = __uint_as_float(x1 << 16), e = __uint_as_float(x1 & 0xffff0000u);
         // BF16-valued inputs times 4-bit codes are exact products: a fused multiply-add equals the reference's multiply and add
-        dot += __builtin_fmaf(e, float(nib >> 12), __builtin_fmaf(d, float((nib >> 8) & 15u), __builtin_fmaf(c, float((nib >> 4) & 15u), a * float(nib & 15u))));
+        quad[q] = __builtin_fmaf(e, float((w >> (at + 12)) & 15u), __builtin_fmaf(d, float((w >> (at + 8)) & 15u),
+                  __builtin_fmaf(c, float((w >> (at + 4)) & 15u), a * float((w >> at) & 15u))));
     }
+    float dot = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dot += quad[q];
     return dot;
 }
 
@@ -407,7 +426,7 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
     for (int t = 0; t < NTOK; ++t)
 #pragma unroll
         for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
-    const uint32_t shamt = (lane & 32u) ? 0u : 16u;   // group 2d + (G >> 1): low half for G < 2
+    const uint32_t half = (lane & 32u) ? 0x03020c0cu : 0x01000c0cu;   // group 2d + (G >> 1): the low BF16 of a dword for G < 2
     const bool live = (c_a == G) && p_a < 3;
     const uint32_t a_first = live ? 2 * G * 48 + p_a * 16 : L.blocks() * 48, a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
     const uint32_t M = 0x0f0f0f0fu;
@@ -445,9 +464,8 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
                 const float4 fi = *reinterpret_cast<const float4*>(img[t] + info_at + d * 64);   // {2^e, sum} of blocks 2G, 2G+1
                 const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, zero, 0, 0, 0);
                 const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, zero, 0, 0, 0);
-                // digits recombined by Horner's rule: ((d2 << 7) + d1 << 7) + d0
-                dot[t][0] = float((((r0[2] << 7) + r0[1]) << 7) + r0[0]) * fi.x; bsum[t][0] = fi.y;
-                dot[t][1] = float((((r1[2] << 7) + r1[1]) << 7) + r1[0]) * fi.z; bsum[t][1] = fi.w;
+                dot[t][0] = float(xint_digits(r0)) * fi.x; bsum[t][0] = fi.y;
+                dot[t][1] = float(xint_digits(r1)) * fi.z; bsum[t][1] = fi.w;
             }
 #ifndef ZC_TIMING_NO_LITERAL
             if (__builtin_expect(literal_body, 0)) {
@@ -472,7 +490,7 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
                 }
             }
 #endif
-            const float scale = __uint_as_float((sdw[j] << shamt) & 0xffff0000u), bias = __uint_as_float((bdw[j] << shamt) & 0xffff0000u);
+            const float scale = xint_bf16_of(sdw[j], half), bias = xint_bf16_of(bdw[j], half);
 #pragma unroll
             for (int t = 0; t < NTOK; ++t) {
                 acc[t][j][0] += scale * dot[t][0] + bsum[t][0] * bias;
@@ -518,7 +536,7 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
     for (int t = 0; t < NTOK; ++t)
 #pragma unroll
         for (int m = 0; m < 4; ++m) { acc[t][m][0] = 0; acc[t][m][1] = 0; }
-    const uint32_t shamt = (lane & 32u) ? 0u : 16u;   // group 2d + (G >> 1): low half for G < 2
+    const uint32_t half = (lane & 32u) ? 0x03020c0cu : 0x01000c0cu;   // group 2d + (G >> 1): the low BF16 of a dword for G < 2
     const bool live = (c_a == G) && p_a < 3;
     const uint32_t a_first = live ? 2 * G * 48 + p_a * 16 : L.blocks() * 48, a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
     const uint32_t M = 0x0f0f0f0fu;
@@ -582,9 +600,8 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
             float dot[TG][2];
 #pragma unroll
             for (int t = 0; t < TG; ++t) {
-                // digits recombined by Horner's rule: ((d2 << 7) + d1 << 7) + d0
-                dot[t][0] = float((((r0[t][2] << 7) + r0[t][1]) << 7) + r0[t][0]) * fi[buf][t].x;
-                dot[t][1] = float((((r1[t][2] << 7) + r1[t][1]) << 7) + r1[t][0]) * fi[buf][t].z;
+                dot[t][0] = float(xint_digits(r0[t])) * fi[buf][t].x;
+                dot[t][1] = float(xint_digits(r1[t])) * fi[buf][t].z;
             }
             if (__builtin_expect(literal_body, 0)) {
                 // pending (token, block) pairs of this lane in this step: bit 2t + h; every lane takes its next one in turn
@@ -607,7 +624,7 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
                     }
                 }
             }
-            const float scale = __uint_as_float((sdw[j] << shamt) & 0xffff0000u), bias = __uint_as_float((bdw[j] << shamt) & 0xffff0000u);
+            const float scale = xint_bf16_of(sdw[j], half), bias = xint_bf16_of(bdw[j], half);
 #pragma unroll
             for (int t = 0; t < TG; ++t) {
                 acc[g * TG + t][j][0] += scale * dot[t][0] + fi[buf][t].y * bias;

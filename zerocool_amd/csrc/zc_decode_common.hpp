@@ -354,6 +354,15 @@ __device__ __forceinline__ int stage_bf16_rows(const float* const (&rows)[N], in
     return inexact;
 }
 
+// Workgroup wg's share [i0, i1) of a list of `total` items, cut at multiples of `waves` items.  Every entry of the tile
+// lists is a multiple of eight items long (a tile count times a pass count), so with the cuts on such multiples neither a
+// workgroup's range nor its part of any entry ends in a round in which some of its waves have no item.
+__device__ __forceinline__ void share_of_items(uint32_t wg, uint32_t nwg, uint32_t total, uint32_t waves, uint32_t& i0, uint32_t& i1) {
+    const uint32_t rounds = total / waves;
+    i0 = uint32_t(uint64_t(wg) * rounds / nwg) * waves;
+    i1 = wg + 1 == nwg ? total : uint32_t(uint64_t(wg + 1) * rounds / nwg) * waves;
+}
+
 // Which pass of its tile item q of an entry is (tile = q / passes).  The waves of a workgroup take every waves-th item, so
 // with a pass count that divides the wave count a wave would meet the same pass -- the same tokens -- in all its items, and
 // the wave that holds a token with many unsafe blocks would do all of that token's literal chains while the others wait

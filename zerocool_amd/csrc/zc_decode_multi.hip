@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
                 }
             }
             __syncthreads();
-            const int bad = stage_bf16<12>(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), []() {},
+            const int bad = stage_bf16<24>(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), []() {},
                 [&](uint32_t i, float& a, float& b) {
                     if (glue) { const float scale = gatev[(2 * i) / H]; a = bf(a * scale); b = bf(b * scale); }
                 });
@@ -318,7 +318,8 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
         {
             // items = (expert index, tile, pass), passes of a tile adjacent; expert ei owns items [tiles * cum[ei], tiles * cum[ei + 1])
             const uint32_t tiles = I / 8, total = tiles * uint32_t(cum[U + 1]);
-            const uint32_t i0 = uint32_t(uint64_t(wg) * total / nwg), i1 = uint32_t(uint64_t(wg + 1) * total / nwg);
+            uint32_t i0, i1;
+            share_of_items(wg, nwg, total, kMultiWaves, i0, i1);
             uint32_t ei = 0;
             while (ei < U && tiles * uint32_t(uniform(cum[ei + 1])) <= i0) ++ei;
             for (uint32_t at = i0; at < i1; ++ei) {
@@ -357,7 +358,8 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
         // ---------------- phase D: down tiles, one contiguous range of (expert, row tile) per workgroup ----------------
         {
             const uint32_t row_tiles = H / 16, total = row_tiles * uint32_t(cum[U + 1]);
-            const uint32_t i0 = uint32_t(uint64_t(wg) * total / nwg), i1 = uint32_t(uint64_t(wg + 1) * total / nwg);
+            uint32_t i0, i1;
+            share_of_items(wg, nwg, total, kMultiWaves, i0, i1);
             uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
             uint32_t ei = 0;
             while (ei < U && row_tiles * uint32_t(uniform(cum[ei + 1])) <= i0) ++ei;

@@ -316,7 +316,8 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
             const uint32_t cut = q8_shared ? 4u : 1u, routed_passes = uint32_t(cum[U]);
             auto gcum = [&](uint32_t i) { const uint32_t c = uint32_t(uniform(cum[i])); return i <= U ? c : routed_passes + cut * (c - routed_passes); };
             const uint32_t tiles = I / 8, total = tiles * gcum(NE);
-            const uint32_t i0 = uint32_t(uint64_t(wg) * total / nwg), i1 = uint32_t(uint64_t(wg + 1) * total / nwg);
+            uint32_t i0, i1;
+            share_of_items(wg, nwg, total, kWideWaves, i0, i1);
             uint32_t ei = 0;
             while (ei + 1 < NE && tiles * gcum(ei + 1) <= i0) ++ei;
             for (uint32_t at = i0; at < i1; ++ei) {
@@ -383,7 +384,8 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
         // ---------------- phase D: down tiles; items (entry, row tile, pass), one contiguous range per workgroup ----------------
         {
             const uint32_t row_tiles = H / 16, total = row_tiles * uint32_t(cum[NE]);
-            const uint32_t i0 = uint32_t(uint64_t(wg) * total / nwg), i1 = uint32_t(uint64_t(wg + 1) * total / nwg);
+            uint32_t i0, i1;
+            share_of_items(wg, nwg, total, kWideWaves, i0, i1);
             uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
             uint32_t ei = 0;
             while (ei + 1 < NE && row_tiles * uint32_t(uniform(cum[ei + 1])) <= i0) ++ei;

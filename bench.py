@@ -62,10 +62,10 @@ def write_traffic_file(fetch_dir, write_dir):
     import collections, csv, glob
     def averages(folder, counter):
         values = collections.defaultdict(list)
-        for path in glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True):
-            for row in csv.DictReader(open(path)):
-                if row["Counter_Name"] == counter:
-                    values[row["Kernel_Name"]].append(float(row["Counter_Value"]))
+        files = glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True)
+        for row in csv.DictReader(open(max(files, key=os.path.getmtime))):   # a folder that was used before: the latest run's file
+            if row["Counter_Name"] == counter:
+                values[row["Kernel_Name"]].append(float(row["Counter_Value"]))
         pick = lambda word: [v for k, v in values.items() if word in k]
         copies, = pick("copyBuffer")          # the runtime's copy kernel also serves small copies: the 1 GiB one is the largest
         kernel, = pick("decode_stack_kernel")
@@ -74,7 +74,7 @@ def write_traffic_file(fetch_dir, write_dir):
     write, write_copy, _ = averages(write_dir, "WRITE_SIZE")
     read_bytes = fetch * (1048576.0 / fetch_copy) * 1024
     written_bytes = write * (1048576.0 / write_copy) * 1024
-    record = {"kernel": "zc::decode_stack_kernel<1>", "workload": "48 F-shape layers, batch 1 (the default run of bench.py)",
+    record = {"kernel": "zc::decode_stack_kernel<1, false>", "workload": "48 F-shape layers, batch 1 (the default run of bench.py)",
               "dispatches_averaged": calls, "FETCH_SIZE_KiB": fetch, "FETCH_SIZE_KiB_of_1GiB_copy": fetch_copy,
               "WRITE_SIZE_KiB": write, "WRITE_SIZE_KiB_of_1GiB_copy": write_copy,
               "hbm_bytes_read": int(read_bytes), "hbm_bytes_written": int(written_bytes),

@@ -142,8 +142,10 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
 #pragma unroll
                     for (int i = 0; i < kRing; ++i) early[i] = ldg_u4(wr, wave * kRing + i);
                 } else if (blk < H / 16) {
+                    // (the staging lanes side by side: word pair w * H/16 + blk, so that a load covers four whole cache lines --
+                    // a lane fetching its own block's eight pairs touches thirty-two; the blocks are built from the BF16 copy)
 #pragma unroll
-                    for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + blk * 8 + w);
+                    for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + uint32_t(w) * (H / 16) + blk);
                 }
             } else if (keep_in_flight) {
 #pragma unroll
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 if (blk < H / 16 && stale())
                     bar.until([&]() {
 #pragma unroll
-                        for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + own * 8 + w);
+                        for (int w = 0; w < 8; ++w) v[w] = ZC_LD(row + (side ? uint32_t(w) * (H / 16) + own : own * 8 + uint32_t(w)));
                         return !stale();
                     });
                 // every workgroup has taken what it needed from the buffers this layer is about to overwrite
@@ -215,9 +217,14 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     packed[w] = (ua >> 16) | (uc & 0xffff0000u);
                 }
                 if (low) atomicOr(p.status, 4);   // inputs must be BF16-valued
-                uint4* copy = reinterpret_cast<uint4*>(xh + blk * 16);
-                copy[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]); copy[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
-                if (!side) xint_prepare_block(block, LH, lds + lp.img_rg, blk);
+                if (side) {
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) reinterpret_cast<uint32_t*>(xh)[uint32_t(w) * (H / 16) + blk] = packed[w];
+                } else {
+                    uint4* copy = reinterpret_cast<uint4*>(xh + blk * 16);
+                    copy[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]); copy[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
+                    xint_prepare_block(block, LH, lds + lp.img_rg, blk);
+                }
             }
             if (tid < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid] = gate_piece;
             lds_barrier();
@@ -454,20 +461,32 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 constexpr int PER = int(sizeof(cand) / sizeof(float));
                 const float ninf = __uint_as_float(0xff800000u);
                 if constexpr (NT == 1) {
+                    // polled with the lanes side by side (word i * 64 + lane: four whole cache lines per load; lane-major, as
+                    // the selection wants its candidates, a load touched thirty-two), turned lane-major through LDS
                     uint64_t w[PER];
                     bar.until([&]() {
                         uint32_t bad = 0;
 #pragma unroll
                         for (int i = 0; i < PER; ++i) {
-                            const uint32_t e = lane * per + i;
-                            w[i] = (uint32_t(i) < per && e < E) ? ZC_LD(p.tlogits + e) : (uint64_t(tag) << 32) | 0xff800000u;
+                            const uint32_t e = uint32_t(i) * 64 + lane;
+                            w[i] = e < E ? ZC_LD(p.tlogits + e) : (uint64_t(tag) << 32) | 0xff800000u;
                         }
 #pragma unroll
                         for (int i = 0; i < PER; ++i) bad |= uint32_t(w[i] >> 32) ^ tag;
-                        return bad == 0;
+                        return __ballot(bad != 0) == 0;
                     });
+                    float* turned = reinterpret_cast<float*>(experts);   // E words: the expert list is built later, the selection's scratch used after this
+                    auto wave_order = [&]() {
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    };
 #pragma unroll
-                    for (int i = 0; i < PER; ++i) cand[i] = __uint_as_float(uint32_t(w[i]));
+                    for (int i = 0; i < PER; ++i) if (uint32_t(i) * 64 + lane < E) turned[uint32_t(i) * 64 + lane] = __uint_as_float(uint32_t(w[i]));
+                    wave_order();
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) cand[i] = (uint32_t(i) < per && lane * per + i < E) ? turned[lane * per + i] : ninf;
+                    wave_order();
                 } else {
 #pragma unroll
                     for (int i = 0; i < PER; ++i) {
@@ -689,28 +708,38 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         __builtin_amdgcn_wave_barrier();
                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                     };
+                    // (the first poll goes out before the tile's weights are requested: loads come back in the order they were sent)
+                    const int32_t from = uniform(spec[slot]);   // the prediction pass's row of the same expert, or this layer's own
+                    const uint64_t* words = reinterpret_cast<const uint64_t*>(from >= 0 ? p.tspec + uint64_t(from) * I : p.tact + uint64_t(slot) * I) + lane;
+                    uint64_t w[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) w[i] = ZC_LD(words + i * 64);
                     auto prologue = [&]() {
                         if (lane < LI.mask_bytes() / 4) reinterpret_cast<uint32_t*>(image + LI.planes_bytes() + LI.info_bytes())[lane] = 0;
                         if (lane < 4) reinterpret_cast<uint32_t*>(image + LI.blocks() * 48)[lane] = 0;
                         wave_sync();
-                        for (uint32_t b = lane; b < I / 16; b += 64) {
-                            const int32_t from = uniform(spec[slot]);   // the prediction pass's row of the same expert, or this layer's own
-                            const uint64_t* words = reinterpret_cast<const uint64_t*>((from >= 0 ? p.tspec + uint64_t(from) * I : p.tact + uint64_t(slot) * I) + b * 16);
-                            uint64_t w[8];
+                        {
+                            // The slot's 1024 tagged words, polled with the lanes side by side (word pair i * 64 + lane: a load
+                            // instruction covers four whole cache lines; with a lane fetching its own block of sixteen it
+                            // touched sixty-four), packed into the BF16 copy in LDS, from which every lane then builds the image
+                            // of one block.
+                            bool again = false;
                             bar.until([&]() {
                                 uint32_t bad = 0;
+                                if (again) {
 #pragma unroll
-                                for (int i = 0; i < 8; ++i) w[i] = ZC_LD(words + i);
+                                    for (int i = 0; i < 8; ++i) w[i] = ZC_LD(words + i * 64);
+                                }
+                                again = true;
 #pragma unroll
                                 for (int i = 0; i < 8; ++i) bad |= ((uint32_t(w[i]) ^ tag) | (uint32_t(w[i] >> 32) ^ tag)) & 0xffffu;
-                                return bad == 0;
+                                return __ballot(bad != 0) == 0;   // the whole row, for every lane
                             });
-                            uint4* copy = reinterpret_cast<uint4*>(copy_row + b * 16);
-                            uint32_t packed[8];
+                            uint32_t* copy = reinterpret_cast<uint32_t*>(copy_row) + lane;
 #pragma unroll
-                            for (int i = 0; i < 8; ++i) packed[i] = (uint32_t(w[i]) >> 16) | (uint32_t(w[i] >> 32) & 0xffff0000u);
-                            copy[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]); copy[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
-                            xint_prepare_block(LdsBf16{copy_row}, LI, image, b);   // from the copy just written: fewer registers held
+                            for (int i = 0; i < 8; ++i) copy[i * 64] = (uint32_t(w[i]) >> 16) | (uint32_t(w[i] >> 32) & 0xffff0000u);
+                            wave_sync();
+                            xint_prepare_block(LdsBf16{copy_row}, LI, image, lane);
                         }
                         wave_sync();
                     };

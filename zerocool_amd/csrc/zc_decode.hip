@@ -58,7 +58,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };   // after the slowest wave of the workgroup
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
-    if (tid == 0) { misc[10] = 0; misc[11] = 0; }   // the router chain's hand-off word and the ids-ready word: no tag is 0
+    if (tid == 0) { misc[10] = 0; misc[11] = 0; misc[12] = 0; misc[13] = 0; misc[14] = 0; }   // the router chain's hand-off word, the ids-ready word, the staging waves' image-ready words: no tag is 0
     // SwiGLU of a finished gate/up tile (gate rows in columns 0-7, up rows in 8-15), stored as packed BF16 pairs:
     // the lane of an even row writes rows r and r+1 of activation row `slot_row` as one word.
     auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {
@@ -102,6 +102,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         uint4 early[kRing];
 #pragma unroll
         for (int i = 0; i < kRing; ++i) early[i] = make_uint4(0, 0, 0, 0);
+        // One token, a workgroup that owns a router unit, guesses at hand: its guessed gate/up tiles go to the waves AFTER the
+        // router's (the staging waves and the ones behind them), which start them as soon as the image is complete -- told
+        // so through flag words in LDS, not by a workgroup barrier, for which the router's waves would have to finish their
+        // chains first (a tile is then 2.6 us late, and the layer with it: the gate/up burst is what the routing waits for).
+        const bool apart = NT == 1 && !MIXED && pred != nullptr && segmented && wg < (E + 3) / 4 && 64 * router_segments + H / 16 <= kDecodeThreads &&
+                           (k * (I / 8)) % nwg == 0 && (E + 3) / 4 + I / 8 <= nwg && kDecodeWaves - router_segments >= k * (I / 8) / nwg && (H / 16 + 63) / 64 <= 3;
         if constexpr (NT == 1) {
             // One token: thread b fetches the sixteen values of block b, applies the glue's scale, writes the BF16 copy and
             // builds the block's image pieces straight from registers; the shared gate row rides along.  After the first
@@ -229,6 +235,10 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             if (tid < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[tid] = gate_piece;
             lds_barrier();
             if (side && blk < H / 16) xint_prepare_block(LdsBf16{xh}, LH, lds + lp.img_rg, blk);   // from the BF16 copy, beside the router's waves; the tiles come after a barrier
+            if (apart && wave >= router_segments && wave < router_segments + (H / 16 + 63) / 64) {   // this staging wave's part of the image is complete
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                if (lane == 0) __hip_atomic_store(misc + 12 + (wave - router_segments), int32_t(tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
         } else {
             {
                 uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
@@ -445,8 +455,22 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
         }
-        clock_all();
-        if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the routing below polls the logits themselves
+        if (apart) {
+            clock();
+            if (wave >= router_segments) {   // the tile waves: until every staging wave has said that its blocks are built
+                const uint32_t staging = (H / 16 + 63) / 64;
+                for (uint32_t i = 0; i < (1u << 22); ++i) {
+                    bool ready = true;
+                    for (uint32_t w = 0; w < staging; ++w) ready = ready && uint32_t(__hip_atomic_load(misc + 12 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) == tag;
+                    if (ready) break;
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            }
+        } else {
+            clock_all();
+            if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the routing below polls the logits themselves
+        }
         refresh();
         clock();
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
@@ -584,6 +608,10 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     if (!pred || wave == 0) continue;
                     far_end = !q8_shared && (k * tiles) % nwg == 0 && tiles <= nwg;
                     first = wg + nwg * (wave - 1); stride = nwg * (kDecodeWaves - 1);
+                    if (apart) {   // (this workgroup has no shared tile: those go to the far end)
+                        if (wave < router_segments) continue;
+                        first = wg + nwg * (wave - router_segments);
+                    }
                     units = far_end ? k * tiles + nwg : k * tiles + tiles * shared_cut;
                 } else {
                     if (wave != 0) {

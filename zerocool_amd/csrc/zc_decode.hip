@@ -531,7 +531,10 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                     const int32_t mine = lane < k ? ids[lane] : -1;
                     int32_t from = -1;
-                    if (pred) for (uint32_t j = 0; j < k; ++j) { const int32_t pj = __builtin_amdgcn_readlane(guess, int(j)); if (pj == mine && mine >= 0) from = int32_t(j); }
+                    if (pred)
+                        for (uint32_t j0 = 0; j0 < k; j0 += 4)   // (lanes from k on hold no guess: -1 matches nothing)
+#pragma unroll
+                            for (uint32_t j = j0; j < j0 + 4; ++j) { const int32_t pj = __builtin_amdgcn_readlane(guess, int(j & 63u)); if (pj == mine && mine >= 0) from = int32_t(j); }
                     const uint64_t missing = __ballot(lane < k && from < 0);
                     if (lane < k) {
                         spec[lane] = from;

@@ -207,9 +207,9 @@ __device__ __forceinline__ void stage_copy(const uint64_t* src, uint32_t count, 
 // found by a binary search over the bits of an order-preserving integer key (one compare and one ballot per step,
 // stopping as soon as exactly k lanes remain); k elements are then known to be at least that large, so the final top-k
 // lies among the elements at or above it: usually k to 2k of them.  They are gathered in ascending id order (`scratch`,
-// 128 words of LDS owned by this wave), one per lane, and each counts the candidates that beat it: larger value, or
-// equal value and lower id.  More than 64 candidates (masses of equal logits) or fewer than k valid lanes take the
-// picks one by one as before.
+// 128 words of LDS owned by this wave), one per lane, and each counts the candidates that beat it (larger value, or
+// equal value and lower id): that count is its slot.  More than 64 candidates (masses of equal logits) or fewer than k
+// valid lanes take the picks one by one.
 //
 // fetch(cand, per) fills the lane's logits (-inf where it has no expert); ready() runs once the ids are final, before the
 // softmax weights are formed.
@@ -244,13 +244,14 @@ __device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t to
             }
             // candidates in ascending id order: lower lanes first, then the lane's own slots
             const uint64_t below = (1ull << lane) - 1;
-            uint32_t before = 0, count = 0, mine = 0;
+            uint32_t before = 0, count = 0;
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
                 const uint64_t m = __ballot(key[i] >= bar);
                 before += uint32_t(__popcll(m & below)); count += uint32_t(__popcll(m));
             }
             if (count <= 64) {
+                uint32_t mine = 0;
 #pragma unroll
                 for (int i = 0; i < PER; ++i)
                     if (key[i] >= bar) { scratch[before + mine] = key[i]; scratch[64 + before + mine] = lane * per + uint32_t(i); ++mine; }
@@ -258,23 +259,20 @@ __device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t to
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 const uint32_t k_mine = lane < count ? scratch[lane] : 0u, id_mine = lane < count ? scratch[64 + lane] : 0u;
+                // a candidate's slot is the number of candidates that beat it; as one 64-bit compare: the key above the
+                // inverted position (lanes from `count` on hold key 0, which beats nothing)
+                const uint64_t wide_mine = (uint64_t(k_mine) << 32) | (63u - lane);
                 uint32_t rank = 0;
-                for (uint32_t j = 0; j < count; ++j) {
-                    const uint32_t other = uint32_t(__builtin_amdgcn_readlane(int(k_mine), int(j)));
-                    rank += (other > k_mine || (other == k_mine && j < lane)) ? 1u : 0u;
-                }
-                if (lane < topk) { ids[lane] = -1; weights[lane] = ninf; }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                if (lane < count && rank < topk) {
+                for (uint32_t j = 0; j < count; j += 4)   // count <= 64, so lane j + 3 exists
+#pragma unroll
+                    for (uint32_t u = 0; u < 4; ++u) {
+                        const uint64_t other = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(k_mine), int(j + u)))) << 32) | (63u - (j + u));
+                        rank += other > wide_mine ? 1u : 0u;
+                    }
+                if (lane < count && rank < topk) {   // the slots are a permutation of 0 .. count-1: one owner each
                     ids[rank] = int32_t(id_mine);
                     weights[rank] = __uint_as_float(k_mine ^ ((k_mine >> 31) ? 0x80000000u : 0xffffffffu));   // the value back from its key
                 }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                if (lane < topk) score = weights[lane];
-                top = weights[0];
                 done = true;
             }
         }
@@ -305,6 +303,13 @@ __device__ __forceinline__ void route_token(Fetch fetch, uint32_t E, uint32_t to
     }
     ready();
     clock();
+    if (done) {   // the scores as the picks above would have left them
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (lane < topk) score = weights[lane];
+        top = weights[0];
+    }
     // softmax over the selected: reference lane l sums values 4l..4l+3 (qwen.metal:758-764)
     const float v = lane < topk ? exp32(score - top) : 0.0f;
     float s4 = 0;

@@ -69,6 +69,11 @@ __device__ __forceinline__ uint4 ldg_u4(const void* p, uint32_t index = 0) {
     const u32x4 v = as_global<u32x4>(p)[index];
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+__device__ __forceinline__ uint2 ldg_u2(const void* p, uint32_t index = 0) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 v = as_global<u32x2>(p)[index];
+    return make_uint2(v.x, v.y);
+}
 __device__ __forceinline__ uint16_t ldg_u16(const void* p, uint32_t index = 0) { return as_global<uint16_t>(p)[index]; }
 __device__ __forceinline__ uint32_t ldg_u32(const void* p, uint32_t index = 0) { return as_global<uint32_t>(p)[index]; }
 __device__ __forceinline__ float ldg_f32(const void* p, uint32_t index = 0) { return as_global<float>(p)[index]; }

@@ -116,8 +116,11 @@ __global__ __launch_bounds__(1024) void prefill_tiles_kernel(const int32_t* offs
 template <bool GATED>
 __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     __shared__ __align__(16) uint16_t a_s[2][kTileRowsMax * kPitch];
-    __shared__ __align__(16) uint16_t b_s[2][kTileCols * kPitch];
-    __shared__ float scale_s[2][kTileCols], bias_s[2][kTileCols], sum_s[2][kTileRowsMax];
+    // The scales and biases of the workgroup's 128 weight rows and the chain sums of its token rows, for every step, are
+    // brought in once (whole runs of consecutive bytes: fetched step by step they cost a cache access per row and step
+    // for two or four bytes each, more accesses than the codes and the token rows together).
+    extern __shared__ __align__(16) uint8_t meta_s[];
+    __shared__ uint32_t row_s[kTileRowsMax];
     const uint32_t tile = blockIdx.y;
     if (tile >= uint32_t(*p.tile_count)) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, j = lane & 15u, g4 = lane >> 4;
@@ -135,59 +138,75 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     const uint32_t a_pos2 = first + min(32u + (a_r & 15u), rows - 1);
     const uint32_t a_row2 = p.a_rows ? uint32_t(p.a_rows[a_pos2]) / p.a_div : a_pos2;
     const uint16_t* a_src2 = p.a + uint64_t(a_row2) * K + a_c * 8;
-    const uint32_t b_r = tid >> 1, b_h = tid & 1u;                       // weight row of the tile, half of the step (32 codes)
-    const uint32_t b_proj = GATED ? b_r >> 6 : 0u, b_n = n0 + (GATED ? (b_r & 63u) : b_r);
-    const uint8_t* b_src = record + p.off[b_proj * 3] + uint64_t(b_n) * (K / 2) + b_h * 16;
-    const uint32_t m_r = tid & 127u;                                     // metadata row (threads 0..127)
-    const uint32_t m_proj = GATED ? m_r >> 6 : 0u, m_n = n0 + (GATED ? (m_r & 63u) : m_r);
-    const uint16_t* s_src = reinterpret_cast<const uint16_t*>(record + p.off[m_proj * 3 + 1]) + uint64_t(m_n) * groups;
-    const uint16_t* o_src = reinterpret_cast<const uint16_t*>(record + p.off[m_proj * 3 + 2]) + uint64_t(m_n) * groups;
-    const uint32_t x_pos = first + min(tid - 128u < kTileRowsMax ? tid - 128u : 0u, rows - 1);   // threads 128..175: one row's group sums each
-    const uint32_t x_row = p.a_rows ? uint32_t(p.a_rows[x_pos]) / p.a_div : x_pos;
-    const float* x_src = p.asum + uint64_t(x_row) * groups;
+    // The wave's two column tiles (rows of the workgroup's 128 weight rows) for every block of sixteen token rows; gate/up:
+    // a gate tile and the up tile of the same rows.  The codes go from memory straight into the lanes that feed them to
+    // the matrix cores: lane (j, g4) holds codes 16 g4 .. 16 g4 + 15 of the step for weight row j of each tile (eight
+    // bytes), the first eight for one product and the rest for the next; the token rows are read from LDS in the same
+    // order, and the order of k inside a step is free.
+    uint32_t col_row[2];
+    const uint8_t* b_src[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        col_row[q] = (GATED ? (uint32_t(q) * 64u + wave * 16u) : (2 * wave + uint32_t(q)) * 16u) + j;
+        const uint32_t b_proj = GATED ? col_row[q] >> 6 : 0u, b_n = n0 + (GATED ? (col_row[q] & 63u) : col_row[q]);
+        b_src[q] = record + p.off[b_proj * 3] + uint64_t(b_n) * (K / 2) + g4 * 8;
+    }
+    // scales then biases as bf16 [128][groups + 2] (the pad keeps sixteen rows on different banks), then the chain sums
+    // [groups][48]
+    const uint32_t pitch = groups + 2;
+    uint16_t* scale_s = reinterpret_cast<uint16_t*>(meta_s);
+    uint16_t* bias_s = scale_s + kTileCols * pitch;
+    float* sum_s = reinterpret_cast<float*>(bias_s + kTileCols * pitch);
+    if (tid < kTileRowsMax) {
+        const uint32_t x_pos = first + min(tid, rows - 1);
+        row_s[tid] = p.a_rows ? uint32_t(p.a_rows[x_pos]) / p.a_div : x_pos;
+    }
+    {   // a projection's 64 (gate/up) or 128 rows are consecutive in the record: groups / 2 dwords per row
+        const uint32_t half = groups / 2, per_proj = (GATED ? 64u : 128u) * half;
+        for (uint32_t i = tid; i < 128u * half; i += 256) {
+            const uint32_t proj = GATED ? i / per_proj : 0u, at = GATED ? i % per_proj : i, r = i / half, g2 = i % half;
+            const uint32_t sv = ldg_u32(record + p.off[proj * 3 + 1] + uint64_t(n0) * groups * 2, at);
+            const uint32_t ov = ldg_u32(record + p.off[proj * 3 + 2] + uint64_t(n0) * groups * 2, at);
+            *reinterpret_cast<uint32_t*>(scale_s + r * pitch + 2 * g2) = sv;
+            *reinterpret_cast<uint32_t*>(bias_s + r * pitch + 2 * g2) = ov;
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < kTileRowsMax * groups; i += 256) {
+        const uint32_t r = i / groups, g = i % groups;
+        sum_s[g * kTileRowsMax + r] = p.asum[uint64_t(row_s[r]) * groups + g];
+    }
 
     // What a step needs is requested two steps ahead and waits in registers (two sets, taken in turn): with one step of
     // lead the loads' latency, several times a step's arithmetic, was paid at every step.
-    struct Fetched { uint4 a, a2, b; uint16_t s, o; float x; };
+    struct Fetched { uint4 a, a2; uint2 b[2]; };
     Fetched ahead[2];
-    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), 0, 0, 0.0f};
+    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), {make_uint2(0, 0), make_uint2(0, 0)}};
     auto fetch = [&](uint32_t g, Fetched& f) {
         f.a = *reinterpret_cast<const uint4*>(a_src + g * 64);
-        f.b = ldg_u4(b_src + g * 32);
-        if (tid < 128) { f.s = ldg_u16(s_src, g); f.o = ldg_u16(o_src, g); if (tall) f.a2 = *reinterpret_cast<const uint4*>(a_src2 + g * 64); }
-        else if (tid < 128 + kTileRowsMax) f.x = x_src[g];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) f.b[q] = ldg_u2(b_src[q] + g * 32);
+        if (tall && tid < 128) f.a2 = *reinterpret_cast<const uint4*>(a_src2 + g * 64);
     };
-    auto stash = [&](uint32_t buf, const Fetched& f) {
-        const uint4 a_next = f.a, b_next = f.b; const uint16_t s_next = f.s, o_next = f.o; const float x_next = f.x;
-        *reinterpret_cast<uint4*>(&a_s[buf][a_r * kPitch + a_c * 8]) = a_next;
+    auto stash = [&](uint32_t buf, const Fetched& f) {   // the token rows
+        *reinterpret_cast<uint4*>(&a_s[buf][a_r * kPitch + a_c * 8]) = f.a;
         if (tall && tid < 128) *reinterpret_cast<uint4*>(&a_s[buf][(32 + a_r) * kPitch + a_c * 8]) = f.a2;
-        // 32 codes -> 32 bf16: nibble i of a word is element 8w+i
-        const uint32_t words[4] = {b_next.x, b_next.y, b_next.z, b_next.w};
-        uint32_t out[16];
+    };
+    // eight codes -> eight bf16: nibble i of the word is element i
+    auto expand = [](uint32_t word) {
+        uint32_t even = word & 0x0f0f0f0fu, odd = (word >> 4) & 0x0f0f0f0fu;
+        // the masked words are kept from the optimiser, which would otherwise fold mask and shift into a bit-field extract
+        // per element and convert that: with whole bytes every element is one byte-to-float conversion
+        asm volatile("" : "+v"(even), "+v"(odd));
+        uint32_t out[4];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            uint32_t even = words[w] & 0x0f0f0f0fu, odd = (words[w] >> 4) & 0x0f0f0f0fu;
-            // the masked words are kept from the optimiser, which would otherwise fold mask and shift into a bit-field extract
-            // per element and convert that: with whole bytes every element is one byte-to-float conversion
-            asm volatile("" : "+v"(even), "+v"(odd));
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x2 pair = {float((even >> (8 * q)) & 0xffu), float((odd >> (8 * q)) & 0xffu)};
-                out[4 * w + q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
-            }
+        for (int q = 0; q < 4; ++q) {
+            const f32x2 pair = {float((even >> (8 * q)) & 0xffu), float((odd >> (8 * q)) & 0xffu)};
+            out[q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
         }
-        uint4* dst = reinterpret_cast<uint4*>(&b_s[buf][b_r * kPitch + b_h * 32]);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) dst[q] = make_uint4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
-        if (tid < 128) { scale_s[buf][m_r] = b16(s_next); bias_s[buf][m_r] = b16(o_next); }
-        else if (tid < 128 + kTileRowsMax) sum_s[buf][tid - 128u] = x_next;
+        return __builtin_bit_cast(bf16x8, make_uint4(out[0], out[1], out[2], out[3]));
     };
 
-    // the wave's two column tiles (rows of b_s) for every block of sixteen token rows; gate/up: a gate tile and the up tile of
-    // the same rows
-    uint32_t col_row[2];
-#pragma unroll
-    for (int q = 0; q < 2; ++q) col_row[q] = (GATED ? (uint32_t(q) * 64u + wave * 16u) : (2 * wave + uint32_t(q)) * 16u) + j;
     constexpr int kBlocks = int(kTileRowsMax / 16);
     const int blocks = tall ? kBlocks : 2;
     f32x4 total[kBlocks][2], mag[kBlocks][2];   // mag: sum of the magnitudes of the folded terms, the scale of the rounding error
@@ -200,10 +219,49 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     if (groups > 1) fetch(1, ahead[1]);
     stash(0, ahead[0]);
     __syncthreads();
+    // The bias half of the magnitudes, sum over the groups of |bias| * |chain sum|, is a product over the group index:
+    // one matrix-core instruction per accumulator tile and 32 groups instead of a multiply-add per element and step (the
+    // chain sums rounded to bf16 for it, made up for by the factor below: the magnitudes only scale a margin).
+    for (uint32_t g0 = 0; g0 < groups; g0 += 32) {
+        bf16x8 bias_abs[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t g = g0 + 8 * g4 + 2 * uint32_t(i);
+                w[i] = g < groups ? *reinterpret_cast<const uint32_t*>(bias_s + col_row[q] * pitch + g) & 0x7fff7fffu : 0u;
+            }
+            bias_abs[q] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+        }
+#pragma unroll
+        for (int rb = 0; rb < kBlocks; ++rb) {
+            if (rb >= blocks) break;
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t g = min(g0 + 8 * g4 + 2 * uint32_t(i), groups - 2);   // (past the end: times a zero bias)
+                const f32x2 pair = {fabsf(sum_s[g * kTileRowsMax + 16 * rb + j]), fabsf(sum_s[(g + 1) * kTileRowsMax + 16 * rb + j])};
+                w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+            }
+            const bf16x8 sum_abs = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+#pragma unroll
+            for (int q = 0; q < 2; ++q) mag[rb][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sum_abs, bias_abs[q], mag[rb][q], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int rb = 0; rb < kBlocks; ++rb)
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mag[rb][q][r] *= 1.0078125f;
     // two steps per trip, so that the register sets are named at compile time: step g computes from LDS buffer g & 1, requests
     // step g + 2 into the set that step g's data has just left, and stashes step g + 1 from the other set
     auto step = [&](uint32_t g, Fetched& mine, Fetched& next) {
         const uint32_t buf = g & 1u;
+        bf16x8 b[2][2];   // [tile][half of the lane's sixteen codes]
+#pragma unroll
+        for (int q = 0; q < 2; ++q) { b[q][0] = expand(mine.b[q].x); b[q][1] = expand(mine.b[q].y); }
         if (g + 2 < groups) fetch(g + 2, mine);
         f32x4 dot[kBlocks][2];
 #pragma unroll
@@ -212,32 +270,28 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
             for (int q = 0; q < 2; ++q) dot[rb][q] = f32x4{0, 0, 0, 0};
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-            bf16x8 b[2];
-#pragma unroll
-            for (int q = 0; q < 2; ++q) b[q] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&b_s[buf][col_row[q] * kPitch + kk * 32 + g4 * 8]));
 #pragma unroll
             for (int rb = 0; rb < kBlocks; ++rb) {
                 if (rb >= blocks) break;
-                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&a_s[buf][(16 * rb + j) * kPitch + kk * 32 + g4 * 8]));
+                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&a_s[buf][(16 * rb + j) * kPitch + g4 * 16 + kk * 8]));
 #pragma unroll
-                for (int q = 0; q < 2; ++q) dot[rb][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[q], dot[rb][q], 0, 0, 0);
+                for (int q = 0; q < 2; ++q) dot[rb][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[q][kk], dot[rb][q], 0, 0, 0);
             }
         }
         float scale[2], bias[2];
 #pragma unroll
-        for (int q = 0; q < 2; ++q) { scale[q] = scale_s[buf][col_row[q]]; bias[q] = bias_s[buf][col_row[q]]; }
+        for (int q = 0; q < 2; ++q) { scale[q] = b16(scale_s[col_row[q] * pitch + g]); bias[q] = b16(bias_s[col_row[q] * pitch + g]); }
 #pragma unroll
         for (int rb = 0; rb < kBlocks; ++rb) {
             if (rb >= blocks) break;
-            float sums[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sums[r] = sum_s[buf][16 * rb + 4 * g4 + r];
+            const float4 sums4 = *reinterpret_cast<const float4*>(sum_s + g * kTileRowsMax + 16 * rb + 4 * g4);
+            const float sums[4] = {sums4.x, sums4.y, sums4.z, sums4.w};
 #pragma unroll
             for (int q = 0; q < 2; ++q)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     total[rb][q][r] = __builtin_fmaf(scale[q], dot[rb][q][r], __builtin_fmaf(bias[q], sums[r], total[rb][q][r]));
-                    mag[rb][q][r] = __builtin_fmaf(fabsf(scale[q]), fabsf(dot[rb][q][r]), __builtin_fmaf(fabsf(bias[q]), fabsf(sums[r]), mag[rb][q][r]));
+                    mag[rb][q][r] = __builtin_fmaf(fabsf(scale[q]), fabsf(dot[rb][q][r]), mag[rb][q][r]);
                 }
         }
         if (g + 1 < groups) stash(buf ^ 1u, next);
@@ -393,10 +447,14 @@ void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t expert
                           int32_t* tile_rows, int32_t* tile_count) {
     hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(1024), 0, s, offsets, experts, rows, tile_expert, tile_first, tile_rows, tile_count);
 }
+// LDS beyond the kernel's fixed arrays: the scales and biases of 128 weight rows and the chain sums of 48 token rows for
+// every step of K.
+static uint32_t prefill_gemm_lds(uint32_t K) { const uint32_t groups = K / 64; return 2 * kTileCols * (groups + 2) * 2 + groups * kTileRowsMax * 4; }
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles) {
     const dim3 grid(gated ? p.N / 64 : p.N / 128, max_tiles);
-    if (gated) hipLaunchKernelGGL(prefill_gemm_kernel<true>, grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL(prefill_gemm_kernel<false>, grid, dim3(256), 0, s, p);
+    const uint32_t lds = prefill_gemm_lds(p.K);
+    if (gated) hipLaunchKernelGGL(prefill_gemm_kernel<true>, grid, dim3(256), lds, s, p);
+    else hipLaunchKernelGGL(prefill_gemm_kernel<false>, grid, dim3(256), lds, s, p);
 }
 void launch_prefill_patch(hipStream_t s, const PrefillGemm& p, bool gated) {
     const bool wide = p.K % 512 == 0 && p.N % 8 == 0;     // the reference's lane-width rule (metal.mm:649-674)
@@ -408,6 +466,9 @@ void launch_prefill_patch(hipStream_t s, const PrefillGemm& p, bool gated) {
     else { if (tabled) ZC_PATCH(16, false, true); else if (wide) ZC_PATCH(16, false, false); else ZC_PATCH(8, false, false); }
 #undef ZC_PATCH
 }
-bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts) { return hidden % 128 == 0 && inter % 128 == 0 && experts <= 1024; }
+// (hidden and intermediate sizes up to 4096: the product kernel keeps a whole K of scales, biases and chain sums in LDS)
+bool prefill_shape(uint32_t hidden, uint32_t inter, uint32_t experts) {
+    return hidden % 128 == 0 && inter % 128 == 0 && hidden <= 4096 && inter <= 4096 && experts <= 1024;
+}
 
 }  // namespace zc

@@ -184,7 +184,7 @@ zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* cfg, c
  * q4_mm / q4_gate_up, qwen.metal:289-376).  Router ids, softmax weights and the dispatch are the exact kernels (bit-equal
  * to zc_hip_moe_forward); expert outputs agree with zc_hip_moe_forward to a few fp32 ulps before their BF16 rounding, so
  * the layer output is checked against a tolerance (max relative error 2e-3), not bit for bit.  Affine Q4 group 64 only,
- * hidden and intermediate sizes multiples of 128; x must be BF16-valued (else status bit 4 at zc_hip_moe_check).
+ * hidden and intermediate sizes multiples of 128 up to 4096; x must be BF16-valued (else status bit 4 at zc_hip_moe_check).
  * The workspace is larger than zc_hip_moe_forward's: zc_hip_moe_prefill_workspace_bytes (0: shape not supported). */
 uint64_t zc_hip_moe_prefill_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens);
 zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* layer,

@@ -683,7 +683,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
                              float* out, void* workspace, const zc_moe_trace* trace) {
     Timed timed(ctx, "moe_prefill");
     if (const zc_status s = validate_config(c)) return s;
-    ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 group 64 with hidden and intermediate sizes that are multiples of 128");
+    ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 group 64 with hidden and intermediate sizes that are multiples of 128 up to 4096");
     ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
     ZC_REQUIRE(uint64_t(T) * c->topk * std::max(c->hidden, c->inter) < (1ull << 32), "too many product elements for one prefill call");
     ZC_REQUIRE(l->router && l->shared_gate && l->shared_record && l->expert_records, "missing MoE layer weights");

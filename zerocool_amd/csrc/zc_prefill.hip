@@ -15,11 +15,12 @@
 //
 // Tiling.  One workgroup (4 waves) owns up to 48 sorted token rows of ONE expert and 128 weight rows (gate/up: 64 gate rows
 // and the 64 up rows of the same indices, so SwiGLU is fused in registers), and walks K in steps of 64 = one scale
-// group: the 4-bit codes of the step are expanded to bf16 once per workgroup into LDS, the token rows are gathered into
-// LDS as bf16, both double-buffered.  Each wave multiplies all (two or three) 16-row blocks of the tokens by 2 of the 8
-// column tiles.  An expert's rows are cut into tiles of 32, except that a run of up to 48 rows (a whole expert with few
-// rows, or the last rows of a longer run) is ONE tile: with about forty rows per expert -- an unskewed router at 2048
-// tokens -- every expert's codes are then expanded once, not twice.
+// group.  Each wave multiplies all (two or three) 16-row blocks of the tokens by 2 of the 8 column tiles: the 4-bit codes
+// of its 32 weight rows go from memory straight into the lanes that feed them to the matrix cores and are expanded to
+// bf16 there (once per workgroup and step), the token rows are gathered into LDS as bf16, double-buffered, and the
+// scales, biases and chain sums of all steps are brought into LDS once.  An expert's rows are cut into tiles of 32, except
+// that a run of up to 48 rows (a whole expert with few rows, or the last rows of a longer run) is ONE tile: with about
+// forty rows per expert -- an unskewed router at 2048 tokens -- every expert's codes are then expanded once, not twice.
 #include "zc_kernels.hpp"
 #include "zc_device.hpp"
 

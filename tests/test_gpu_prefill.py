@@ -46,7 +46,8 @@ ONE_BF16_STEP = 2.0 ** -7   # the spacing of BF16 numbers relative to their magn
 
 
 @pytest.mark.parametrize("shape,tokens", [((512, 32, 4, 128), 1), ((512, 32, 4, 128), 37), ((512, 32, 4, 128), 300),
-                                          ((1024, 64, 10, 256), 129), ((2048, 512, 10, 512), 96)])
+                                          ((1024, 64, 10, 256), 129), ((2048, 512, 10, 512), 96),
+                                          ((3072, 16, 4, 1024), 70), ((4096, 8, 2, 128), 33)])   # 48 and 64 scale groups: the largest K
 def test_prefill_matches_the_exact_path(ctx, shape, tokens):
     cfg = workload.tiny_config(*shape)
     weights = workload.LayerWeights(ctx, cfg, 61 + tokens, ("normal", 0.5))
@@ -147,6 +148,8 @@ def test_prefill_reports_unroutable_rows(ctx):
 def test_prefill_rejects_what_it_cannot_run(ctx):
     mixed = workload.tiny_config(512, 32, 4, 128, bits=(4, 8, 8, 8))
     assert ctx.moe_prefill_workspace_bytes(mixed, 64) == 0
+    assert ctx.moe_prefill_workspace_bytes(workload.tiny_config(4224, 32, 4, 128), 64) == 0   # K beyond what the product kernel keeps in LDS
+    assert ctx.moe_prefill_workspace_bytes(workload.tiny_config(4096, 32, 4, 4096), 64) > 0
     cfg = workload.tiny_config(512, 32, 4, 128)
     weights = workload.LayerWeights(ctx, cfg, 93, None)
     T = 40

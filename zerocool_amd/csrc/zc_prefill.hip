@@ -418,10 +418,12 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
                 for (int i = 0; i < WIDTH; i += 8) {
                     // nibble j of a word is element j: the even ones and the odd ones as bytes, each converted by one byte-to-float instruction
                     const uint32_t even = words[u][proj][i / 8] & 0x0f0f0f0fu, odd = (words[u][proj][i / 8] >> 4) & 0x0f0f0f0fu;
-                    dot += xb[i] * float(even & 0xffu) + xb[i + 1] * float(odd & 0xffu) +
-                           xb[i + 2] * float((even >> 8) & 0xffu) + xb[i + 3] * float((odd >> 8) & 0xffu);
-                    dot += xb[i + 4] * float((even >> 16) & 0xffu) + xb[i + 5] * float((odd >> 16) & 0xffu) +
-                           xb[i + 6] * float(even >> 24) + xb[i + 7] * float(odd >> 24);
+                    // (a BF16 value times a 4-bit code is exact in fp32, so a fused multiply-add rounds as the reference's
+                    // multiply and add do: ((p0 + p1) + p2) + p3, then onto the block's sum)
+                    dot += __builtin_fmaf(xb[i + 3], float((odd >> 8) & 0xffu), __builtin_fmaf(xb[i + 2], float((even >> 8) & 0xffu),
+                           __builtin_fmaf(xb[i + 1], float(odd & 0xffu), xb[i] * float(even & 0xffu))));
+                    dot += __builtin_fmaf(xb[i + 7], float(odd >> 24), __builtin_fmaf(xb[i + 6], float(even >> 24),
+                           __builtin_fmaf(xb[i + 5], float((odd >> 16) & 0xffu), xb[i + 4] * float((even >> 16) & 0xffu))));
                 }
                 result[proj] += b16(scale_bits[u][proj]) * dot + sum * b16(bias_bits[u][proj]);
             }

@@ -74,3 +74,32 @@ def test_xint_matches_oracle(ctx, K, N, kind):
         ctx.free(dx)
     for b in dl._keep + du._keep:
         ctx.free(b)
+
+
+@pytest.mark.parametrize("kind", ["normal", "wide-range", "special", "activations"])
+def test_xint_32_column_tiles(ctx, kind):
+    """Calls with enough tokens to fill the chip take the tile engine's 32-column form (v_mfma_i32_32x32x32_i8, up to four
+    tokens per instruction): the same bytes as the literal lane kernels on every token, and as the oracle on a sample; the
+    sizes leave partial tiles (2056 rows) and a partial last group of tokens (130)."""
+    K, N, T = 1024, 2056, 130
+    rng = np.random.default_rng(77 + len(kind))
+    a, u = make(rng, K, N), make(rng, K, N)
+    ol, ou = oracle.make_linear(*a, K, N), oracle.make_linear(*u, K, N)
+    dl, du = dev_linear(ctx, *a, K, N), dev_linear(ctx, *u, K, N)
+    x = inputs(rng, K, T, kind); dx = ctx.upload(x)
+    rows = rng.integers(0, T, T).astype(np.int32); drows = ctx.upload(rows)
+    ctx.configure(1)
+    got = [ctx.linear(dl, dx, T).numpy(f32), ctx.linear(dl, dx, T, float_output=True).numpy(f32),
+           ctx.gated_linear(dl, du, dx, T, T).numpy(f32), ctx.gated_linear(dl, du, dx, T, T, drows).numpy(f32)]
+    ctx.configure(0)
+    lit = [ctx.linear(dl, dx, T).numpy(f32), ctx.linear(dl, dx, T, float_output=True).numpy(f32),
+           ctx.gated_linear(dl, du, dx, T, T).numpy(f32), ctx.gated_linear(dl, du, dx, T, T, drows).numpy(f32)]
+    ctx.configure(1)
+    for g, l in zip(got, lit):
+        assert g.tobytes() == l.tobytes(), (kind, int((g.view(np.uint32) != l.view(np.uint32)).sum()))
+    sample = np.r_[0:6, T - 2:T]
+    want = [oracle.linear(ol, x[sample], len(sample)), oracle.gated_linear(ol, ou, x[sample], len(sample))]
+    assert got[0].reshape(T, N)[sample].tobytes() == want[0].tobytes()
+    assert got[2].reshape(T, N)[sample].tobytes() == want[1].tobytes()
+    for b in dl._keep + du._keep + (dx, drows):
+        ctx.free(b)

@@ -63,7 +63,7 @@ __device__ __forceinline__ float load_shared_f32(const float* p) {
 // sixteen elements of block b.  kExactProducts: every element is BF16-valued, so x*q is
 // exact and a fused multiply-add equals the reference's separate multiply and add.
 struct LdsBf16 {     // BF16 copy of a BF16-valued row
-    static constexpr bool kExactProducts = true;
+    static constexpr bool kExactProducts = true, kRowInLds = true;
     const uint16_t* x;
     __device__ __forceinline__ void block(uint32_t b, uint32_t* out) const {
         const uint4 lo = *reinterpret_cast<const uint4*>(x + b * 16), hi = *reinterpret_cast<const uint4*>(x + b * 16 + 8);
@@ -73,7 +73,7 @@ struct LdsBf16 {     // BF16 copy of a BF16-valued row
     }
 };
 struct RegBf16 {     // one block of sixteen BF16 values held in registers (block index ignored)
-    static constexpr bool kExactProducts = true;
+    static constexpr bool kExactProducts = true, kRowInLds = false;
     uint64_t w[4];
     __device__ __forceinline__ void block(uint32_t, uint32_t* out) const {
 #pragma unroll
@@ -84,7 +84,7 @@ struct RegBf16 {     // one block of sixteen BF16 values held in registers (bloc
     }
 };
 struct RegF32 {      // one block of sixteen BF16-valued fp32 bit patterns held in registers (block index ignored)
-    static constexpr bool kExactProducts = true;
+    static constexpr bool kExactProducts = true, kRowInLds = false;
     uint32_t bits[16];
     __device__ __forceinline__ void block(uint32_t, uint32_t* out) const {
 #pragma unroll
@@ -92,7 +92,7 @@ struct RegF32 {      // one block of sixteen BF16-valued fp32 bit patterns held 
     }
 };
 struct LdsF32 {      // fp32 copy of an arbitrary row
-    static constexpr bool kExactProducts = false;
+    static constexpr bool kExactProducts = false, kRowInLds = false;
     const float* x;
     __device__ __forceinline__ void block(uint32_t b, uint32_t* out) const {
 #pragma unroll
@@ -663,6 +663,150 @@ __device__ __forceinline__ void xint_run_tile_upto4(const uint8_t* w_row, const 
     if (nt <= 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     else if (nt == 2) xint_run_tile_tokens<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     else xint_run_tile_tokens<4, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+}
+
+// A tile of 32 weight rows for NTOK <= 4 tokens on v_mfma_i32_32x32x32_i8, which costs a SIMD the same time as the
+// 16x16x64 form and has four times the room: its 32 rows hold (token t, block c of two, plane p) as row 8 t + 4 c + p, its
+// 32 k are two blocks (half wave h supplies block h of the pair), its 32 columns the tile's weight rows.  lane = (n = column,
+// h = lane / 32).  Per span of 128 elements lane (n, h) fetches the 32 bytes of codes of blocks 4 h .. 4 h + 3 of weight row
+// n; instruction i of the span multiplies blocks i and 4 + i; result elements 4 t .. 4 t + 2 of lane (n, h) are token t's
+// three plane sums for block 4 h + i.  Reference lane 8 (d mod 4) + 4 h + i of the row is acc[t][d mod 4][i] of lane (n, h):
+// per-lane accumulation order and the butterfly (strides 16 and 8 pair accumulators, 4 the half waves, 2 and 1 the
+// blocks of a lane) are those of xint_run_tile_after, so the sums are the same bits.  Images beyond the live tokens are
+// not read (their rows of the operand are zeros).
+typedef int v16i __attribute__((ext_vector_type(16)));
+template <int NTOK, class Source, class Emit>
+__device__ __forceinline__ void xint_run_tile32(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans,
+                                                const uint8_t* const* img, const Source* src, const XintLayout L, uint32_t lane,
+                                                int nt, Emit emit) {
+    static_assert(NTOK >= 1 && NTOK <= 4, "four tokens fill the instruction's rows");
+    constexpr int R = 4;   // spans per body: one scale / bias vector of 16 bytes and one mask word per token
+    const uint32_t h = lane >> 5, m = lane & 31u, t_a = m >> 3, c_a = (m >> 2) & 1u, p_a = m & 3u;
+    const uint8_t* c = w_row + 32 * h;   // the lane's 32 bytes of each 64-byte span
+    // codes travel two spans at a time (four 16-byte loads per lane in flight while the two spans before are multiplied), the
+    // scale and bias vectors four spans at a time
+    uint4 ring[4], sring, bring;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ring[j] = ldg_u4(c, (j / 2) * 4 + (j & 1));
+    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
+    float acc[NTOK][4][4];
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[t][q][i] = 0;
+    const uint32_t half = (lane & 32u) ? 0x03020c0cu : 0x01000c0cu;   // group 2d + h: the low BF16 of a dword for h = 0
+    // left operand: row (t, c, p) of half wave h holds digit plane p of token t's block 4 h + i when c == h, zeros otherwise
+    const bool live = c_a == h && p_a < 3 && t_a < uint32_t(nt);
+    const uint8_t* a_image = img[0];
+#pragma unroll
+    for (int t = 1; t < NTOK; ++t) a_image = t_a == uint32_t(t) ? img[t] : a_image;
+    const uint8_t* a_base = live ? a_image + 4 * h * 48 + p_a * 16 : img[0] + L.blocks() * 48;
+    const uint32_t a_span = live ? 8 * 48 : 0, a_next = live ? 48 : 0;
+    const uint32_t M = 0x0f0f0f0fu;
+    v16i zero;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) zero[e] = 0;
+    const uint32_t info_at = L.planes_bytes() + 4 * h * 8, mask_at = L.planes_bytes() + L.info_bytes();
+    for (uint32_t d0 = 0; d0 < spans; d0 += R) {
+        const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
+        if (d0 + R < spans) { sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4); }
+        // the unsafe bits of the lane's blocks, per token: block 8 d + 4 h + i is bit 8 (d - d0) + 4 h + i of mask word d0 / 4
+        uint32_t unsafe[NTOK], any = 0;
+#pragma unroll
+        for (int t = 0; t < NTOK; ++t) {
+            unsafe[t] = t < nt ? (reinterpret_cast<const uint32_t*>(img[t] + mask_at)[d0 / 4] >> (4 * h)) & 0x0f0f0f0fu : 0u;
+            any |= unsafe[t];
+        }
+        const bool literal_body = __ballot(any != 0) != 0;
+#pragma unroll
+        for (int part = 0; part < 2; ++part) {
+            uint4 codes[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) codes[j] = ring[j];
+            if (d0 + 2 * uint32_t(part) + 2 < spans) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ring[j] = ldg_u4(c, (d0 + 2 * uint32_t(part) + 2 + j / 2) * 4 + (j & 1));
+            }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = 2 * part + jj;
+            const uint32_t d = d0 + uint32_t(j);
+            const uint32_t words[8] = {codes[2 * jj].x, codes[2 * jj].y, codes[2 * jj].z, codes[2 * jj].w,
+                                       codes[2 * jj + 1].x, codes[2 * jj + 1].y, codes[2 * jj + 1].z, codes[2 * jj + 1].w};
+            float dot[NTOK][4], bsum[NTOK][4];
+#pragma unroll
+            for (int t = 0; t < NTOK; ++t) {
+                const float4 f0 = *reinterpret_cast<const float4*>(img[t < nt ? t : 0] + info_at + d * 64);        // {2^e, sum} of blocks 4h, 4h+1
+                const float4 f1 = *reinterpret_cast<const float4*>(img[t < nt ? t : 0] + info_at + d * 64 + 16);   // of blocks 4h+2, 4h+3
+                dot[t][0] = f0.x; bsum[t][0] = f0.y; dot[t][1] = f0.z; bsum[t][1] = f0.w;
+                dot[t][2] = f1.x; bsum[t][2] = f1.y; dot[t][3] = f1.z; bsum[t][3] = f1.w;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const v4i b = {int(words[2 * i] & M), int((words[2 * i] >> 4) & M), int(words[2 * i + 1] & M), int((words[2 * i + 1] >> 4) & M)};
+                const v4i a = *reinterpret_cast<const v4i*>(a_base + d * a_span + uint32_t(i) * a_next);
+                const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < NTOK; ++t) {
+                    const v4i planes = {r[4 * t], r[4 * t + 1], r[4 * t + 2], 0};
+                    dot[t][i] = float(xint_digits(planes)) * dot[t][i];
+                }
+                if constexpr (!Source::kRowInLds) {
+                    if (__builtin_expect(literal_body, 0)) {
+#pragma unroll
+                        for (int t = 0; t < NTOK; ++t)
+                            if ((unsafe[t] >> (8 * j + i)) & 1u) dot[t][i] = xint_literal_dot(b, src[t], 8 * d + 4 * h + uint32_t(i));
+                    }
+                }
+            }
+            if constexpr (Source::kRowInLds) {
+                // BF16 rows in LDS: ONE loop serves the literal chains of all tokens and blocks of the span, every lane taking its
+                // next unsafe (token, block) in turn (bit 4 t + i), so the chain's code exists once per span
+                if (__builtin_expect(literal_body, 0)) {
+                    uint32_t pending = 0;
+#pragma unroll
+                    for (int t = 0; t < NTOK; ++t) pending |= ((unsafe[t] >> (8 * j)) & 15u) << (4 * t);
+                    while (__ballot(pending != 0) != 0) {
+                        if (pending) {
+                            const uint32_t item = uint32_t(__builtin_ctz(pending)), t = item >> 2, i = item & 3u;
+                            const uint16_t* row = src[0].x;
+#pragma unroll
+                            for (int q = 1; q < NTOK; ++q) row = t == uint32_t(q) ? src[q].x : row;
+                            uint32_t lo = words[0], hi = words[1];
+#pragma unroll
+                            for (int q = 1; q < 4; ++q) { lo = i == uint32_t(q) ? words[2 * q] : lo; hi = i == uint32_t(q) ? words[2 * q + 1] : hi; }
+                            const float lit = xint_literal_block(row + (8 * d + 4 * h + i) * 16, lo, hi);
+#pragma unroll
+                            for (int q = 0; q < NTOK; ++q)
+#pragma unroll
+                                for (int ii = 0; ii < 4; ++ii) dot[q][ii] = item == uint32_t(4 * q + ii) ? lit : dot[q][ii];
+                            pending &= pending - 1;
+                        }
+                    }
+                }
+            }
+            const float scale = xint_bf16_of(sdw[j], half), bias = xint_bf16_of(bdw[j], half);
+#pragma unroll
+            for (int t = 0; t < NTOK; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[t][j][i] += scale * dot[t][i] + bsum[t][i] * bias;
+        }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+        float z[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float x0 = acc[t][0][i] + acc[t][2][i], x1 = acc[t][1][i] + acc[t][3][i];
+            const float y = x0 + x1;
+            z[i] = y + __shfl_xor(y, 32);
+        }
+        const float w0 = z[0] + z[2], w1 = z[1] + z[3];
+        if (t < nt) emit(t, w0 + w1);
+    }
 }
 
 template <int PT, int R, class Source, class Emit>

@@ -185,6 +185,9 @@ zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* cfg, c
  * to zc_hip_moe_forward); expert outputs agree with zc_hip_moe_forward to a few fp32 ulps before their BF16 rounding, so
  * the layer output is checked against a tolerance (max relative error 2e-3), not bit for bit.  Affine Q4 group 64 only,
  * hidden and intermediate sizes multiples of 128 up to 4096; x must be BF16-valued (else status bit 4 at zc_hip_moe_check).
+ * From 128 tokens on the router logits are formed exactly only for the experts that can reach the top k (a matrix-core
+ * product with a rigorous bound decides which; ids and weights are unchanged); a trace that asks for the logits gets
+ * all of them from the exact kernel.
  * The workspace is larger than zc_hip_moe_forward's: zc_hip_moe_prefill_workspace_bytes (0: shape not supported). */
 uint64_t zc_hip_moe_prefill_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens);
 zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* layer,

@@ -161,3 +161,48 @@ def test_prefill_rejects_what_it_cannot_run(ctx):
     assert "BF16" in str(err.value)
     with pytest.raises(z.ZcError):
         ctx.moe_prefill(mixed, weights.layer, x, T, out, ws)
+
+
+@pytest.mark.parametrize("skew", [None, ("zipf", 1.1)])
+def test_prefill_router_on_bounds_picks_the_exact_ids(ctx, skew):
+    """From 128 tokens on (and when the logits themselves are not asked for) the prefill router forms every logit with a
+    bf16 matrix-core product, bounds its distance from the reference's chains, and recomputes exactly only the experts that
+    can be among the top k.  Ids and softmax weights must be the exact path's bits, also where logits tie exactly (router
+    rows repeated, an all-zero input row), nearly tie (a row that differs from another in one element's last bit), where an
+    input row is huge or tiny, and where it holds inf or NaN (then no expert is selectable: reported, other tokens
+    untouched)."""
+    cfg = workload.tiny_config(1024, 128, 8, 128)
+    weights = workload.LayerWeights(ctx, cfg, 301, skew)
+    E, H, T = cfg.experts, cfg.hidden, 200
+    router = weights.router.numpy(np.uint16).reshape(E, H).copy()
+    router[17] = router[5]; router[90] = router[5]; router[33] = router[64]      # exact ties
+    router[70] = router[12]; router[70, 100] ^= 1                                  # one element differs by its last bit
+    ctx.upload(router.ravel(), into=weights.router)
+    x = workload.hidden_rows(ctx, T, H, 302).numpy(f32).reshape(T, H).copy()
+    x[7] = 0.0
+    x[8] = oracle.bf(x[8] * f32(2.0 ** 60)); x[9] = oracle.bf(x[9] * f32(2.0 ** -60))
+    x[12] = oracle.bf(x[12] * f32(2.0 ** -75)); x[13] = oracle.bf(x[13] * f32(2.0 ** -120))   # squares below the normal range
+    x[10] = x[11]                                                                  # two tokens alike
+    dx = ctx.upload(x.ravel())
+    exact, fast = run_both(ctx, cfg, weights, dx, T)
+    assert fast["ids"].tobytes() == exact["ids"].tobytes()
+    assert fast["weights"].tobytes() == exact["weights"].tobytes()
+    assert (exact["ids"].reshape(T, cfg.topk)[7] == np.arange(cfg.topk)).all() or skew is not None   # all logits equal: the lowest ids
+    # rows that no expert can be selected for
+    bad = x.copy(); bad[20, 5] = np.nan; bad[21, 9] = np.inf; bad[22, 9] = -np.inf; bad[22, 10] = np.inf
+    dbad = ctx.upload(bad.ravel())
+    n = T * cfg.topk
+    got = {}
+    for prefill in (False, True):
+        out = ctx.alloc(T * H * 4); ids = ctx.alloc(n * 4)
+        ws = ctx.alloc(ctx.moe_prefill_workspace_bytes(cfg, T) if prefill else ctx.moe_workspace_bytes(cfg, T))
+        (ctx.moe_prefill if prefill else ctx.moe_forward)(cfg, weights.layer, dbad, T, out, ws, z.Trace(None, ids.ptr, None, None, None, None))
+        with pytest.raises(z.ZcError) as err:
+            ctx.moe_check()
+        assert "invalid router output" in str(err.value)
+        got[prefill] = ids.numpy(np.int32).copy()
+        for b in (out, ids, ws):
+            ctx.free(b)
+    assert got[True].tobytes() == got[False].tobytes()
+    for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, dx, dbad):
+        ctx.free(b)

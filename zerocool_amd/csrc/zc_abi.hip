@@ -648,6 +648,7 @@ struct PrefillSpace {
     int32_t *tile_expert, *tile_first, *tile_rows, *tile_count, *stile_expert, *stile_first, *stile_rows, *stile_count;
     uint32_t max_tiles, max_shared_tiles;
     uint32_t* near_bits;      // one bit per product element: recompute exactly
+    float* norms;             // |row| of the inputs and of the router's rows (the fast router's bound)
     uint64_t bytes;
 };
 PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
@@ -667,6 +668,7 @@ PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
     w.near_bits = (uint32_t*)take(n * std::max(c->hidden, c->inter) / 8);
     w.xsum16 = (float*)take(uint64_t(T) * (c->hidden / 16) * 4); w.asum16 = (float*)take(n * (c->inter / 16) * 4);
     w.ssum16 = (float*)take(uint64_t(T) * (c->inter / 16) * 4);
+    w.norms = (float*)take((uint64_t(T) + c->experts) * 4);
     w.bytes = at;
     return w;
 }
@@ -696,8 +698,11 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     hipStream_t s = ctx->stream;
     const uint32_t H = c->hidden, I = c->inter, E = c->experts, k = c->topk;
     const uint64_t n = uint64_t(T) * k;
-    // exact kernels: router logits, top-k + softmax, dispatch (model.cpp:434-479), shared gate
-    zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
+    // router logits, top-k + softmax, dispatch (model.cpp:434-479), shared gate: the exact kernels, except that a long batch
+    // whose logits nobody asks for gets exact logits only where the selection can see the difference (launch_prefill_router)
+    zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, w.xsum16, ctx->moe_status);
+    if (T >= 128 && !(trace && trace->logits)) zc::launch_prefill_router(s, x, w.xb, l->router, l->router_offsets, T, H, E, k, w.norms, w.base.logits);
+    else zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
     zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
     zc::launch_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, w.base.selected, w.base.count, ctx->moe_status);
     zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
@@ -705,7 +710,6 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     const float margin = zc::kPrefillMargin;
     // the per-block chain sums pay where a lane of the recomputation has several blocks of a row (long rows); short rows form them in place
     const bool table_inter = I / 16 >= 128;
-    zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, w.xsum16, ctx->moe_status);
     zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
     zc::launch_prefill_tiles(s, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
     auto offsets_of = [&](const void* record, int shared, uint64_t* off, int first, int count) {

@@ -30,6 +30,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kTileRows = 32, kTileRowsMax = 48, kTileCols = 128, kPitch = 72;   // LDS row pitch in bf16 elements (144 bytes)
 
@@ -436,6 +437,201 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
         else p.out_f[uint64_t(p.out_rows ? uint32_t(p.out_rows[pos]) : pos) * N + n] = bf(result[0]);
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Router logits of a long batch without the exact chains for every (token, expert): a bf16 matrix-core product gives
+// every logit to within a bound that holds whatever the order of its additions, the top-k can only come from the
+// logits within that bound of the k-th largest, and only those are recomputed with the reference's chains
+// (qwen.metal:512-534: sixteen contiguous K partitions, a k-ascending multiply-accumulate chain in each, partials added
+// 0..15).  The other logits are written as -inf, so the exact selection kernel that follows picks what it would pick from
+// all the exact logits: ids and softmax weights are the reference's bits.
+//
+// The bound.  Inputs and router weights are BF16-valued, so every product is exact in fp32.  Two fp32 sums of the same n
+// exact products, each formed with at most n additions that round or truncate to fp32, differ by at most
+// n * 2^-22 * sum |x_k w_k| (n * 2^-23 for a truncating accumulator plus n * 2^-24 for the reference's rounded chain
+// leaves a factor 1.3), and sum |x_k w_k| <= |x| |w| (Cauchy-Schwarz).  Adding the expert's offset rounds both once more:
+// 2^-22 |logit| on top.  With lower bounds a - m and upper bounds a + m of the exact logits: the k-th largest exact logit
+// is at least the k-th largest lower bound, which is at least the k-th largest of the 64 lanes' largest lower bounds; an
+// expert whose upper bound is below that cannot be among the top k, ties included.  A token with a logit that is not
+// finite has every expert recomputed.
+// ---------------------------------------------------------------------------------------------------------------------
+// |row| of bf16 rows, rounded up a little: one wavefront per row; rows [0, rows_a) come from a, the rest from b.
+__global__ __launch_bounds__(256) void row_norms_kernel(const uint16_t* a, uint32_t rows_a, const uint16_t* b, uint32_t rows_b, uint32_t K, float* norms) {
+    const uint32_t row = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x & 63u;
+    if (row >= rows_a + rows_b) return;
+    const uint16_t* src = row < rows_a ? a + uint64_t(row) * K : b + uint64_t(row - rows_a) * K;
+    float sum = 0;
+    for (uint32_t i = lane * 8; i < K; i += 512) {
+        const uint4 v = *reinterpret_cast<const uint4*>(src + i);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float lo = __uint_as_float(w[q] << 16), hi = __uint_as_float(w[q] & 0xffff0000u);
+            sum = __builtin_fmaf(lo, lo, sum); sum = __builtin_fmaf(hi, hi, sum);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o; o >>= 1) sum += __shfl_xor(sum, o);
+    // (a row so small that its squares leave the normal range has no usable norm: +inf makes the caller recompute everything)
+    if (lane == 0) norms[row] = sum < 0x1p-100f ? __uint_as_float(0x7f800000u) : sqrtf(sum) * 1.0001f;
+}
+// approx[t][e] = sum_k a[t][k] b[e][k] (+ offsets[e]): 64 tokens x 64 experts per workgroup, a wave a 32 x 32 block on
+// v_mfma_f32_32x32x16_bf16, K in steps of 64 through LDS (rows padded to 144 bytes), the next step's rows in registers.
+__global__ __launch_bounds__(256) void router_product_kernel(const uint16_t* a, const uint16_t* b, uint32_t T, uint32_t E, uint32_t K,
+                                                             const float* offsets, float* approx) {
+    __shared__ __align__(16) uint16_t a_s[2][64 * kPitch], b_s[2][64 * kPitch];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, m = lane & 31u, h = lane >> 5;
+    const uint32_t t0 = blockIdx.y * 64, e0 = blockIdx.x * 64;
+    const uint32_t r = tid >> 3, c8 = tid & 7u;   // a thread moves rows r and r + 32, sixteen bytes each, of both operands
+    const uint16_t* a_src0 = a + uint64_t(min(t0 + r, T - 1)) * K + c8 * 8;
+    const uint16_t* a_src1 = a + uint64_t(min(t0 + r + 32, T - 1)) * K + c8 * 8;
+    const uint16_t* b_src0 = b + uint64_t(min(e0 + r, E - 1)) * K + c8 * 8;
+    const uint16_t* b_src1 = b + uint64_t(min(e0 + r + 32, E - 1)) * K + c8 * 8;
+    uint4 ra0, ra1, rb0, rb1;
+    auto fetch = [&](uint32_t g) {
+        ra0 = *reinterpret_cast<const uint4*>(a_src0 + g * 64); ra1 = *reinterpret_cast<const uint4*>(a_src1 + g * 64);
+        rb0 = *reinterpret_cast<const uint4*>(b_src0 + g * 64); rb1 = *reinterpret_cast<const uint4*>(b_src1 + g * 64);
+    };
+    auto stash = [&](uint32_t buf) {
+        *reinterpret_cast<uint4*>(&a_s[buf][r * kPitch + c8 * 8]) = ra0; *reinterpret_cast<uint4*>(&a_s[buf][(r + 32) * kPitch + c8 * 8]) = ra1;
+        *reinterpret_cast<uint4*>(&b_s[buf][r * kPitch + c8 * 8]) = rb0; *reinterpret_cast<uint4*>(&b_s[buf][(r + 32) * kPitch + c8 * 8]) = rb1;
+    };
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    const uint32_t steps = K / 64, row_a = (wave >> 1) * 32 + m, row_b = (wave & 1u) * 32 + m;
+    fetch(0); stash(0);
+    __syncthreads();
+    for (uint32_t g = 0; g < steps; ++g) {
+        const uint32_t buf = g & 1u;
+        if (g + 1 < steps) fetch(g + 1);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const bf16x8 av = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&a_s[buf][row_a * kPitch + q * 16 + h * 8]));
+            const bf16x8 bv = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&b_s[buf][row_b * kPitch + q * 16 + h * 8]));
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+        }
+        if (g + 1 < steps) stash(buf ^ 1u);
+        __syncthreads();
+    }
+    const uint32_t e = e0 + (wave & 1u) * 32 + m;
+    const float offset = (offsets && e < E) ? offsets[e] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t t = t0 + (wave >> 1) * 32 + 8 * uint32_t(i / 4) + 4 * h + uint32_t(i % 4);
+        if (t < T && e < E) approx[uint64_t(t) * E + e] = offsets ? acc[i] + offset : acc[i];
+    }
+}
+// One wavefront per token: bounds, the experts that can be among the top k, their exact logits; everything else -inf.
+// (A whole workgroup per token, each wavefront taking a quarter of the list, measured slower: 35 against 29 us.)
+constexpr int kRefinePerLane = 16;   // experts <= 1024
+__global__ __launch_bounds__(256) void router_refine_kernel(const uint16_t* xb, const uint16_t* w, const float* offsets, const float* norms,
+                                                            uint32_t T, uint32_t E, uint32_t K, uint32_t topk, float* logits) {
+    __shared__ float row_s[4][1024];
+    __shared__ uint16_t list_s[4][1024];
+    extern __shared__ __align__(16) uint16_t x_s[];   // the four tokens' input rows (BF16-valued, so the bf16 copy is the input)
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x & 63u, t = blockIdx.x * 4 + wave;
+    if (t >= T) return;
+    uint16_t* x_row = x_s + wave * K;
+    for (uint32_t i = lane * 8; i < K; i += 512) *reinterpret_cast<uint4*>(x_row + i) = *reinterpret_cast<const uint4*>(xb + uint64_t(t) * K + i);
+    const float ninf = __uint_as_float(0xff800000u);
+    float* row = logits + uint64_t(t) * E;
+    const float reach = float(K) * 0x1p-22f * norms[t];
+    float upper[kRefinePerLane], best_lower = ninf;
+    bool strange = false;
+#pragma unroll
+    for (int i = 0; i < kRefinePerLane; ++i) {
+        const uint32_t e = lane + 64u * uint32_t(i);
+        upper[i] = ninf;
+        if (e < E) {
+            const float a = row[e], bound = reach * norms[T + e] + 0x1p-22f * fabsf(a);
+            strange = strange || !(fabsf(a) < __uint_as_float(0x7f800000u)) || !(bound < __uint_as_float(0x7f800000u));
+            upper[i] = a + bound;
+            best_lower = fmaxf(best_lower, a - bound);
+        }
+    }
+    // the k-th largest of the lanes' largest lower bounds (fewer than k lanes with an expert: nothing can be ruled out)
+    float threshold = ninf;
+    bool all = __ballot(strange) != 0;
+    {
+        float mine = best_lower;
+        for (uint32_t j = 0; j < topk && !all; ++j) {
+            float top = mine;
+#pragma unroll
+            for (int o = 32; o; o >>= 1) top = fmaxf(top, __shfl_xor(top, o));
+            if (!(top > ninf)) { all = true; break; }
+            threshold = top;
+            const uint64_t holders = __ballot(mine == top);
+            if (lane == uint32_t(__ffsll((long long)holders) - 1)) mine = ninf;
+        }
+    }
+    // the list of experts to recompute, in any order
+    uint32_t count = 0;
+#pragma unroll
+    for (int i = 0; i < kRefinePerLane; ++i) {
+        const uint32_t e = lane + 64u * uint32_t(i);
+        const bool take = e < E && (all || upper[i] >= threshold);
+        const uint64_t takers = __ballot(take);
+        if (take) list_s[wave][count + uint32_t(__popcll(takers & ((1ull << lane) - 1)))] = uint16_t(e);
+        count += uint32_t(__popcll(takers));
+        if (e < E) row_s[wave][e] = ninf;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // four experts at a time: sixteen lanes run an expert's sixteen partition chains (router_kernel's arithmetic).  Eight weight
+    // pieces = 64 elements are requested together, and the next eight -- of this expert or of the next four's -- before the
+    // current ones are used.
+    const uint32_t split = lane % 16, P = K / 16, base = lane & ~15u;
+    const uint16_t* xr = x_row + split * P;
+    const uint32_t batches = (P + 63) / 64, total = (count + 3) / 4 * batches;
+    auto request = [&](uint32_t index, uint4 (&piece)[8]) {
+        const uint32_t at = min(index / batches * 4 + lane / 16, count - 1), i0 = index % batches * 64;
+        const uint16_t* wr = w + uint64_t(list_s[wave][at]) * K + split * P;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) piece[q] = *reinterpret_cast<const uint4*>(wr + min(i0 + 8 * uint32_t(q), P - 8));
+    };
+    uint4 ahead[8];
+    if (total) request(0, ahead);
+    float c = 0;
+    for (uint32_t index = 0; index < total; ++index) {
+        uint4 piece[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) piece[q] = ahead[q];
+        if (index + 1 < total) request(index + 1, ahead);
+        const uint32_t i0 = index % batches * 64;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            if (i0 + 8 * uint32_t(q) >= P) break;
+            const uint4 xv4 = *reinterpret_cast<const uint4*>(xr + i0 + 8 * q);
+            const uint32_t ww[4] = {piece[q].x, piece[q].y, piece[q].z, piece[q].w}, xw[4] = {xv4.x, xv4.y, xv4.z, xv4.w};
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                c = __builtin_fmaf(__uint_as_float((k & 1) ? (xw[k / 2] & 0xffff0000u) : (xw[k / 2] << 16)),
+                                   __uint_as_float((k & 1) ? (ww[k / 2] & 0xffff0000u) : (ww[k / 2] << 16)), c);
+        }
+        if (index % batches + 1 == batches) {   // the expert's chains are complete: partials added 0..15, then the offset
+            const uint32_t at = index / batches * 4 + lane / 16;
+            float sum = 0;
+            for (uint32_t sidx = 0; sidx < 16; ++sidx) sum += __shfl(c, base + sidx);
+            if (split == 0 && at < count) { const uint32_t e = list_s[wave][at]; row_s[wave][e] = offsets ? sum + offsets[e] : sum; }
+            c = 0;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (uint32_t e = lane; e < E; e += 64) row[e] = row_s[wave][e];
+}
+// Router logits for the selection that follows: exact where it can matter, -inf elsewhere.  xb: the inputs as bf16 rows;
+// norms: rows + experts floats of scratch.  K % 128 == 0, experts <= 1024.
+void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, const void* w, const float* offsets, uint32_t T, uint32_t K,
+                           uint32_t E, uint32_t topk, float* norms, float* logits) {
+    const uint16_t* wb = static_cast<const uint16_t*>(w);
+    hipLaunchKernelGGL(row_norms_kernel, dim3((T + E + 3) / 4), dim3(256), 0, s, xb, T, wb, E, K, norms);
+    hipLaunchKernelGGL(router_product_kernel, dim3((E + 63) / 64, (T + 63) / 64), dim3(256), 0, s, xb, wb, T, E, K, offsets, logits);
+    hipLaunchKernelGGL(router_refine_kernel, dim3((T + 3) / 4), dim3(256), 4 * K * 2, s, xb, wb, offsets, norms, T, E, K, topk, logits);
 }
 
 void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status) {

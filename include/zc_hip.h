@@ -171,8 +171,8 @@ zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc
  * of zc_hip_moe_static_scratch_bytes() bytes (4 MiB) that every GPU the library runs on holds until the process ends;
  * its address is looked up once per device in zc_hip_create.  A call whose workspace
  * (zc_hip_moe_workspace_bytes(cfg, tokens)) does not fit is refused with ZC_INVALID_ARGUMENT and a message that names
- * both sizes.  The call itself performs no hipMalloc / hipFree and creates no stream or event; inputs, outputs and the
- * optional trace buffers are the caller's.  All calls on one GPU share the one array, whatever context they come
+ * both sizes.  The call itself performs no hipMalloc / hipFree and creates no stream or event, also while a recording
+ * is on (zc_hip_profile: this entry point records no row); inputs, outputs and the optional trace buffers are the caller's.  All calls on one GPU share the one array, whatever context they come
  * through: calls that can overlap on that GPU (two contexts, two threads) race; calls on one context's stream are
  * ordered and safe.  Nothing in the array has to start at zero (every word a kernel reads has been written by an earlier
  * kernel of the same call), so a call leaves the previous call's contents in place without reading them. */

@@ -116,6 +116,12 @@ def router_logits(w_bf16, x, tokens, K, E, offsets=None):
     return out
 
 
+def exp32(x):
+    """zco_expf elementwise: the fp32 exponential shared by the sigmoid and the routing softmax."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    return np.array([lib.zco_expf(float(v)) for v in x.ravel()], dtype=np.float32).reshape(x.shape)
+
+
 def route(logits, tokens, E, topk=10):
     logits = np.ascontiguousarray(logits, dtype=np.float32)
     ids = np.empty((tokens, topk), np.int32); w = np.empty((tokens, topk), np.float32)

@@ -32,9 +32,14 @@
  *                     the lane chain k = lane + 32 j (2^24 / 1 absorption rows)
  *   Q4 lane widths    exact closed forms that tell sixteen-element lane steps from
  *                     eight-element ones, and the every-32nd-block revisit, bit for bit
- *   route softmax WEIGHT BITS and the final simd_sum association of the affine
- *   dots: parity unpinned at bit level (only an Apple GPU run could pin them);
- *   sum-to-one and tolerance checks only.
+ *   route softmax     weight VALUES against a float64 softmax over the ten selected
+ *                     scores, relative 1e-6 (random, spread, tied and near-tied rows, the
+ *                     reference's ramp, a closed form with three finite scores); the
+ *                     swapped subtraction is shown to miss; zco_expf against double
+ *                     precision, relative 2e-7.  (qwen.metal:758-764)
+ *   Still unpinned at BIT level (only an Apple GPU run could pin them): the last
+ *   bits of the softmax weights (Metal fast::exp) and the final simd_sum association
+ *   of the affine dots.  Both sit far inside the 2e-3 layer tolerance.
  *
  * The callers' glue either side of the layer (tests/test_oracle_glue.py):
  *   softplus, unary   64-point captured softplus table, exact (…:881); ops 2 and 3

@@ -1,7 +1,7 @@
 // GPU tests of the C++ host shim, written the way the reference tests its own operator layer
 // (tests/test_qwen.cpp, cited per case): build tiny deterministic inputs through the Buffer
 // interface, run the operators, compare bytes.  The CPU oracle (oracle/zc_oracle.h) is the checker.
-#include "../../zerocool_amd/csrc/engine/engine.hpp"
+#include "reference_callers.hpp"
 #include "../../zerocool_amd/csrc/engine/route_trace.hpp"
 #include <unistd.h>
 #include "../../oracle/zc_oracle.h"

@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstring>
 #include <fstream>
+#include <sys/stat.h>
 #include <unistd.h>
 
 using namespace zerocool::engine;
@@ -30,6 +31,10 @@ int main() {
     CHECK(j.at("a").at(2).at("b").str() == "x\nA" && j.contains("t") && !j.contains("z") && j.at("big").u64() == 9007199254740991ull);
     CHECK_THROWS(Json::parse("{\"a\": }")); CHECK_THROWS(Json::parse("[1, 2")); CHECK_THROWS(Json::parse("{} x")); CHECK_THROWS(j.at("zz"));
     CHECK_THROWS(Json::parse("-1").u64()); CHECK_THROWS(Json::parse("1.5").u64());
+    // integers beyond 2^53 are kept exactly (nanosecond time stamps, storage.cpp:346-348 reads them with get<uint64_t>())
+    CHECK(Json::parse("1764000000123456789").u64() == 1764000000123456789ull && Json::parse("18446744073709551615").u64() == 18446744073709551615ull);
+    CHECK(Json::parse("[-3, 7]").at(0).number() == -3.0 && Json::parse("[-3, 7]").at(1).number() == 7.0 && Json::parse("1e3").u64() == 1000);
+    CHECK_THROWS(Json::parse("18446744073709551616").u64());            // one past 2^64 - 1: a double, and not an exact integer below 2^53
 
     std::printf("record layout\n");
     const auto layout = expert_layout(s);
@@ -123,6 +128,65 @@ int main() {
     CHECK_THROWS(PreparedExperts(dir, s));                                // the bytes are back, the receipt's time stamps are stale
     verify_prepared_experts(dir);
     { PreparedExperts again(dir, s); CHECK(again.layers() == 2); }
+    std::printf("prepared directory in the reference's own layout: more files than expert files, integer time stamps\n");
+    {
+        // What the reference's tools leave (prepare.cpp:262-300 for the manifest, storage.cpp:337-354 for what is read back):
+        // "files" lists every prepared file -- the per-layer expert files AND the n-gram tables -- and the receipt holds
+        // size / device / inode / mtime_ns / ctime_ns as JSON integers, with keys this reader does not know beside them.
+        const auto ref_dir = root / "reference_layout";
+        write_prepared_experts(ref_dir, s, 2, fill);
+        spit(ref_dir / "ngram-000.bin", std::string(100, 'n')); spit(ref_dir / "ngram-001.bin", std::string(90, 'm'));
+        const Json made = Json::parse(slurp(ref_dir / "manifest.json"));
+        std::string m = slurp(ref_dir / "manifest.json");
+        const uint64_t expert_bytes_total = made.at("prepared_bytes").u64();
+        m = replaced(m, "\n ],\n \"prepared_bytes\": " + std::to_string(expert_bytes_total),
+                     ",\n  {\"path\": \"ngram-000.bin\", \"size\": 100, \"sha256\": \"" + sha256_hex(std::string(100, 'n')) + "\"}"
+                     ",\n  {\"path\": \"ngram-001.bin\", \"size\": 90, \"sha256\": \"" + sha256_hex(std::string(90, 'm')) + "\"}"
+                     "\n ],\n \"ngrams\": [{\"order\": 0, \"file\": \"ngram-000.bin\"}, {\"order\": 1, \"file\": \"ngram-001.bin\"}],"
+                     "\n \"source_files\": {\"model.safetensors\": \"00\"},\n \"prepared_bytes\": " + std::to_string(expert_bytes_total + 190));
+        spit(ref_dir / "manifest.json", m);
+        const Json listed = Json::parse(m);
+        CHECK(listed.at("files").size() == 4 && listed.at("experts").size() == 2);
+        const auto receipt_with = [&](bool integers) {
+            std::string r = "{\n  \"schema\": 1,\n  \"verified_at\": 1764000000,\n  \"manifest_sha256\": \"" + sha256_hex(m) + "\",\n  \"source_revision\": \"synthetic\",\n  \"files\": {";
+            for (size_t i = 0; i < listed.at("files").size(); ++i) {
+                const std::string name = listed.at("files").at(i).at("path").str();
+                struct stat st{}; ::stat((ref_dir / name).c_str(), &st);
+                const std::string mt = std::to_string(uint64_t(st.st_mtim.tv_sec) * 1000000000ull + uint64_t(st.st_mtim.tv_nsec));
+                const std::string ct = std::to_string(uint64_t(st.st_ctim.tv_sec) * 1000000000ull + uint64_t(st.st_ctim.tv_nsec));
+                const std::string q = integers ? "" : "\"";
+                r += std::string(i ? "," : "") + "\n    \"" + name + "\": {\n      \"size\": " + std::to_string(st.st_size) + ",\n      \"device\": " + std::to_string(st.st_dev) +
+                     ",\n      \"inode\": " + std::to_string(st.st_ino) + ",\n      \"mtime_ns\": " + q + mt + q + ",\n      \"ctime_ns\": " + q + ct + q +
+                     ",\n      \"sha256\": \"" + listed.at("files").at(i).at("sha256").str() + "\"\n    }";
+            }
+            return r + "\n  }\n}\n";
+        };
+        spit(ref_dir / "verification.json", receipt_with(true));
+        {
+            PreparedExperts p(ref_dir, s);
+            std::vector<std::byte> record(bytes);
+            p.expert({1, 6}, record);
+            CHECK(p.layers() == 2 && record[777] == value({1, 6}, 777));
+        }
+        spit(ref_dir / "verification.json", receipt_with(false));       // stamps as decimal strings: still read
+        { PreparedExperts p(ref_dir, s); CHECK(p.layers() == 2); }
+        // an integer stamp that is off by one nanosecond is a changed file: no rounding through a double hides it
+        struct stat st{}; ::stat((ref_dir / "ngram-001.bin").c_str(), &st);
+        const uint64_t mt = uint64_t(st.st_mtim.tv_sec) * 1000000000ull + uint64_t(st.st_mtim.tv_nsec);
+        const std::string good = receipt_with(true);
+        spit(ref_dir / "verification.json", replaced(good, "\"mtime_ns\": " + std::to_string(mt) + ",\n      \"ctime_ns\"", "\"mtime_ns\": " + std::to_string(mt + 1) + ",\n      \"ctime_ns\""));
+        if (mt > (1ull << 53)) CHECK_THROWS(PreparedExperts(ref_dir, s));
+        // the receipt this library writes holds integers too
+        verify_prepared_experts(ref_dir);
+        const Json own = Json::parse(slurp(ref_dir / "verification.json"));
+        CHECK(std::holds_alternative<uint64_t>(own.at("files").at("ngram-000.bin").at("mtime_ns").value));
+        { PreparedExperts p(ref_dir, s); CHECK(p.layers() == 2); }
+        // an expert range that names a file the manifest does not list is still refused
+        spit(ref_dir / "manifest.json", replaced(m, "\"path\": \"experts-01.bin\"", "\"path\": \"experts-1.bin\""));
+        std::filesystem::copy_file(ref_dir / "experts-01.bin", ref_dir / "experts-1.bin");
+        verify_prepared_experts(ref_dir);
+        CHECK_THROWS(PreparedExperts(ref_dir, s));
+    }
     std::filesystem::resize_file(dir / "experts-01.bin", std::filesystem::file_size(dir / "experts-01.bin") - 1); CHECK_THROWS(PreparedExperts(dir, s));
     CHECK_THROWS(verify_prepared_experts(dir));
     std::filesystem::remove(dir / "experts-01.bin"); CHECK_THROWS(PreparedExperts(dir, s));

@@ -149,6 +149,18 @@ def test_stand_in_stack_shape(ctx):  # hidden 3072 / intermediate 1024, two laye
     check_stack(ctx, workload.config("F"), 2, [1, 8])
 
 
+def test_benchmark_shapes_through_the_single_launch_kernels(ctx):
+    # The exact shapes the benchmark quotes, 512 experts and top-10, each through the kernel its figure comes from:
+    # the single layer (hidden 2048, intermediate 512) with N(0, 0.5) router offsets at 1 token (one-token kernel),
+    # 8 (two to eight), 32 and 64 (nine to sixty-four); the mixed 4/8-bit artifact at 1 and 16 tokens.
+    check_stack(ctx, workload.config("S"), 1, [1, 8, 32, 64], seed=61, skew=("normal", 0.5))
+    check_stack(ctx, workload.config("S-mixed"), 1, [1, 16], seed=67, skew=("normal", 0.5))
+
+
+def test_stand_in_stack_six_layers(ctx):  # the 48-layer stack's shape and Zipf(1.1) routers, six layers deep, 1 and 8 tokens
+    check_stack(ctx, workload.config("F"), 6, [1, 8], seed=71)
+
+
 def test_stack_reports_invalid_router_output(ctx):
     cfg = workload.tiny_config(hidden=2048, experts=32, topk=4, inter=512)
     layers = [workload.LayerWeights(ctx, cfg, 77 + l, None) for l in range(2)]

@@ -186,6 +186,63 @@ def test_route_ties_and_exceptional_scores():  # :755-781
         assert w2.tobytes() == w[offset:offset + count].tobytes()
 
 
+def _softmax64(scores):
+    """w_j = exp(s_j - s_0) / sum_i exp(s_i - s_0) in double precision (qwen.metal:758-764)."""
+    s = np.asarray(scores, dtype=np.float64)
+    e = np.exp(s - s[0])
+    return e / e.sum()
+
+
+def test_route_weight_values_are_the_softmax_of_the_selected_scores():  # qwen.metal:758-764
+    """The weight VALUES against an independent float64 softmax over the ten selected scores, relative 1e-6.
+    A swapped subtraction (exp(s_0 - s_j)), a base other than e, a sum over more than the ten, or weights
+    left in selection order of another row each miss this by orders of magnitude."""
+    rng = np.random.default_rng(2718)
+    rows = [np.array([i % 41 - 100 for i in range(512)], dtype=np.float32),        # the reference's ramp, ties of 12 or 13
+            rng.standard_normal(512).astype(np.float32),
+            (rng.standard_normal(512) * 4).astype(np.float32),                     # spread: weights over many decades
+            np.round(rng.standard_normal(512) * 2).astype(np.float32),             # heavy exact ties
+            (rng.standard_normal(512) * 0.01 + 7).astype(np.float32),              # near ties, nonzero base
+            np.where(np.arange(512) % 7 == 0, np.float32(3.5), rng.standard_normal(512).astype(np.float32))]
+    v = np.stack(rows).astype(np.float32)
+    ids, w = oracle.route(v, v.shape[0], 512)
+    for t in range(v.shape[0]):
+        assert list(ids[t]) == _stable_top([float(a) for a in v[t]]), t
+        scores = v[t][ids[t]]
+        assert (np.diff(scores) <= 0).all()                                        # descending, so scores[0] is the base
+        want = _softmax64(scores)
+        got = w[t].astype(np.float64)
+        assert np.max(np.abs(got - want) / want) <= 1e-6, (t, got, want)
+        wrong = np.exp(scores[0].astype(np.float64) - scores.astype(np.float64))
+        wrong /= wrong.sum()
+        if scores[0] != scores[-1]:
+            assert np.max(np.abs(got - wrong) / wrong) > 1e-3                       # the swapped subtraction is far away
+    # eight selected scores of 3.5 or ties at the top: equal scores give equal weights, bit for bit
+    t = 5
+    assert len({bits(x) for x in w[t]}) == 1 and w[t][0] == pytest.approx(0.1, rel=1e-6)
+    # fewer than ten finite scores: the missing slots carry weight exactly 0 (exp(-inf)) and the rest still sum to 1
+    few = np.full((1, 512), -np.inf, np.float32)
+    few[0, [5, 77, 300]] = [1.0, 0.0, -1.0]
+    ids, w = oracle.route(few, 1, 512)
+    assert list(ids[0]) == [5, 77, 300] + [-1] * 7
+    assert (w[0, 3:] == 0).all()
+    e = math.e
+    want = np.array([e * e, e, 1.0]) / (e * e + e + 1.0)                            # closed form
+    assert np.max(np.abs(w[0, :3].astype(np.float64) - want) / want) <= 1e-6
+
+
+def test_exp32_against_double_precision():
+    """The fp32 exponential shared by the oracle and the kernels, over the range the softmax uses (arguments <= 0)
+    and the activations use, against libm's double exp: relative 2e-7 (about two units in the last place)."""
+    xs = np.concatenate([-np.linspace(0, 87, 2001), np.linspace(0, 20, 501), [-0.0, -1e-8, -103.0, -200.0]]).astype(np.float32)
+    got = oracle.exp32(xs).astype(np.float64)
+    want = np.exp(xs.astype(np.float64))
+    normal = want > 1.2e-38
+    assert np.max(np.abs(got[normal] - want[normal]) / want[normal]) <= 2e-7
+    assert (got[~normal] <= 1.2e-38).all() and (got >= 0).all()
+    assert oracle.exp32(np.array([0.0], np.float32))[0] == 1.0
+
+
 def test_moe_sum_midpoint():  # :827-842
     m = G["moe_sum"]; H = 2560
     e = np.zeros((10, H), np.float32); e[:, 0] = np.array(m["values"], dtype=np.float32)

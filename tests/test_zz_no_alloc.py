@@ -2,6 +2,7 @@
 workspace in the library's static device array.  Checked through the C ABI against zc_hip_moe_forward on the same
 inputs, byte for byte (outputs and every traced intermediate), on two calls in a row, the second with a smaller input,
 so that the second call runs over whatever the first one left in the shared array."""
+import ctypes as C
 import numpy as np
 import pytest
 import zerocool_amd as z
@@ -61,4 +62,43 @@ def test_static_scratch_layer_equals_the_workspace_layer(ctx, name):
         ctx.moe_forward_static(cfg, weights.layer, x, big, out)
     assert "bytes of scratch" in str(err.value) and str(4 << 20) in str(err.value)
     for b in (x, out, weights.router, weights.shared_gate, weights.shared_record, weights.records):
+        ctx.free(b)
+
+
+def _free_bytes():
+    """Free device memory as the HIP runtime reports it (hipMemGetInfo of the runtime this process has loaded)."""
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_static_scratch_layer_allocates_nothing_while_a_recording_is_on(ctx):
+    # With per-operator timing recorded (zc_hip_profile) every ordinary operator call creates two events and a row.  The
+    # allocation-free entry point must not: no row, no change in the library's own count, none in the runtime's free memory.
+    cfg = workload.tiny_config()
+    weights = workload.LayerWeights(ctx, cfg, 57, ("normal", 0.5))
+    T = 5
+    x = workload.hidden_rows(ctx, T, cfg.hidden, 571)
+    out, want = ctx.alloc(T * cfg.hidden * 4), ctx.alloc(T * cfg.hidden * 4)
+    ws = ctx.alloc(ctx.moe_workspace_bytes(cfg, T))
+    ctx.moe_forward_static(cfg, weights.layer, x, T, out); ctx.moe_check()     # first use of every kernel is behind us
+    ctx.profile(True)
+    try:
+        ctx.moe_forward(cfg, weights.layer, x, T, want, ws); ctx.moe_check()
+        rows = len(ctx.stats()["profile"]["rows"])
+        assert rows >= 1
+        allocated, free = ctx.allocated, _free_bytes()
+        for _ in range(3):
+            ctx.moe_forward_static(cfg, weights.layer, x, T, out)
+        ctx.moe_check()
+        assert ctx.allocated == allocated and _free_bytes() == free
+        stats = ctx.stats()["profile"]
+        assert len(stats["rows"]) == rows and all(r["operator"] != "moe_forward_static" for r in stats["rows"])
+        ctx.moe_forward(cfg, weights.layer, x, T, want, ws); ctx.moe_check()   # the recording itself still works afterwards
+        assert len(ctx.stats()["profile"]["rows"]) == rows + 1
+    finally:
+        ctx.profile(False)
+    assert out.numpy(np.uint8).tobytes() == want.numpy(np.uint8).tobytes()
+    for b in (x, out, want, ws, weights.router, weights.shared_gate, weights.shared_record, weights.records):
         ctx.free(b)

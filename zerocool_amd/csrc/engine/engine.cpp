@@ -248,86 +248,10 @@ Linear expert_linear(const MoeShape& shape, const Buf& record, int projection, b
             {record, uint64_t(reinterpret_cast<uintptr_t>(l.biases) - base)}, l.input, l.output, l.group, 0, true, l.bits};
 }
 
-// ---- The reference's CALLERS of the operator layer, restated (not product logic) --------------------------------------
-// encode_expert_rows (pipeline.cpp:7-31) and moe (model.cpp:431-557) below are the two reference functions that sit
-// ABOVE the drop-in boundary.  Their signatures are part of the boundary and their bodies follow the reference's order
-// of operator calls on purpose: they exist so that the reference's own tests of the path (tests/test_qwen.cpp:1087-1099,
-// 1500-1600) can be restated against this library call for call, and so that the shim can be exercised the way the
-// engine would exercise it.  Everything the library adds of its own is below the C ABI; the fused, device-resident
-// orchestration is zc_hip_moe_forward / zc_hip_stack_decode (moe_resident further down).
-
-// pipeline.cpp:7-31
-void encode_expert_rows(Metal& gpu, const Buf& record, const Buf& input, const Buf& output, std::span<const int> positions,
-                        uint32_t tokens, uint32_t chunk, bool direct, int layer, uint32_t offset, const std::atomic<bool>* cancel) {
-    const auto& s = gpu.shape();
-    if (!chunk || chunk > 256 || !tokens || tokens > 1024 || !input || !output || input->bytes < uint64_t(tokens) * s.hidden * 4 ||
-        output->bytes < uint64_t(tokens) * s.topk * s.hidden * 4)
-        throw std::invalid_argument("invalid expert row encoding geometry");
-    for (auto p : positions) if (p < 0 || uint64_t(p) >= uint64_t(tokens) * s.topk) throw std::invalid_argument("expert destination outside input");
-    auto ints = [&](std::span<const int> values) { auto b = gpu.allocate(values.size_bytes()); std::memcpy(b->data, values.data(), values.size_bytes()); return b; };
-    direct = direct || gpu.direct_rows();
-    for (size_t at_ = 0; at_ < positions.size(); at_ += chunk) {
-        if (cancel && cancel->load()) throw std::runtime_error("generation cancelled");
-        const auto pos = positions.subspan(at_, std::min<size_t>(chunk, positions.size() - at_));
-        const auto n = uint32_t(pos.size());
-        gpu.label("routed_expert", layer, n, offset);
-        std::vector<int> rows; rows.reserve(n);
-        for (auto p : pos) rows.push_back(p / int(s.topk));
-        auto rowsbuf = tokens == 1 ? Buf{} : ints(rows);
-        auto activated = gpu.gated_linear(expert_linear(s, record, 0), expert_linear(s, record, 1), input, n, rowsbuf);
-        if (tokens == 1 && direct) gpu.linear_into(expert_linear(s, record, 2), activated, 1, {output, uint64_t(pos[0]) * s.hidden * 4});
-        else {
-            auto posbuf = ints(pos);
-            auto down = gpu.linear(expert_linear(s, record, 2), activated, n);
-            gpu.dispatch("scatter_experts", {{down}, {posbuf}, {output}}, {n}, s.hidden, n);
-        }
-    }
-}
-
-// model.cpp:431-557 without the cache, prefetch, trace and timing branches
-Buf moe(Metal& gpu, const MoeLayerWeights& w, const Buf& x, uint32_t tokens, const std::atomic<bool>* cancel, uint32_t chunk,
-        const Buf& predict, PredictionStats* prediction) {
-    const auto& s = gpu.shape();
-    auto cancelled = [&] { if (cancel && cancel->load()) throw std::runtime_error("generation cancelled"); };
-    auto router = gpu.linear(w.router, x, tokens, true);
-    auto ids = gpu.allocate(uint64_t(tokens) * s.topk * 4), weights = gpu.allocate(uint64_t(tokens) * s.topk * 4);
-    gpu.route(router, ids, weights, tokens);
-    Buf predicted;
-    if (predict && w.next_router.weight.buffer) {   // model.cpp:437-445: shares this readback, never feeds the arithmetic
-        if (predict->bytes < uint64_t(tokens) * s.hidden * 4) throw std::invalid_argument("invalid prediction input");
-        auto logits = gpu.linear(w.next_router, predict, tokens, true);
-        predicted = gpu.allocate(uint64_t(tokens) * s.topk * 4);
-        gpu.route(logits, predicted, gpu.allocate(uint64_t(tokens) * s.topk * 4), tokens);
-    }
-    gpu.finish(); cancelled();
-    if (predicted) {                                // model.cpp:489-500: the first token's guesses, distinct, depth-limited
-        PredictionStats local; PredictionStats& st = prediction ? *prediction : local; st = {};
-        const auto guesses = std::span<const int>(reinterpret_cast<const int*>(predicted->data), s.topk);
-        for (int e : guesses)
-            if (e >= 0 && e < int(s.experts) && std::find(st.experts.begin(), st.experts.end(), e) == st.experts.end()) {
-                const bool issued = st.experts.size() < w.prefetch_depth && w.prefetch && w.prefetch(uint32_t(e));
-                st.experts.push_back(e); ++st.guesses; st.issued += issued;
-            }
-    }
-    std::vector<std::vector<int>> positions(s.experts);
-    auto raw = std::span<const int>(reinterpret_cast<const int*>(ids->data), size_t(tokens) * s.topk);
-    for (uint32_t p = 0; p < tokens * s.topk; ++p) {
-        if (raw[p] < 0 || raw[p] >= int(s.experts)) throw std::runtime_error("invalid router output");
-        positions[raw[p]].push_back(int(p));
-    }
-    auto expert_out = gpu.allocate(uint64_t(tokens) * s.topk * s.hidden * 4);
-    auto shared_activation = gpu.gated_linear(expert_linear(s, w.shared_record, 0, true), expert_linear(s, w.shared_record, 1, true), x, tokens);
-    auto shared = gpu.linear(expert_linear(s, w.shared_record, 2, true), shared_activation, tokens);
-    auto gate = gpu.linear(w.shared_gate, x, tokens);
-    for (uint32_t e = 0; e < s.experts; ++e) {
-        if (positions[e].empty()) continue;
-        cancelled();
-        encode_expert_rows(gpu, w.record(e), x, expert_out, positions[e], tokens, chunk, true, 0, 0, cancel);
-    }
-    auto out = gpu.allocate(uint64_t(tokens) * s.hidden * 4);
-    gpu.dispatch("moe_sum", {{expert_out}, {weights}, {shared}, {gate}, {out}}, {tokens}, s.hidden, tokens);
-    return out;
-}
+// Model::moe (model.cpp:431-557) as ONE enqueue: routing, dispatch, expert products and the combine stay on the device
+// (zc_hip_moe_forward).  The reference's own host-side orchestration of the same operators (one readback of the ids per
+// layer, encode_expert_rows per expert) is what an engine keeps when it only swaps the operator class; it is restated
+// next to the C++ tests, which drive this library through it call for call.
 Buf moe_resident(Metal& gpu, const MoeLayerWeights& w, const Buf& records, uint64_t stride, const Buf& x, uint32_t tokens) {
     const auto& s = gpu.shape();
     if (!records || !x || !tokens || x->bytes < uint64_t(tokens) * s.hidden * 4 || records->bytes < checked_mul(stride, s.experts))
@@ -343,7 +267,6 @@ Buf moe_resident(Metal& gpu, const MoeLayerWeights& w, const Buf& records, uint6
     return out;
 }
 
-// ---- end of the restated callers ----------------------------------------------------------------------------------------
 
 // ---- expert cache (storage.cpp:525-725 over zc_hip_store_*)
 ExpertCache::ExpertCache(Metal& gpu, uint32_t layers, size_t slots) : gpu_(gpu), record_bytes_(gpu.shape().expert_bytes()) {

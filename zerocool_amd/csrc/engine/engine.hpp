@@ -115,11 +115,6 @@ private:
 // metal.hpp:154, metal.mm:1124-1129
 Linear expert_linear(const MoeShape& shape, const Buf& record, int projection, bool shared = false);
 
-// pipeline.hpp:6-8, pipeline.cpp:7-31
-void encode_expert_rows(Metal& gpu, const Buf& record, const Buf& input, const Buf& output, std::span<const int> positions,
-                        uint32_t tokens, uint32_t chunk, bool direct, int layer, uint32_t offset,
-                        const std::atomic<bool>* cancel = nullptr);
-
 // storage.hpp:168-172, 183-192, 198-269: the expert cache, with the reference's names.  The records' home is pinned host
 // memory (home()), the slots are HBM, fills run on the store's side stream (zc_hip_store_*).  A Lease pins its slot
 // until it is destroyed: keep it until the GPU work that reads the slot has finished, as the reference does.
@@ -175,18 +170,14 @@ struct MoeLayerWeights {
     Linear shared_gate;       // [1][hidden] BF16 (model.cpp:485)
     Buf shared_record;        // gate, up, down of the shared expert
     std::function<Buf(uint32_t expert)> record;   // the expert store: record of a routed expert
-    // Next-layer prediction (model.cpp:437-445, 489-500), a cache hint only that never feeds model arithmetic: when
-    // moe() is given a `predict` input, the NEXT layer's router runs on it beside this layer's, its top-k ids come back
-    // with the same readback, and prefetch(expert) is called for each distinct guess, at most prefetch_depth of them.
+    // Next-layer prediction (model.cpp:437-445, 489-500), a cache hint only that never feeds model arithmetic: a caller
+    // that has a `predict` input runs the NEXT layer's router on it beside this layer's, reads its top-k ids back with
+    // the same readback, and calls prefetch(expert) for each distinct guess, at most prefetch_depth of them.
     Linear next_router;                             // [experts][hidden] BF16 of layer + 1; unused when empty
     std::function<bool(uint32_t expert)> prefetch;  // e.g. ExpertCache::prefetch({layer + 1, expert}); returns "issued"
     uint32_t prefetch_depth = 10;
 };
-struct PredictionStats { uint32_t guesses = 0, issued = 0; std::vector<int> experts; };
-// model.hpp:156, model.cpp:431-557: the reference's orchestration, one CPU readback of the ids per call.
-Buf moe(Metal& gpu, const MoeLayerWeights& weights, const Buf& x, uint32_t tokens,
-        const std::atomic<bool>* cancel = nullptr, uint32_t chunk = 128, const Buf& predict = {}, PredictionStats* prediction = nullptr);
-// The same layer as one enqueue with routing and dispatch kept on the device (zc_hip_moe_forward);
+// The layer as one enqueue with routing and dispatch kept on the device (zc_hip_moe_forward);
 // records must be one buffer of experts * stride bytes.
 Buf moe_resident(Metal& gpu, const MoeLayerWeights& weights, const Buf& records, uint64_t stride, const Buf& x, uint32_t tokens);
 

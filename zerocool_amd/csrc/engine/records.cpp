@@ -75,7 +75,11 @@ struct Parser {
             const size_t start = i;
             while (i < s.size() && (std::isdigit(static_cast<unsigned char>(s[i])) || s[i] == '-' || s[i] == '+' || s[i] == '.' || s[i] == 'e' || s[i] == 'E')) ++i;
             if (start == i) fail("unexpected character");
-            const std::string text(s.substr(start, i - start)); char* end = nullptr;
+            const std::string text(s.substr(start, i - start));
+            uint64_t whole = 0;
+            const auto r = std::from_chars(text.data(), text.data() + text.size(), whole);
+            if (r.ec == std::errc() && r.ptr == text.data() + text.size() && std::isdigit(static_cast<unsigned char>(text[0]))) { j.value = whole; return j; }
+            char* end = nullptr;
             const double v = std::strtod(text.c_str(), &end);
             if (!end || *end) fail("bad number");
             j.value = v;
@@ -114,9 +118,11 @@ FileIdentity identity_of(const std::filesystem::path& path) {
             uint64_t(st.st_ctim.tv_sec) * 1000000000ull + uint64_t(st.st_ctim.tv_nsec)};
 }
 bool plain_filename(const std::string& name) { return !name.empty() && std::filesystem::path(name).filename() == name && name != "." && name != ".."; }
-// Nanosecond stamps exceed 2^53: the receipt keeps them as decimal strings.
-std::string quoted(uint64_t v) { return "\"" + std::to_string(v) + "\""; }
+// Nanosecond stamps exceed 2^53.  The reference writes them as JSON integers (scripts/qwen/verify_checkpoint.py:18-22,
+// read with get<uint64_t>() in storage.cpp:346-348) and so does this writer; the parser keeps such integers exactly.
+// A receipt that holds them as decimal strings (what earlier versions of this library wrote) is still read.
 uint64_t stamp(const Json& j) {
+    if (std::holds_alternative<uint64_t>(j.value)) return j.u64();
     const std::string& s = j.str(); uint64_t v = 0;
     const auto r = std::from_chars(s.data(), s.data() + s.size(), v);
     if (r.ec != std::errc() || r.ptr != s.data() + s.size()) throw std::runtime_error("invalid time stamp in the verification receipt");
@@ -193,7 +199,13 @@ const Json& Json::at(const std::string& key) const { const auto& o = object(); a
 const Json& Json::at(size_t index) const { if (auto* a = std::get_if<Array>(&value); a && index < a->size()) return (*a)[index]; throw std::out_of_range("JSON index out of range"); }
 bool Json::contains(const std::string& key) const { auto* o = std::get_if<Object>(&value); return o && o->count(key); }
 size_t Json::size() const { if (auto* a = std::get_if<Array>(&value)) return a->size(); if (auto* o = std::get_if<Object>(&value)) return o->size(); return 0; }
+double Json::number() const {
+    if (auto* w = std::get_if<uint64_t>(&value)) return double(*w);
+    if (auto* d = std::get_if<double>(&value)) return *d;
+    throw std::runtime_error("JSON value is not a number");
+}
 uint64_t Json::u64() const {
+    if (auto* w = std::get_if<uint64_t>(&value)) return *w;
     if (auto* d = std::get_if<double>(&value); d && *d >= 0 && *d < 9007199254740992.0 && std::floor(*d) == *d) return uint64_t(*d);
     throw std::runtime_error("JSON value is not a non-negative integer");
 }
@@ -246,7 +258,9 @@ PreparedExperts::PreparedExperts(const std::filesystem::path& dir, const MoeShap
             throw std::runtime_error("prepared file changed since verification: " + name);
         total += now.size;
     }
-    if (m.at("prepared_bytes").u64() != total || listed.size() != m.at("experts").size()) throw std::runtime_error("incomplete prepared layout");   // storage.cpp:351-354
+    // The reference's manifest lists more than the expert files (one per layer plus its 128 n-gram tables, storage.cpp:351);
+    // what this reader needs is that the listed bytes add up and, below, that every expert range names a listed file.
+    if (m.at("prepared_bytes").u64() != total) throw std::runtime_error("incomplete prepared layout");   // storage.cpp:351-354
     const auto layout = expert_layout(shape);
     if (m.at("expert_layout").size() != 9) throw std::runtime_error("incomplete prepared layout");      // storage.cpp:352-354
     uint64_t offset = 0;
@@ -391,7 +405,7 @@ void verify_prepared_experts(const std::filesystem::path& dir) {
         if (now.size != entry.at("size").u64() || digest != entry.at("sha256").str())
             throw std::runtime_error("prepared file differs from its manifest entry: " + name);
         r << (i ? "," : "") << "\n  \"" << name << "\": {\"sha256\": \"" << digest << "\", \"size\": " << now.size << ", \"device\": " << now.device
-          << ", \"inode\": " << now.inode << ", \"mtime_ns\": " << quoted(now.mtime_ns) << ", \"ctime_ns\": " << quoted(now.ctime_ns) << "}";
+          << ", \"inode\": " << now.inode << ", \"mtime_ns\": " << now.mtime_ns << ", \"ctime_ns\": " << now.ctime_ns << "}";
     }
     r << "\n }\n}\n";
     std::ofstream f(dir / "verification.json", std::ios::trunc); f << r.str(); f.close();

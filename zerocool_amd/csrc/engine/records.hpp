@@ -24,13 +24,16 @@ namespace zerocool::engine {
 struct Json {
     using Array = std::vector<Json>;
     using Object = std::map<std::string, Json>;
-    std::variant<std::nullptr_t, bool, double, std::string, Array, Object> value;
+    // A number written as a plain run of digits is kept exactly (nanosecond stamps, sizes and offsets exceed 2^53);
+    // everything else numeric (a sign, a fraction, an exponent) is a double.
+    std::variant<std::nullptr_t, bool, double, std::string, Array, Object, uint64_t> value;
     static Json parse(std::string_view text);
     const Json& at(const std::string& key) const;      // std::out_of_range when absent or not an object
     const Json& at(size_t index) const;
     bool contains(const std::string& key) const;
     size_t size() const;
     uint64_t u64() const;                               // std::runtime_error unless a non-negative integer
+    double number() const;                              // either kind of number; std::runtime_error otherwise
     const std::string& str() const;
     const Object& object() const;
 };

@@ -156,7 +156,7 @@ inline TraceSummary read_route_trace(const std::filesystem::path& path) {
             out.forwards.push_back(std::move(fw));
         } else if (event == "routes") {
             if (out.forwards.empty() || d.at("layer").u64() != out.forwards.back().routes.size()) throw std::runtime_error("route pass does not match active forward");
-            std::vector<int> ids; for (size_t i = 0; i < d.at("routes").size(); ++i) ids.push_back(int(std::get<double>(d.at("routes").at(i).value)));
+            std::vector<int> ids; for (size_t i = 0; i < d.at("routes").size(); ++i) ids.push_back(int(d.at("routes").at(i).number()));
             out.forwards.back().routes.push_back(std::move(ids));
         } else if (event == "forward_commit") { if (out.forwards.empty()) throw std::runtime_error("commit without a forward"); out.forwards.back().committed = true; }
         else if (event == "trace_end") out.complete = d.at("status").str() == "complete";

@@ -87,6 +87,13 @@ struct Timed {
         if (end) (void)hipEventRecord(end, ctx->stream);
     }
 };
+// Keeps a recording off for one call: the operators inside see a call already in progress and record nothing, so the
+// call creates no event and touches no host container.
+struct Untimed {
+    zc_hip_ctx* ctx;
+    explicit Untimed(zc_hip_ctx* c) : ctx(c && c->profile ? c : nullptr) { if (ctx) ++ctx->profile_depth; }
+    ~Untimed() { if (ctx) --ctx->profile_depth; }
+};
 void json_text(std::string& out, const std::string& text) {
     out += '"';
     for (const char c : text) {
@@ -562,10 +569,11 @@ uint64_t zc_hip_moe_workspace_bytes(const zc_moe_config* cfg, uint32_t tokens) {
 }
 uint64_t zc_hip_moe_static_scratch_bytes(void) { return kStaticScratchBytes; }
 // zc_hip_moe_forward with its workspace in the static scratch array of the context's device.  Nothing on this path
-// allocates or frees: no hipMalloc / hipFree / hipHostMalloc, no stream or event creation, no host containers.
+// allocates or frees: no hipMalloc / hipFree / hipHostMalloc, no stream or event creation, no host containers --
+// also while a recording is on (zc_hip_profile): this call records no row, and neither do the operators inside it.
 zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_moe_layer* l, const float* x, uint32_t T,
                                     float* out, const zc_moe_trace* trace) {
-    Timed timed(ctx, "moe_forward_static");
+    Untimed untimed(ctx);
     if (const zc_status s = validate_config(c)) return s;
     ZC_REQUIRE(ctx && T, "invalid MoE layer buffers");
     ZC_REQUIRE(ctx->static_scratch, "the static scratch array was not located for this device");
@@ -1070,7 +1078,10 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
             ZC_HIP(hipStreamSynchronize(ctx->stream));
             int32_t status = 0;
             ZC_HIP(hipMemcpy(&status, ctx->moe_status, 4, hipMemcpyDeviceToHost));
-            if (!status)   // ids of a launch that gave up are not routes
+            // Only a launch that gave up waiting (bit 2) has no routes to observe; the other bits (an unroutable row, an
+            // input that is not BF16-valued) are sticky reports of this or an earlier call, and an id outside the
+            // expert range is skipped one by one inside the observation.
+            if (!(status & 2))
                 if (const zc_status s = zc_hip_store_table_observe_layers(st->store, st->route_ids_host, uint32_t(per_layer))) return s;
         }
         return ZC_OK;

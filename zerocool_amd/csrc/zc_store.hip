@@ -336,6 +336,7 @@ static zc_status observe_layers(zc_hip_store* s, uint32_t first_layer, uint32_t 
             std::sort(distinct.begin(), distinct.end());
             distinct.erase(std::unique(distinct.begin(), distinct.end()), distinct.end());
             for (const int32_t e : distinct) {
+                if (e == -1) continue;   // the router's padding for a row with fewer finite logits than picks: no record was read
                 if (e < 0 || uint32_t(e) >= s->experts) throw std::out_of_range("invalid expert id");
                 const uint64_t key = key_of(s, first_layer + l, uint32_t(e));
                 const uint8_t* at = s->mirror[key];

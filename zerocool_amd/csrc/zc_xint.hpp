@@ -371,12 +371,6 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
     }
 }
 
-// (timing experiments only: -DZC_TIMING_NO_WEIGHTS feeds the tile engines register constants instead of weights)
-#ifdef ZC_TIMING_NO_WEIGHTS
-#define ZC_TILE_LOAD(p, i) make_uint4(0x12345678u + uint32_t(i), 0x9abcdef0u ^ lane, 0x3c003c00u, 0x0f1e2d3cu + uint32_t(i))
-#else
-#define ZC_TILE_LOAD(p, i) ldg_u4(p, i)
-#endif
 // The literal fp32 chain of one block (reference: qwen.metal:52-57) from the block's two raw code words (nibble i of word w
 // is element 8 w + i) and the block's sixteen BF16 inputs in LDS.  The four quads' nested sums do not depend on each other:
 // all sixteen inputs are read at once and the four chains run side by side, then the quad sums are added in order -- one
@@ -419,8 +413,8 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
     const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
     uint4 ring[R], sring, bring;
 #pragma unroll
-    for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, j * 4);
-    sring = ZC_TILE_LOAD(s_row, 0); bring = ZC_TILE_LOAD(b_row, 0);
+    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
+    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
     float acc[NTOK][4][2];
 #pragma unroll
     for (int t = 0; t < NTOK; ++t)
@@ -439,8 +433,8 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
         const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
         if (d0 + R < spans) {
 #pragma unroll
-            for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, (d0 + j + R) * 4);
-            sring = ZC_TILE_LOAD(s_row, (d0 + R) / 4); bring = ZC_TILE_LOAD(b_row, (d0 + R) / 4);
+            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
+            sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4);
         }
         // the unsafe bits of this body's blocks, per token: blocks 8d + 2G + h of spans d0 .. d0+3 sit in mask word d0/4,
         // moved down so that bits 8j, 8j+1 are the lane's two blocks of span j
@@ -467,7 +461,6 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
                 dot[t][0] = float(xint_digits(r0)) * fi.x; bsum[t][0] = fi.y;
                 dot[t][1] = float(xint_digits(r1)) * fi.z; bsum[t][1] = fi.w;
             }
-#ifndef ZC_TIMING_NO_LITERAL
             if (__builtin_expect(literal_body, 0)) {
                 // pending (token, block) pairs of this lane in span j: bit 2t + h
                 uint32_t pending = 0;
@@ -489,7 +482,6 @@ __device__ __forceinline__ void xint_run_tile_tokens(const uint8_t* w_row, const
                     }
                 }
             }
-#endif
             const float scale = xint_bf16_of(sdw[j], half), bias = xint_bf16_of(bdw[j], half);
 #pragma unroll
             for (int t = 0; t < NTOK; ++t) {
@@ -529,8 +521,8 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
     const uint8_t* c = w_row + 16 * G;   // the lane's 16 bytes of each 64-byte span
     uint4 ring[R], sring, bring;
 #pragma unroll
-    for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, j * 4);
-    sring = ZC_TILE_LOAD(s_row, 0); bring = ZC_TILE_LOAD(b_row, 0);
+    for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, j * 4);
+    sring = ldg_u4(s_row, 0); bring = ldg_u4(b_row, 0);
     float acc[NTOK][4][2];
 #pragma unroll
     for (int t = 0; t < NTOK; ++t)
@@ -554,8 +546,8 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
         const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
         if (d0 + R < spans) {
 #pragma unroll
-            for (int j = 0; j < R; ++j) ring[j] = ZC_TILE_LOAD(c, (d0 + j + R) * 4);
-            sring = ZC_TILE_LOAD(s_row, (d0 + R) / 4); bring = ZC_TILE_LOAD(b_row, (d0 + R) / 4);
+            for (int j = 0; j < R; ++j) ring[j] = ldg_u4(c, (d0 + j + R) * 4);
+            sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4);
         }
         uint32_t unsafe[NTOK], any = 0;
 #pragma unroll
@@ -563,11 +555,7 @@ __device__ __forceinline__ void xint_run_tile_tokens_piped(const uint8_t* w_row,
             unsafe[t] = (reinterpret_cast<const uint32_t*>(img[t] + mask_at)[d0 / 4] >> (2 * G)) & 0x03030303u;
             any |= unsafe[t];
         }
-#ifdef ZC_TIMING_NO_LITERAL
-        const bool literal_body = false;
-#else
         const bool literal_body = __ballot(any != 0) != 0;
-#endif
         // operand buffers of two steps: A operands (digit planes of blocks 2G, 2G+1) and {2^e, sum} pairs of those blocks
         v4i a0[2][TG], a1[2][TG]; float4 fi[2][TG];
         auto load = [&](int buf, int step) {

@@ -12,7 +12,9 @@ Prints one JSON line.  `roofline.achieved` = algorithmic bytes of one launch (ro
 shared gate + distinct routed records + shared record + activations, summed over the 48
 layers) / average launch duration.  `cpu_baseline` = the CPU oracle (a restatement of the
 reference arithmetic; the reference has no CPU path of its own) on a bounded sample of the
-same workload, on this box's host cores.
+same workload, on this box's host cores.  `other_configs` holds, timed in the same run: the same stack with the
+guessing switched off, at decode batch 8 and 64, and the 2048-token prefill layer -- each with its time per step, tokens/s
+and its own fraction of the roofline that bounds it.
 """
 import argparse
 import json
@@ -85,7 +87,7 @@ def write_traffic_file(fetch_dir, write_dir):
 
 def one_launch_layer(ctx, name, tokens, reps, warmup=5, skew=("zipf", 1.1), speculate=True):
     """The same single-layer configuration through the persistent decode kernels as a stack of one layer: one launch per
-    step up to eight tokens, one launch per eight tokens above that; over 8 distinct inputs in rotation."""
+    step up to sixty-four tokens (pieces of sixty-four above that); over 8 distinct inputs in rotation."""
     import numpy as np
     import zerocool_amd as z
     from zerocool_amd import workload
@@ -150,7 +152,8 @@ def main():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--extra", action="store_true", help="also time decode batch 8 and the single-layer configurations")
+    ap.add_argument("--headline-only", action="store_true", help="skip the other_configs block (batch 1 without guessing, batch 8 and 64, the prefill layer)")
+    ap.add_argument("--extra", action="store_true", help="also time batch 32, milder router skews, the capped-HBM stack and the single-layer configurations")
     ap.add_argument("--workload", choices=("stack", "prefill"), default="stack",
                     help="stack: the 48-layer decode stack (the headline); prefill: one 2048-token batch through one layer of "
                          "hidden 2048 / 512 experts / top-10 / intermediate 512 on the bf16 matrix cores")
@@ -181,7 +184,7 @@ def main():
     L, T = args.layers, args.batch
     layers = [workload.LayerWeights(ctx, cfg, workload.BASE_SEED + 4 * 1000 + l, ("zipf", 1.1)) for l in range(L)]
     ctx.finish()
-    stack = ctx.stack_create(cfg, [l.layer for l in layers], max(T, 64 if args.extra else 8))
+    stack = ctx.stack_create(cfg, [l.layer for l in layers], max(T, 64))
 
     def run(stack, cfg, n_layers, tokens, steps, warmup, speculate=True, inputs=INPUTS, seed=workload.BASE_SEED + 4 * 7):
         """Times `steps` launches that cycle through `inputs` distinct token batches (a decode loop never sees the same
@@ -254,6 +257,28 @@ def main():
                      "kernel": "zc::decode_stack_kernel (one launch = one step)" if T == 1 else "zc::decode_multi_kernel (one launch = one step)",
                      "algorithmic_bytes_per_launch": int(nbytes), "launch_us": ms * 1e3},
     }
+
+    if not args.headline_only and (L, T) == (48, 1):
+        # The other configurations on the same clock, each with its own fraction of the roofline that bounds it: the same stack
+        # with the guessing switched off (every gate/up tile waits for the routing), at decode batch 8 and 64 (bytes = the
+        # DISTINCT records of a step), and BASELINE configs[2], the 2048-token prefill layer on the bf16 matrix cores.
+        quick = max(8, args.steps // 2)
+        def line(m, tokens, kernel):
+            return {"ms_per_step": m["ms"], "tokens_per_s": tokens / (m["ms"] * 1e-3), "GBps": m["bytes"] / (m["ms"] * 1e-3) / 1e9,
+                    "frac": m["bytes"] / (m["ms"] * 1e-3) / 8e12, "bound": "hbm", "distinct_experts_per_layer": m["unique"], "kernel": kernel}
+        also = {"stack_batch1_without_guessing": line(run(stack, cfg, L, 1, quick, 2, speculate=False), 1, "zc::decode_stack_kernel"),
+                "stack_batch8": line(run(stack, cfg, L, 8, quick, 2), 8, "zc::decode_multi_kernel"),
+                "stack_batch64": line(run(stack, cfg, L, 64, max(4, quick // 4), 1, inputs=2), 64, "zc::decode_wide_kernel")}
+        ctx.stack_set_speculation(stack, True)
+        pf = single_layer(ctx, "S", 2048, True, 20, 3, skew=None)
+        s_cfg = workload.config("S")
+        weight_bytes = s_cfg.experts * ctx.record_bytes(s_cfg) + ctx.record_bytes(s_cfg, shared=True) + 2 * s_cfg.hidden * s_cfg.experts
+        also["prefill_layer_2048_tokens"] = {
+            "ms_per_step": pf["us_per_layer"] * 1e-3, "tokens_per_s": pf["tokens_per_s"], "TFLOPs": pf["TFLOPs"], "bound": "mfma",
+            "frac": pf["TFLOPs"] / 2500.0, "frac_of_hbm_floor": weight_bytes / 8e12 / (pf["us_per_layer"] * 1e-6),
+            "workload": "BASELINE configs[2]: hidden 2048, 512 experts, top-10, intermediate 512, affine Q4, no router skew",
+            "kernel": "zc::prefill_gemm_kernel and the layer's other kernels (whole-layer rate)"}
+        result["other_configs"] = also
 
     if not args.no_cpu:
         import oracle

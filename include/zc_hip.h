@@ -214,9 +214,11 @@ typedef struct {       /* optional device buffers, any may be NULL */
     int32_t* ids;      /* [n_layers][tokens][topk] */
     float* weights;    /* [n_layers][tokens][topk] */
     float* outputs;    /* [n_layers][tokens][hidden] layer outputs before the glue */
-    uint64_t* clocks;  /* [n_layers * 15][workgroups] timestamps (100 MHz) that every workgroup of the
-                          persistent kernel takes at its phase boundaries, 15 per layer (tuning aid;
-                          persistent path only; workgroups = compute units of the device) */
+    uint64_t* clocks;  /* [n_layers * 24][workgroups] timestamps (100 MHz) of the persistent kernels, 24 slots
+                          per layer: the one-token kernel fills 0..14 from every workgroup's first thread at its
+                          phase boundaries and 15..21 from the first lane of its fifth wave inside the gate/up
+                          and down phases; the kernels for more tokens write their own, smaller number of stamps per
+                          layer back to back (tuning aid; persistent path only; workgroups = compute units) */
 } zc_stack_trace;
 zc_status zc_hip_stack_create(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
                               uint32_t n_layers, uint32_t max_tokens, zc_hip_stack** out);

@@ -52,10 +52,11 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
     const uint16_t* xh_all = reinterpret_cast<const uint16_t*>(lds + lp.xh);
     const XintLayout LH{H}, LI{I};
     Barrier bar{p.sync, p.epoch, p.spin_limit, p.status, p.epoch};
-    uint32_t stamp = 0;
-    // stamps of every workgroup: clocks[(stamp index) * workgroups + workgroup]
-    auto clock = [&]() { if (p.clocks && tid == 0) p.clocks[uint64_t(stamp) * nwg + wg] = wall_clock64(); ++stamp; };
-    auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };   // after the slowest wave of the workgroup
+    constexpr uint32_t kStamps = kDecodeStamps;   // slots per layer; this kernel fills 0..14, from the first thread of the workgroup
+    // stamps of every workgroup: clocks[(layer * kStamps + stamp index) * workgroups + workgroup]
+    uint32_t stamp_layer = 0;
+    auto clock = [&](uint32_t i) { if (p.clocks && tid == 0) p.clocks[uint64_t(stamp_layer * kStamps + i) * nwg + wg] = wall_clock64(); };
+    auto clock_all = [&](uint32_t i) { if (p.clocks) __syncthreads(); clock(i); };   // after the slowest wave of the workgroup
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
     if (tid == 0) { misc[10] = 0; misc[11] = 0; misc[12] = 0; misc[13] = 0; misc[14] = 0; }   // the router chain's hand-off word, the ids-ready word, the staging waves' image-ready words: no tag is 0
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             lane = tid & 63u; wave = uint32_t(uniform(int32_t(tid >> 6))); col = lane & 15u; G = lane >> 4;
         };
         refresh();
-        clock();
+        stamp_layer = layer; clock(0);
         // One token: the 16-bit tag of everything layer l exchanges, never 0 (the buffers start as zeros) and different
         // from the tags of the layers (and launches) just before it
         auto tag_of = [&](uint32_t l) { return (p.tag_base + l) % 65535u + 1u; };
@@ -284,7 +285,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             __syncthreads();
             xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
         }
-        clock();
+        clock(1);
         {
             // One token: the shared gate/up tiles run in phase G beside the routed ones, on waves that have no routed tile;
             // this phase then only has the router.
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             }
         }
         if (apart) {
-            clock();
+            clock(2);
             if (wave >= router_segments) {   // the tile waves: until every staging wave has said that its blocks are built
                 const uint32_t staging = (H / 16 + 63) / 64;
                 for (uint32_t i = 0; i < (1u << 22); ++i) {
@@ -468,15 +469,15 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
             }
         } else {
-            clock_all();
+            clock_all(2);
             if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the routing below polls the logits themselves
         }
         refresh();
-        clock();
+        clock(3);
         // ---------------- phase G: route, group slots by expert, routed gate/up ----------------
         for (uint32_t t = wave; t < T; t += kDecodeWaves)
         {
-            auto stamp = [&]() { if (t == 0) clock(); };
+            uint32_t route_stamp = 4; auto stamp = [&]() { if (t == 0) clock(route_stamp++); };
             // the previous step's ids of this layer, one per lane: requested now, compared when this step's ids are final
             const int32_t guess = (NT == 1 && pred && lane < k) ? pred[lane] : -1;
             uint32_t* scratch = reinterpret_cast<uint32_t*>(experts) + 128 * wave;   // the expert list is built later; 128 words per wave fit it for 512 experts
@@ -560,7 +561,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
             __syncthreads();
         }
-        clock();
+        clock(6);
         if (tid < n) {
             const int32_t e = ids[tid];
             if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); if constexpr (NT != 1) next[tid] = -1; }
@@ -591,7 +592,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         __syncthreads();
         U = uint32_t(uniform(misc[0]));
         }
-        clock();
+        clock(7);
         if constexpr (NT == 1) {
             // Two passes over gate/up tiles.  Pass 0 runs BEFORE the ids are known, on the seven waves that do not route: the
             // tiles of the experts this layer picked at the previous step (the reference predicts a layer's experts for its
@@ -700,14 +701,14 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
         }
-        clock_all();
+        clock_all(8);
         if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the staging below polls the activations themselves
         refresh();
-        clock();
+        clock(9);
         // ---------------- phase D: down tiles per 16 output rows, combine ----------------
         float* otile = reinterpret_cast<float*>(lds + lp.otile);
         const uint32_t slots_total = n + T, SB = lp.slots_per_batch;
-        if (wg >= H / 16) { clock(); clock(); clock(); }   // workgroups without a row tile keep the stamp count
+        if (wg >= H / 16) { clock(10); clock(11); clock(12); }   // workgroups without a row tile keep the stamp count
         if constexpr (NT == 1) { if (wg >= H / 16) bar.arrive(); }
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
             const uint32_t row = rt * 16 + col;
@@ -717,7 +718,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 // BF16 copy under the latency of those loads, and runs the tile; no workgroup barrier until the combine, and
                 // a wave starts as soon as its own slot is complete.
                 __syncthreads();
-                clock(); clock();
+                clock(10); clock(11);
                 uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
                 for (uint32_t slot = wave; slot <= k; slot += kDecodeWaves) {   // slot k is the shared expert's
                     const uint8_t* rec = L.shared_record; const uint64_t* off = p.so;
@@ -846,7 +847,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                             }
                         }
                     }
-                    if (s0 == 0) { clock(); clock(); }
+                    if (s0 == 0) { clock(10); clock(11); }
                     __syncthreads();
                     if (rt + nwg >= H / 16 && s0 + SB >= slots_total) bar.arrive();   // nothing more to read from other workgroups in this layer
                 } else {
@@ -857,9 +858,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                                                        reinterpret_cast<uint64_t*>(ah + routed * I));
                     }
                     __syncthreads();
-                    if (s0 == 0) clock();
+                    if (s0 == 0) clock(10);
                     xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
-                    if (s0 == 0) clock();
+                    if (s0 == 0) clock(11);
                 }
                 if constexpr (NT == 1) {
                     for (uint32_t slot = wave; slot <= k; slot += kDecodeWaves) {   // slot k is the shared expert's
@@ -915,7 +916,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             }
             __syncthreads();
             if (!MIXED && NT == 1 && SB >= slots_total && I == 1024 && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
-            clock();
+            clock(12);
             // weighted combine of the tile (reference: qwen.metal:804-816)
             if (tid < T * 16) {
                 const uint32_t t = tid / 16, c = tid % 16;
@@ -961,9 +962,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 }
             }
         }
-        clock_all();
+        clock_all(13);
         if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the next layer polls the output words themselves
-        clock();
+        clock(14);
     }
 }
 

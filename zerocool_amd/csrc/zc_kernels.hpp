@@ -84,7 +84,7 @@ struct DecodeParams {
     uint32_t tag_base;               // one token: layer l exchanges under tag (tag_base + l) % 65535 + 1; advances only with one-token launches
     unsigned long long* clocks;      // optional [L * kDecodeStamps][workgroups] 100 MHz timestamps, one per workgroup
 };
-constexpr uint32_t kDecodeStamps = 15;
+constexpr uint32_t kDecodeStamps = 24;
 struct DecodeLdsPlan {
     uint32_t ids, weights, gatev, head, next, experts, misc, region, total;
     uint32_t img_rg, xh, gprod, img_d, ah, otile, slots_per_batch, gatew, spec;

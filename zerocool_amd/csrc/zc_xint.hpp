@@ -28,11 +28,11 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 // 16 bytes in MFMA byte order, a {2^e, bias-sum} pair, and an unsafe bit.
 struct XintLayout {
     uint32_t K;
-    __host__ __device__ uint32_t blocks() const { return K / 16; }
-    __host__ __device__ uint32_t planes_bytes() const { return blocks() * 48 + 16; }   // + one zero slot
-    __host__ __device__ uint32_t info_bytes() const { return blocks() * 8; }
-    __host__ __device__ uint32_t mask_bytes() const { return (blocks() + 31) / 32 * 4; }
-    __host__ __device__ uint32_t bytes() const { return (planes_bytes() + info_bytes() + mask_bytes() + 15) / 16 * 16; }
+    __host__ __device__ constexpr uint32_t blocks() const { return K / 16; }
+    __host__ __device__ constexpr uint32_t planes_bytes() const { return blocks() * 48 + 16; }   // + one zero slot
+    __host__ __device__ constexpr uint32_t info_bytes() const { return blocks() * 8; }
+    __host__ __device__ constexpr uint32_t mask_bytes() const { return (blocks() + 31) / 32 * 4; }
+    __host__ __device__ constexpr uint32_t bytes() const { return (planes_bytes() + info_bytes() + mask_bytes() + 15) / 16 * 16; }
 };
 
 // The three digit sums of a block recombined, d0 + 2^7 d1 + 2^14 d2, by Horner's rule in two shift-and-add instructions.
@@ -66,7 +66,9 @@ struct LdsBf16 {     // BF16 copy of a BF16-valued row
     static constexpr bool kExactProducts = true, kRowInLds = true;
     const uint16_t* x;
     __device__ __forceinline__ void block(uint32_t b, uint32_t* out) const {
-        const uint4 lo = *reinterpret_cast<const uint4*>(x + b * 16), hi = *reinterpret_cast<const uint4*>(x + b * 16 + 8);
+        // (native vector types: the compiler then keeps track of where the read comes from, and does not make it wait for
+        // loads whose target is another part of LDS)
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(x + b * 16), hi = *reinterpret_cast<const u32x4*>(x + b * 16 + 8);
         const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
         for (int i = 0; i < 8; ++i) { out[2 * i] = w[i] << 16; out[2 * i + 1] = w[i] & 0xffff0000u; }
@@ -376,7 +378,7 @@ __device__ __forceinline__ void xint_run_tile_after(const uint8_t* w_row, const 
 // all sixteen inputs are read at once and the four chains run side by side, then the quad sums are added in order -- one
 // LDS latency and a chain of eight dependent operations instead of four latencies and twenty.
 __device__ __forceinline__ float xint_literal_block(const uint16_t* x_block, uint32_t w_lo, uint32_t w_hi) {
-    const uint4 xa = *reinterpret_cast<const uint4*>(x_block), xb = *reinterpret_cast<const uint4*>(x_block + 8);
+    const u32x4 xa = *reinterpret_cast<const u32x4*>(x_block), xb = *reinterpret_cast<const u32x4*>(x_block + 8);
     const uint32_t xw[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
     float quad[4];
 #pragma unroll

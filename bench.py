@@ -398,6 +398,7 @@ def main():
         extra["single_layer_mixed_one_launch"] = [one_launch_layer(ctx, "S-mixed", t, 100) for t in (1, 8, 16)]
         extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8, 16)]
         extra["prefill_q4"] = [single_layer(ctx, "S", t, True, 20) for t in (32, 64, 256, 2048)]
+        extra["prefill_mixed"] = [single_layer(ctx, "S-mixed", t, True, 20, skew=None) for t in (256, 2048)]
         result["extra"] = extra
 
     print(json.dumps(result))

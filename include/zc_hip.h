@@ -181,10 +181,11 @@ zc_status zc_hip_moe_forward_static(zc_hip_ctx* ctx, const zc_moe_config* cfg, c
                                     const float* x, uint32_t tokens, float* out, const zc_moe_trace* trace);
 /* Prefill (many tokens): the same layer with the expert products as a sorted-token grouped GEMM on the bf16 matrix
  * cores with fp32 accumulation -- what encode_expert_rows batches per expert in the reference (pipeline.cpp:7-31 over
- * q4_mm / q4_gate_up, qwen.metal:289-376).  Router ids, softmax weights and the dispatch are the exact kernels (bit-equal
+ * q4_mm / q4_gate_up, qwen.metal:289-376; affine Q8 projections the same way over q8_mm / q8_gate_up, qwen.metal:126-144,
+ * 192-196, so the mixed 4/8-bit artifact has a prefill path too).  Router ids, softmax weights and the dispatch are the exact kernels (bit-equal
  * to zc_hip_moe_forward); expert outputs agree with zc_hip_moe_forward to a few fp32 ulps before their BF16 rounding, so
- * the layer output is checked against a tolerance (max relative error 2e-3), not bit for bit.  Affine Q4 group 64 only,
- * hidden and intermediate sizes multiples of 128 up to 4096; x must be BF16-valued (else status bit 4 at zc_hip_moe_check).
+ * the layer output is checked against a tolerance (max relative error 2e-3), not bit for bit.  Every projection affine
+ * Q4 or affine Q8, group 64; hidden and intermediate sizes multiples of 128 up to 4096; x must be BF16-valued (else status bit 4 at zc_hip_moe_check).
  * From 128 tokens on the router logits are formed exactly only for the experts that can reach the top k (a matrix-core
  * product with a rigorous bound decides which; ids and weights are unchanged); a trace that asks for the logits gets
  * all of them from the exact kernel.

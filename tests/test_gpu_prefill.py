@@ -71,6 +71,40 @@ def test_prefill_matches_the_exact_path(ctx, shape, tokens):
         ctx.free(b)
 
 
+@pytest.mark.parametrize("shape,bits,tokens", [((512, 32, 4, 128), (4, 8, 8, 8), 37),      # the mixed artifact: Q4 gate/up, Q8 down and shared expert
+                                               ((512, 32, 4, 128), (8, 8, 8, 8), 150),     # every projection Q8, narrow lanes (K not a multiple of 512 for the down rows)
+                                               ((1024, 64, 10, 512), (4, 8, 8, 8), 129),   # wide lanes on both sides
+                                               ((1024, 64, 10, 512), (8, 4, 4, 8), 70),
+                                               ((2048, 512, 10, 512), (4, 8, 8, 8), 96)])  # BASELINE config 4's shape
+def test_prefill_with_affine_q8_projections(ctx, shape, bits, tokens):
+    # Affine Q8 records through the same grouped product: byte codes are exact in bf16, the fold uses the Q8 lanes' plain
+    # input sums (qwen.metal:112-125), and the sums near a BF16 rounding boundary are recomputed on the Q8 lanes themselves.
+    cfg = workload.tiny_config(*shape, bits=bits)
+    weights = workload.LayerWeights(ctx, cfg, 161 + tokens, ("normal", 0.5))
+    x = workload.hidden_rows(ctx, tokens, cfg.hidden, 800 + tokens)
+    exact, fast = run_both(ctx, cfg, weights, x, tokens)
+    assert fast["ids"].tobytes() == exact["ids"].tobytes()
+    assert fast["weights"].tobytes() == exact["weights"].tobytes()
+    assert rel(fast["shared"], exact["shared"]) <= ONE_BF16_STEP
+    assert rel(fast["expert_out"], exact["expert_out"]) <= ONE_BF16_STEP
+    same = np.mean(fast["out"].view(np.uint32) == exact["out"].view(np.uint32))
+    print(f"T={tokens} {shape} bits {bits}: layer output max rel err {rel(fast['out'], exact['out']):.3g}, identical {same:.5f}, "
+          f"expert outputs identical {np.mean(fast['expert_out'].view(np.uint32) == exact['expert_out'].view(np.uint32)):.5f}")
+    assert rel(fast["out"], exact["out"]) <= TOLERANCE
+    assert same > 0.9999, same
+    # and against the CPU oracle directly on a few token rows
+    sample = np.arange(0, tokens, max(1, tokens // 8))[:8]
+    h = weights.host()
+    ocfg = oracle.Config(*[getattr(cfg, n) for n, _ in z.Config._fields_])
+    xs = x.numpy(f32).reshape(tokens, cfg.hidden)[sample]
+    want, tr = oracle.moe_layer(ocfg, h["router"], h["shared_gate"], h["shared_record"], h["records"], h["stride"],
+                                xs, len(sample), router_offsets=h["offsets"], threads=8, trace=True)
+    assert fast["ids"].reshape(tokens, cfg.topk)[sample].tobytes() == tr["ids"].tobytes()
+    assert rel(fast["out"].reshape(tokens, cfg.hidden)[sample], want) <= TOLERANCE
+    for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, x):
+        ctx.free(b)
+
+
 def test_prefill_against_the_cpu_oracle(ctx):
     cfg = workload.tiny_config(512, 32, 4, 128)
     T = 70
@@ -146,8 +180,9 @@ def test_prefill_reports_unroutable_rows(ctx):
 
 
 def test_prefill_rejects_what_it_cannot_run(ctx):
-    mixed = workload.tiny_config(512, 32, 4, 128, bits=(4, 8, 8, 8))
-    assert ctx.moe_prefill_workspace_bytes(mixed, 64) == 0
+    odd = workload.tiny_config(512, 32, 4, 128, group=32)     # only group 64
+    assert ctx.moe_prefill_workspace_bytes(odd, 64) == 0
+    assert ctx.moe_prefill_workspace_bytes(workload.tiny_config(512, 32, 4, 128, bits=(4, 8, 8, 8)), 64) > 0   # the mixed artifact is taken
     assert ctx.moe_prefill_workspace_bytes(workload.tiny_config(4224, 32, 4, 128), 64) == 0   # K beyond what the product kernel keeps in LDS
     assert ctx.moe_prefill_workspace_bytes(workload.tiny_config(4096, 32, 4, 4096), 64) > 0
     cfg = workload.tiny_config(512, 32, 4, 128)
@@ -160,7 +195,7 @@ def test_prefill_rejects_what_it_cannot_run(ctx):
         ctx.moe_check()
     assert "BF16" in str(err.value)
     with pytest.raises(z.ZcError):
-        ctx.moe_prefill(mixed, weights.layer, x, T, out, ws)
+        ctx.moe_prefill(odd, weights.layer, x, T, out, ws)
 
 
 @pytest.mark.parametrize("skew", [None, ("zipf", 1.1)])

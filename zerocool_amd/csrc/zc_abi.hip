@@ -652,7 +652,7 @@ zc_status zc_hip_moe_forward(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
 namespace {
 struct PrefillSpace {
     Workspace base;
-    uint16_t *xb, *actb, *sactb; float *xsum, *asum, *ssum, *xsum16, *asum16, *ssum16;
+    uint16_t *xb, *actb, *sactb; float *xsum, *xplain, *asum, *ssum, *xsum16, *asum16, *ssum16;   // xplain: the inputs' sums for affine Q8 gate/up rows
     int32_t *tile_expert, *tile_first, *tile_rows, *tile_count, *stile_expert, *stile_first, *stile_rows, *stile_count;
     uint32_t max_tiles, max_shared_tiles;
     uint32_t* near_bits;      // one bit per product element: recompute exactly
@@ -677,11 +677,14 @@ PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
     w.xsum16 = (float*)take(uint64_t(T) * (c->hidden / 16) * 4); w.asum16 = (float*)take(n * (c->inter / 16) * 4);
     w.ssum16 = (float*)take(uint64_t(T) * (c->inter / 16) * 4);
     w.norms = (float*)take((uint64_t(T) + c->experts) * 4);
+    w.xplain = (float*)take(uint64_t(T) * (c->hidden / 64) * 4);
     w.bytes = at;
     return w;
 }
 bool prefill_config(const zc_moe_config* c) {
-    return c->bits_gate_up == 4 && c->bits_down == 4 && c->shared_bits_gate_up == 4 && c->shared_bits_down == 4 && c->group == 64 &&
+    // every projection affine Q4 or affine Q8 (the mixed 4/8-bit artifact: Q4 routed gate/up, Q8 down and shared expert)
+    auto q = [](uint32_t bits) { return bits == 4 || bits == 8; };
+    return q(c->bits_gate_up) && q(c->bits_down) && q(c->shared_bits_gate_up) && q(c->shared_bits_down) && c->group == 64 &&
            zc::prefill_shape(c->hidden, c->inter, c->experts);
 }
 }  // namespace
@@ -693,7 +696,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
                              float* out, void* workspace, const zc_moe_trace* trace) {
     Timed timed(ctx, "moe_prefill");
     if (const zc_status s = validate_config(c)) return s;
-    ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 group 64 with hidden and intermediate sizes that are multiples of 128 up to 4096");
+    ZC_REQUIRE(prefill_config(c), "the matrix-core prefill path takes affine Q4 and Q8 group 64 with hidden and intermediate sizes that are multiples of 128 up to 4096");
     ZC_REQUIRE(ctx && l && x && out && workspace && T && T <= 8192, "invalid MoE layer buffers");
     ZC_REQUIRE(uint64_t(T) * c->topk * std::max(c->hidden, c->inter) < (1ull << 32), "too many product elements for one prefill call");
     ZC_REQUIRE(l->router && l->shared_gate && l->shared_record && l->expert_records, "missing MoE layer weights");
@@ -708,7 +711,8 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     const uint64_t n = uint64_t(T) * k;
     // router logits, top-k + softmax, dispatch (model.cpp:434-479), shared gate: the exact kernels, except that a long batch
     // whose logits nobody asks for gets exact logits only where the selection can see the difference (launch_prefill_router)
-    zc::launch_prefill_rows(s, x, T, H, w.xb, w.xsum, w.xsum16, ctx->moe_status);
+    const bool x_q4 = c->bits_gate_up == 4 || c->shared_bits_gate_up == 4, x_q8 = c->bits_gate_up == 8 || c->shared_bits_gate_up == 8;
+    zc::launch_prefill_rows(s, x, T, H, w.xb, x_q4 ? w.xsum : nullptr, x_q4 ? w.xsum16 : nullptr, x_q8 ? w.xplain : nullptr, ctx->moe_status);
     if (T >= 128 && !(trace && trace->logits)) zc::launch_prefill_router(s, x, w.xb, l->router, l->router_offsets, T, H, E, k, w.norms, w.base.logits);
     else zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
     zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
@@ -730,7 +734,8 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     };
     {   // routed gate/up + SwiGLU on gathered rows (pipeline.cpp:18-24), then down scattered to the slots (pipeline.cpp:25-29)
         zc::PrefillGemm g{};
-        g.a = w.xb; g.asum = w.xsum; g.asum16 = w.xsum16; g.a_rows = w.base.slots; g.a_div = k; g.out_rows = nullptr;
+        g.bits = c->bits_gate_up;
+        g.a = w.xb; g.asum = g.bits == 4 ? w.xsum : w.xplain; g.asum16 = g.bits == 4 ? w.xsum16 : nullptr; g.a_rows = w.base.slots; g.a_div = k; g.out_rows = nullptr;
         g.records = static_cast<const uint8_t*>(l->expert_records); g.stride = l->record_stride; offsets_of(l->expert_records, 0, g.off, 0, 2);
         g.tile_expert = w.tile_expert; g.tile_first = w.tile_first; g.tile_rows = w.tile_rows; g.tile_count = w.tile_count;
         g.K = H; g.N = I; g.out_b = w.actb;
@@ -738,9 +743,10 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.covered = w.base.offsets + E; g.experts = E;
         zc::launch_prefill_gemm(s, g, true, w.max_tiles);
         zc::launch_prefill_patch(s, g, true);
-        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum, table_inter ? w.asum16 : nullptr);
         zc::PrefillGemm d{};
-        d.a = w.actb; d.asum = w.asum; d.asum16 = table_inter ? w.asum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
+        d.bits = c->bits_down;
+        zc::launch_prefill_sums(s, w.actb, nullptr, uint32_t(n), I, w.asum, table_inter && d.bits == 4 ? w.asum16 : nullptr, d.bits == 8);
+        d.a = w.actb; d.asum = w.asum; d.asum16 = table_inter && d.bits == 4 ? w.asum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
         d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
         d.K = I; d.N = H; d.out_f = w.base.expert_out;
@@ -751,16 +757,18 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     }
     {   // shared expert (model.cpp:482-485): one group of all the tokens
         zc::PrefillGemm g{};
-        g.a = w.xb; g.asum = w.xsum; g.asum16 = w.xsum16; g.a_rows = nullptr; g.a_div = 1;
+        g.bits = c->shared_bits_gate_up;
+        g.a = w.xb; g.asum = g.bits == 4 ? w.xsum : w.xplain; g.asum16 = g.bits == 4 ? w.xsum16 : nullptr; g.a_rows = nullptr; g.a_div = 1;
         g.records = static_cast<const uint8_t*>(l->shared_record); g.stride = 0; offsets_of(l->shared_record, 1, g.off, 0, 2);
         g.tile_expert = w.stile_expert; g.tile_first = w.stile_first; g.tile_rows = w.stile_rows; g.tile_count = w.stile_count;
         g.K = H; g.N = I; g.out_b = w.sactb;
         g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(T) * I / 32); g.near_margin = margin; g.ids = nullptr; g.slots = nullptr;
         zc::launch_prefill_gemm(s, g, true, w.max_shared_tiles);
         zc::launch_prefill_patch(s, g, true);
-        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum, table_inter ? w.ssum16 : nullptr);
         zc::PrefillGemm d{};
-        d.a = w.sactb; d.asum = w.ssum; d.asum16 = table_inter ? w.ssum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
+        d.bits = c->shared_bits_down;
+        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum, table_inter && d.bits == 4 ? w.ssum16 : nullptr, d.bits == 8);
+        d.a = w.sactb; d.asum = w.ssum; d.asum16 = table_inter && d.bits == 4 ? w.ssum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
         d.records = g.records; d.stride = 0; offsets_of(l->shared_record, 1, d.off, 2, 1);
         d.tile_expert = w.stile_expert; d.tile_first = w.stile_first; d.tile_rows = w.stile_rows; d.tile_count = w.stile_count;
         d.K = I; d.N = H; d.out_f = w.base.shared;

@@ -123,6 +123,7 @@ struct PrefillGemm {
     uint64_t off[6];          // byte offsets in a record: codes, scales, biases of the (gate | down) projection, then of up
     const int32_t *tile_expert, *tile_first, *tile_rows, *tile_count;
     uint32_t K, N;            // reduction length, rows of ONE projection
+    uint32_t bits;            // 4: nibble codes, asum = the Q4 lanes' BF16-rounded sum-of-four chains; 8: byte codes, asum = the Q8 lanes' plain sums
     uint16_t* out_b;          // gate/up: SwiGLU activations as bf16 [sorted position][N]
     float* out_f;             // down: BF16-rounded fp32 [output row][N]
     // Sums that land within near_margin * (sum of term magnitudes) of a BF16 rounding boundary are marked in a bit map
@@ -136,10 +137,10 @@ struct PrefillGemm {
     const int32_t* covered; uint32_t experts;
 };
 constexpr float kPrefillMargin = 0x1p-22f;  // of the summed term magnitudes: four fp32 steps at that scale
-void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status);
+void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, float* plain, int32_t* status);
 void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, const void* w, const float* offsets, uint32_t T, uint32_t K,
                            uint32_t E, uint32_t topk, float* norms, float* logits);
-void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16);
+void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16, bool plain);
 void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
                           int32_t* tile_rows, int32_t* tile_count);
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles);

@@ -36,36 +36,44 @@ constexpr uint32_t kTileRows = 32, kTileRowsMax = 48, kTileCols = 128, kPitch = 
 
 // fp32 rows holding BF16 values -> bf16 rows, plus per (row, group of 64) the sum of the four blocks' BF16-rounded
 // sum-of-four chains.  One thread per (row, group).  status bit 4: a value was not BF16-valued.
-__global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status) {
+// plain (optional): per (row, group) the sum of the plain fp32 sums of the group's eight 8-element blocks, the affine Q8
+// lanes' input sum (qwen.metal:112-125: sum += v, element by element).
+__global__ __launch_bounds__(256) void prefill_rows_kernel(const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, float* plain,
+                                                           int32_t* status) {
     const uint32_t groups = K / 64, i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= rows * groups) return;
     const uint32_t r = i / groups, g = i % groups;
     const float4* src = reinterpret_cast<const float4*>(x + uint64_t(r) * K + g * 64);
     uint32_t low = 0;
-    float total = 0;
+    float total = 0, total_plain = 0;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-        float sum = 0;
+        float sum = 0, eight[2] = {0, 0};
         uint32_t packed[8];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 v = src[b * 4 + q];
             sum += bf(bf(bf(v.x + v.y) + v.z) + v.w);
+            eight[q / 2] = (((eight[q / 2] + v.x) + v.y) + v.z) + v.w;
             const uint32_t u0 = __float_as_uint(v.x), u1 = __float_as_uint(v.y), u2 = __float_as_uint(v.z), u3 = __float_as_uint(v.w);
             low |= (u0 | u1 | u2 | u3) & 0xffffu;
             packed[2 * q] = (u0 >> 16) | (u1 & 0xffff0000u); packed[2 * q + 1] = (u2 >> 16) | (u3 & 0xffff0000u);
         }
         total += sum;
+        total_plain = (total_plain + eight[0]) + eight[1];
         if (sums16) sums16[uint64_t(i) * 4 + b] = sum;
         uint4* dst = reinterpret_cast<uint4*>(xb + uint64_t(r) * K + g * 64 + b * 16);
         dst[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
         dst[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
     }
-    sums[i] = total;
+    if (sums) sums[i] = total;
+    if (plain) plain[i] = total_plain;
     if (low) atomicOr(status, 4);
 }
 // The same sums for rows that are already bf16 (the SwiGLU activations).
-__global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16) {
+// plain: the affine Q8 lanes' sums instead (see prefill_rows_kernel); no per-block table then.
+__global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16,
+                                                           bool plain) {
     const uint32_t groups = K / 64, i = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t rows = rows_ptr ? min(uint32_t(*rows_ptr), rows_max) : rows_max;
     if (i >= rows * groups) return;
@@ -76,15 +84,16 @@ __global__ __launch_bounds__(256) void prefill_sums_kernel(const uint16_t* xb, c
     for (int b = 0; b < 4; ++b) {
         const uint4 lo = src[2 * b], hi = src[2 * b + 1];
         const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        float sum = 0;
+        float sum = 0, eight[2] = {0, 0};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float a = __uint_as_float(w[2 * q] << 16), c = __uint_as_float(w[2 * q] & 0xffff0000u);
             const float d = __uint_as_float(w[2 * q + 1] << 16), e = __uint_as_float(w[2 * q + 1] & 0xffff0000u);
             sum += bf(bf(bf(a + c) + d) + e);
+            eight[q / 2] = (((eight[q / 2] + a) + c) + d) + e;
         }
-        total += sum;
-        if (sums16) sums16[uint64_t(i) * 4 + b] = sum;
+        total = plain ? (total + eight[0]) + eight[1] : total + sum;
+        if (sums16 && !plain) sums16[uint64_t(i) * 4 + b] = sum;
     }
     sums[i] = total;
 }
@@ -115,7 +124,10 @@ __global__ __launch_bounds__(1024) void prefill_tiles_kernel(const int32_t* offs
     if (e == 1023) *tile_count = scan[1023];
 }
 
-template <bool GATED>
+// BITS: 4 (nibble codes, eight bytes of a row per lane and step) or 8 (byte codes, sixteen bytes; the chain sums are then
+// the plain ones of the Q8 lanes).  A byte code is exact in bf16 like a nibble code, and its product with a BF16 value is
+// exact in fp32.
+template <bool GATED, int BITS>
 __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     __shared__ __align__(16) uint16_t a_s[2][kTileRowsMax * kPitch];
     // The scales and biases of the workgroup's 128 weight rows and the chain sums of its token rows, for every step, are
@@ -151,7 +163,7 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
     for (int q = 0; q < 2; ++q) {
         col_row[q] = (GATED ? (uint32_t(q) * 64u + wave * 16u) : (2 * wave + uint32_t(q)) * 16u) + j;
         const uint32_t b_proj = GATED ? col_row[q] >> 6 : 0u, b_n = n0 + (GATED ? (col_row[q] & 63u) : col_row[q]);
-        b_src[q] = record + p.off[b_proj * 3] + uint64_t(b_n) * (K / 2) + g4 * 8;
+        b_src[q] = record + p.off[b_proj * 3] + uint64_t(b_n) * (K * BITS / 8) + g4 * (2 * BITS);
     }
     // scales then biases as bf16 [128][groups + 2] (the pad keeps sixteen rows on different banks), then the chain sums
     // [groups][48]
@@ -181,13 +193,16 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 
     // What a step needs is requested two steps ahead and waits in registers (two sets, taken in turn): with one step of
     // lead the loads' latency, several times a step's arithmetic, was paid at every step.
-    struct Fetched { uint4 a, a2; uint2 b[2]; };
+    struct Fetched { uint4 a, a2; uint32_t b[2][BITS / 2]; };   // the lane's sixteen codes of a step: two dwords (Q4) or four (Q8)
     Fetched ahead[2];
-    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), {make_uint2(0, 0), make_uint2(0, 0)}};
+    ahead[0] = ahead[1] = Fetched{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), {}};
     auto fetch = [&](uint32_t g, Fetched& f) {
         f.a = *reinterpret_cast<const uint4*>(a_src + g * 64);
 #pragma unroll
-        for (int q = 0; q < 2; ++q) f.b[q] = ldg_u2(b_src[q] + g * 32);
+        for (int q = 0; q < 2; ++q) {
+            if constexpr (BITS == 4) { const uint2 v = ldg_u2(b_src[q] + g * 32); f.b[q][0] = v.x; f.b[q][1] = v.y; }
+            else { const uint4 v = ldg_u4(b_src[q] + g * 64); f.b[q][0] = v.x; f.b[q][1] = v.y; f.b[q][2] = v.z; f.b[q][3] = v.w; }
+        }
         if (tall && tid < 128) f.a2 = *reinterpret_cast<const uint4*>(a_src2 + g * 64);
     };
     auto stash = [&](uint32_t buf, const Fetched& f) {   // the token rows
@@ -204,6 +219,17 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const f32x2 pair = {float((even >> (8 * q)) & 0xffu), float((odd >> (8 * q)) & 0xffu)};
+            out[q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+        }
+        return __builtin_bit_cast(bf16x8, make_uint4(out[0], out[1], out[2], out[3]));
+    };
+    // eight byte codes (two words, byte i of the pair is element i) -> eight bf16
+    auto expand_bytes = [](uint32_t lo, uint32_t hi) {
+        uint32_t out[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t word = q < 2 ? lo : hi;
+            const f32x2 pair = {float((word >> (16 * (q & 1))) & 0xffu), float((word >> (16 * (q & 1) + 8)) & 0xffu)};
             out[q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
         }
         return __builtin_bit_cast(bf16x8, make_uint4(out[0], out[1], out[2], out[3]));
@@ -263,7 +289,10 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
         const uint32_t buf = g & 1u;
         bf16x8 b[2][2];   // [tile][half of the lane's sixteen codes]
 #pragma unroll
-        for (int q = 0; q < 2; ++q) { b[q][0] = expand(mine.b[q].x); b[q][1] = expand(mine.b[q].y); }
+        for (int q = 0; q < 2; ++q) {
+            if constexpr (BITS == 4) { b[q][0] = expand(mine.b[q][0]); b[q][1] = expand(mine.b[q][1]); }
+            else { b[q][0] = expand_bytes(mine.b[q][0], mine.b[q][1]); b[q][1] = expand_bytes(mine.b[q][2], mine.b[q][3]); }
+        }
         if (g + 2 < groups) fetch(g + 2, mine);
         f32x4 dot[kBlocks][2];
 #pragma unroll
@@ -339,8 +368,10 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 
 // Exact recomputation of the listed elements: one group of 32 lanes plays the reference's 32 lanes for one row
 // (qwen.metal:46-62: lane width 16 when K % 512 == 0 and N % 8 == 0, else 8; xor-butterfly lane sum).
+// BITS 8: the affine Q8 lanes (qwen.metal:112-125: lane width 8 when K % 512 == 0 and N % 8 == 0, else 4; the input sum is the
+// plain fp32 sum, the dot a multiply-add chain element by element).
 constexpr uint32_t kPatchWordsMax = 256;
-template <int WIDTH, bool GATED, bool TABLED>
+template <int WIDTH, bool GATED, bool TABLED, int BITS>
 __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint32_t words_per_group) {
     // each workgroup scans words_per_group words of the map (few for a small map, so that it still spreads over the chip),
     // gathers the marked elements in LDS, then its eight 32-lane groups take them in turn
@@ -369,11 +400,12 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
     const uint8_t* record = p.records + uint64_t(expert) * p.stride;
     const uint32_t a_row = p.a_rows ? uint32_t(p.a_rows[pos]) / p.a_div : pos;
     const uint16_t* xr = p.a + uint64_t(a_row) * K;
-    constexpr int DW = WIDTH / 8, kAhead = 4;   // a lane's next four blocks are fetched together: one memory latency, not four
+    static_assert(WIDTH * BITS >= 32 && !(TABLED && BITS == 8), "a block is whole code words; the table holds Q4 chain sums");
+    constexpr int DW = WIDTH * BITS / 32, XV = WIDTH >= 8 ? WIDTH / 8 : 1, kAhead = 4;   // a lane's next four blocks are fetched together: one memory latency, not four
     float result[2] = {0, 0};
     const uint32_t blocks = K / WIDTH;
     for (uint32_t b0 = lane; b0 < blocks; b0 += 32 * kAhead) {
-        uint4 xv[kAhead][WIDTH / 8];
+        uint4 xv[kAhead][XV];
         uint32_t words[kAhead][GATED ? 2 : 1][DW];
         uint16_t scale_bits[kAhead][GATED ? 2 : 1], bias_bits[kAhead][GATED ? 2 : 1];
         // the block's BF16-rounded chain sum depends on the row only: with 16-element blocks it comes from the table the
@@ -383,13 +415,18 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) {
             const uint32_t b = min(b0 + 32u * u, blocks - 1);   // past the end: the last block again, not used
+            if constexpr (WIDTH >= 8) {
 #pragma unroll
-            for (int i = 0; i < WIDTH / 8; ++i) xv[u][i] = *reinterpret_cast<const uint4*>(xr + b * WIDTH + 8 * i);
+                for (int i = 0; i < WIDTH / 8; ++i) xv[u][i] = *reinterpret_cast<const uint4*>(xr + b * WIDTH + 8 * i);
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>(xr + b * WIDTH);   // four inputs
+                xv[u][0] = make_uint4(v.x, v.y, 0, 0);
+            }
             chain[u] = tabled ? p.asum16[uint64_t(a_row) * (K / 16) + b] : 0.0f;
             const uint32_t g = n * groups + (b * WIDTH) / 64;
 #pragma unroll
             for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
-                const uint32_t* src = reinterpret_cast<const uint32_t*>(record + p.off[proj * 3] + uint64_t(n) * (K / 2)) + b * DW;
+                const uint32_t* src = reinterpret_cast<const uint32_t*>(record + p.off[proj * 3] + uint64_t(n) * (K * BITS / 8)) + b * DW;
 #pragma unroll
                 for (int i = 0; i < DW; ++i) words[u][proj][i] = src[i];
                 scale_bits[u][proj] = reinterpret_cast<const uint16_t*>(record + p.off[proj * 3 + 1])[g];
@@ -401,20 +438,27 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
             if (b0 + 32u * u >= blocks) break;
             float xb[WIDTH];
 #pragma unroll
-            for (int i = 0; i < WIDTH; i += 8) {
+            for (int i = 0; i < WIDTH; i += 2) {
                 const uint4 v = xv[u][i / 8];
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                for (int q = 0; q < 4; ++q) { xb[i + 2 * q] = __uint_as_float(w[q] << 16); xb[i + 2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u); }
+                xb[i] = __uint_as_float(w[(i % 8) / 2] << 16); xb[i + 1] = __uint_as_float(w[(i % 8) / 2] & 0xffff0000u);
             }
             float sum = chain[u];
-            if (!tabled) {
+            if constexpr (BITS == 8) {
+#pragma unroll
+                for (int i = 0; i < WIDTH; ++i) sum += xb[i];
+            } else if (!tabled) {
 #pragma unroll
                 for (int i = 0; i < WIDTH; i += 4) sum += bf(bf(bf(xb[i] + xb[i + 1]) + xb[i + 2]) + xb[i + 3]);
             }
 #pragma unroll
             for (int proj = 0; proj < (GATED ? 2 : 1); ++proj) {
                 float dot = 0;
+                if constexpr (BITS == 8) {
+                    // (a BF16 value times a byte code is exact in fp32: the fused multiply-add rounds as the reference's multiply and add)
+#pragma unroll
+                    for (int i = 0; i < WIDTH; ++i) dot = __builtin_fmaf(xb[i], float((words[u][proj][i / 4] >> (8 * (i % 4))) & 0xffu), dot);
+                } else
 #pragma unroll
                 for (int i = 0; i < WIDTH; i += 8) {
                     // nibble j of a word is element j: the even ones and the odd ones as bytes, each converted by one byte-to-float instruction
@@ -634,13 +678,13 @@ void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, co
     hipLaunchKernelGGL(router_refine_kernel, dim3((T + 3) / 4), dim3(256), 4 * K * 2, s, xb, wb, offsets, norms, T, E, K, topk, logits);
 }
 
-void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, int32_t* status) {
+void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, float* plain, int32_t* status) {
     const uint32_t items = rows * (K / 64);
-    hipLaunchKernelGGL(prefill_rows_kernel, dim3((items + 255) / 256), dim3(256), 0, s, x, rows, K, xb, sums, sums16, status);
+    hipLaunchKernelGGL(prefill_rows_kernel, dim3((items + 255) / 256), dim3(256), 0, s, x, rows, K, xb, sums, sums16, plain, status);
 }
-void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16) {
+void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16, bool plain) {
     const uint32_t items = rows_max * (K / 64);
-    hipLaunchKernelGGL(prefill_sums_kernel, dim3((items + 255) / 256), dim3(256), 0, s, xb, rows_ptr, rows_max, K, sums, sums16);
+    hipLaunchKernelGGL(prefill_sums_kernel, dim3((items + 255) / 256), dim3(256), 0, s, xb, rows_ptr, rows_max, K, sums, sums16, plain);
 }
 void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
                           int32_t* tile_rows, int32_t* tile_count) {
@@ -652,17 +696,25 @@ static uint32_t prefill_gemm_lds(uint32_t K) { const uint32_t groups = K / 64; r
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles) {
     const dim3 grid(gated ? p.N / 64 : p.N / 128, max_tiles);
     const uint32_t lds = prefill_gemm_lds(p.K);
-    if (gated) hipLaunchKernelGGL(prefill_gemm_kernel<true>, grid, dim3(256), lds, s, p);
-    else hipLaunchKernelGGL(prefill_gemm_kernel<false>, grid, dim3(256), lds, s, p);
+    if (p.bits == 8) {
+        if (gated) hipLaunchKernelGGL((prefill_gemm_kernel<true, 8>), grid, dim3(256), lds, s, p);
+        else hipLaunchKernelGGL((prefill_gemm_kernel<false, 8>), grid, dim3(256), lds, s, p);
+    } else {
+        if (gated) hipLaunchKernelGGL((prefill_gemm_kernel<true, 4>), grid, dim3(256), lds, s, p);
+        else hipLaunchKernelGGL((prefill_gemm_kernel<false, 4>), grid, dim3(256), lds, s, p);
+    }
 }
 void launch_prefill_patch(hipStream_t s, const PrefillGemm& p, bool gated) {
     const bool wide = p.K % 512 == 0 && p.N % 8 == 0;     // the reference's lane-width rule (metal.mm:649-674)
     const uint32_t per = p.near_words >= kPatchWordsMax * 1024u ? kPatchWordsMax : 64u;   // words of the map per workgroup
     const dim3 grid((p.near_words + per - 1) / per);
-    const bool tabled = wide && p.asum16;                 // the table holds sums of 16-element blocks
-#define ZC_PATCH(W, G, T) hipLaunchKernelGGL((prefill_patch_kernel<W, G, T>), grid, dim3(256), 0, s, p, per)
-    if (gated) { if (tabled) ZC_PATCH(16, true, true); else if (wide) ZC_PATCH(16, true, false); else ZC_PATCH(8, true, false); }
-    else { if (tabled) ZC_PATCH(16, false, true); else if (wide) ZC_PATCH(16, false, false); else ZC_PATCH(8, false, false); }
+    const bool tabled = wide && p.asum16 && p.bits == 4;  // the table holds the Q4 chain sums of 16-element blocks
+#define ZC_PATCH(W, G, T, B) hipLaunchKernelGGL((prefill_patch_kernel<W, G, T, B>), grid, dim3(256), 0, s, p, per)
+    if (p.bits == 8) {   // the Q8 lanes are half as wide (metal.mm:649-674)
+        if (gated) { if (wide) ZC_PATCH(8, true, false, 8); else ZC_PATCH(4, true, false, 8); }
+        else { if (wide) ZC_PATCH(8, false, false, 8); else ZC_PATCH(4, false, false, 8); }
+    } else if (gated) { if (tabled) ZC_PATCH(16, true, true, 4); else if (wide) ZC_PATCH(16, true, false, 4); else ZC_PATCH(8, true, false, 4); }
+    else { if (tabled) ZC_PATCH(16, false, true, 4); else if (wide) ZC_PATCH(16, false, false, 4); else ZC_PATCH(8, false, false, 4); }
 #undef ZC_PATCH
 }
 // (hidden and intermediate sizes up to 4096: the product kernel keeps a whole K of scales, biases and chain sums in LDS)

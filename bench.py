@@ -162,6 +162,7 @@ def main():
     ap.add_argument("--capped-homes", type=int, default=12,
                     help="--extra: pinned-host homes of the capped-HBM run's records; layer l shares the home of layer l mod this number "
                          "(48 distinct homes would pin 130 GB of host memory, more than this pool's boxes grant; 24 are 65 GB)")
+    ap.add_argument("--capped-only", action="store_true", help="--extra: only the capped-HBM runs")
     ap.add_argument("--calibrate", action="store_true", help="also run one 1 GiB device-to-device copy (a dispatch of known traffic for counter runs)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: rewrite the tracked traffic file from the output folders of the two counter runs")
@@ -304,35 +305,36 @@ def main():
     if args.extra:
         extra = {}
         quick = max(8, args.steps // 2)
-        if T == 1:
-            off = run(stack, cfg, L, 1, quick, 2, speculate=False)
-            extra["stack_batch1_without_guessing"] = {"tokens_per_s": 1 / (off["ms"] * 1e-3), "ms_per_step": off["ms"],
-                                                      "GBps": off["bytes"] / (off["ms"] * 1e-3) / 1e9}
-        r8 = run(stack, cfg, L, 8, quick, 2)
-        extra["stack_batch8"] = {"tokens_per_s": 8 / (r8["ms"] * 1e-3), "ms_per_step": r8["ms"], "GBps": r8["bytes"] / (r8["ms"] * 1e-3) / 1e9,
-                                 "frac_of_hbm_peak": r8["bytes"] / (r8["ms"] * 1e-3) / 8e12, "distinct_experts_per_layer": r8["unique"],
-                                 "kernel": "zc::decode_multi_kernel"}
-        for tokens in (32, 64):   # one launch of the kernel for nine to sixty-four tokens
-            rw = run(stack, cfg, L, tokens, max(4, quick // 4), 1, inputs=2)
-            extra[f"stack_batch{tokens}"] = {"tokens_per_s": tokens / (rw["ms"] * 1e-3), "ms_per_step": rw["ms"], "GBps": rw["bytes"] / (rw["ms"] * 1e-3) / 1e9,
-                                             "distinct_experts_per_layer": rw["unique"], "kernel": "zc::decode_wide_kernel"}
-        # The same records behind routers with a milder popularity skew (Zipf exponent 0.5: the offsets span 3.1 instead
-        # of 6.9) and with none at all, so that consecutive tokens share fewer experts and a batch of eight touches
-        # several times more records.
-        for name, exponent in (("mild_skew_zipf_0.5", 0.5), ("no_skew", None)):
-            offsets = [ctx.upload(synth.zipf_offsets(cfg.experts, (workload.BASE_SEED + 4 * 1000 + l) * 16 + 5, exponent))
-                       for l in range(L)] if exponent else [None] * L
-            other = ctx.stack_create(cfg, [z.Layer(w.router.ptr, o.ptr if o else None, w.shared_gate.ptr, w.shared_record.ptr,
-                                                   w.records.ptr, w.stride) for w, o in zip(layers, offsets)], 8)
-            extra[name] = {}
-            for tokens, spec in ((1, True), (1, False), (8, True)):
-                m = run(other, cfg, L, tokens, quick, 2, speculate=spec)
-                extra[name][f"batch{tokens}" + ("" if spec else "_without_guessing")] = {
-                    "tokens_per_s": tokens / (m["ms"] * 1e-3), "ms_per_step": m["ms"], "GBps": m["bytes"] / (m["ms"] * 1e-3) / 1e9,
-                    "distinct_experts_per_layer": m["unique"], "experts_repeated_from_previous_step": m["repeat_share"]}
-            ctx.stack_destroy(other)
-            for o in offsets:
-                if o: ctx.free(o)
+        if not args.capped_only:
+            if T == 1:
+                off = run(stack, cfg, L, 1, quick, 2, speculate=False)
+                extra["stack_batch1_without_guessing"] = {"tokens_per_s": 1 / (off["ms"] * 1e-3), "ms_per_step": off["ms"],
+                                                          "GBps": off["bytes"] / (off["ms"] * 1e-3) / 1e9}
+            r8 = run(stack, cfg, L, 8, quick, 2)
+            extra["stack_batch8"] = {"tokens_per_s": 8 / (r8["ms"] * 1e-3), "ms_per_step": r8["ms"], "GBps": r8["bytes"] / (r8["ms"] * 1e-3) / 1e9,
+                                     "frac_of_hbm_peak": r8["bytes"] / (r8["ms"] * 1e-3) / 8e12, "distinct_experts_per_layer": r8["unique"],
+                                     "kernel": "zc::decode_multi_kernel"}
+            for tokens in (32, 64):   # one launch of the kernel for nine to sixty-four tokens
+                rw = run(stack, cfg, L, tokens, max(4, quick // 4), 1, inputs=2)
+                extra[f"stack_batch{tokens}"] = {"tokens_per_s": tokens / (rw["ms"] * 1e-3), "ms_per_step": rw["ms"], "GBps": rw["bytes"] / (rw["ms"] * 1e-3) / 1e9,
+                                                 "distinct_experts_per_layer": rw["unique"], "kernel": "zc::decode_wide_kernel"}
+            # The same records behind routers with a milder popularity skew (Zipf exponent 0.5: the offsets span 3.1 instead
+            # of 6.9) and with none at all, so that consecutive tokens share fewer experts and a batch of eight touches
+            # several times more records.
+            for name, exponent in (("mild_skew_zipf_0.5", 0.5), ("no_skew", None)):
+                offsets = [ctx.upload(synth.zipf_offsets(cfg.experts, (workload.BASE_SEED + 4 * 1000 + l) * 16 + 5, exponent))
+                           for l in range(L)] if exponent else [None] * L
+                other = ctx.stack_create(cfg, [z.Layer(w.router.ptr, o.ptr if o else None, w.shared_gate.ptr, w.shared_record.ptr,
+                                                       w.records.ptr, w.stride) for w, o in zip(layers, offsets)], 8)
+                extra[name] = {}
+                for tokens, spec in ((1, True), (1, False), (8, True)):
+                    m = run(other, cfg, L, tokens, quick, 2, speculate=spec)
+                    extra[name][f"batch{tokens}" + ("" if spec else "_without_guessing")] = {
+                        "tokens_per_s": tokens / (m["ms"] * 1e-3), "ms_per_step": m["ms"], "GBps": m["bytes"] / (m["ms"] * 1e-3) / 1e9,
+                        "distinct_experts_per_layer": m["unique"], "experts_repeated_from_previous_step": m["repeat_share"]}
+                ctx.stack_destroy(other)
+                for o in offsets:
+                    if o: ctx.free(o)
         # The capped-HBM run of the same configuration: the records' home is pinned host memory and 2000 of the 24576
         # records fit in HBM slots.  The host cannot pin all 130 GB, so the 48 layers share --capped-homes pinned homes
         # (layer l holds the records of layer l mod that number; routers, shared experts and offsets are every layer's
@@ -350,55 +352,63 @@ def main():
         extra["capped_hbm"] = {}
         # 2000 slots (the configuration), and as many slots as one token selects experts per step (48 x top-10 = 480): fewer than
         # the eight rotating inputs touch, so every step misses and the slots turn over
-        for slots, batches in ((max(cfg.topk + 2, 2000 * CL // 48), (1, 8)), (CL * cfg.topk, (1,))):
-            capped = workload.StoreBackedStack(ctx, cfg, [workload.BASE_SEED + 4 * 1000 + l for l in range(CL)], ("zipf", 1.1), slots, home_layers=homes)
+        # ... and the 2000 slots again behind routers without any skew, where consecutive tokens share fewer experts: the
+        # steady state keeps missing
+        big = max(cfg.topk + 2, 2000 * CL // 48)
+        for name, slots, batches, skew in ((f"{big}_slots", big, (1, 8), ("zipf", 1.1)), (f"{CL * cfg.topk}_slots", CL * cfg.topk, (1,), ("zipf", 1.1)),
+                                           (f"{big}_slots_no_router_skew", big, (1,), None), (f"{big // 4}_slots_no_router_skew", big // 4, (1,), None)):
+            capped = workload.StoreBackedStack(ctx, cfg, [workload.BASE_SEED + 4 * 1000 + l for l in range(CL)], skew, slots, home_layers=homes)
             cstack = capped.decode_stack(8)
-            report = {"layers": CL, "hbm_slots": int(slots), "records": CL * cfg.experts,
+            report = {"layers": CL, "hbm_slots": int(slots), "records": CL * cfg.experts, "router_skew": list(skew) if skew else None,
                       "record_homes": homes, "pinned_home_bytes": homes * cfg.experts * int(capped.store.stride)}
             for tokens in batches:
                 xs = [workload.hidden_rows(ctx, tokens, cfg.hidden, workload.BASE_SEED + 4 * 7 + tokens + 97 * i) for i in range(INPUTS)]
                 out = ctx.alloc(tokens * cfg.hidden * 4)
                 t0 = time.perf_counter()
                 ctx.stack_decode(cstack, xs[0], tokens, out)      # cold: every record comes over the host link
+                ctx.finish()
                 cold = time.perf_counter() - t0
                 for i in range(2 * INPUTS):
                     ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
-                ctx.finish(); ctx.moe_check()
+                ctx.finish(); ctx.moe_check(); ctx.stack_settle(cstack)
                 seen0, st0 = capped.store.table_stats(), capped.store.stats()
-                reads0, slot0, home0, fill0, evict0 = seen0.reads, seen0.slot_reads, seen0.home_read_bytes, st0.bytes, st0.evictions
+                reads0, slot0, home0, fill0, evict0, joined0 = seen0.reads, seen0.slot_reads, seen0.home_read_bytes, st0.bytes, st0.evictions, seen0.joined
                 n_steps = max(16, args.steps)
                 t0 = time.perf_counter()
                 for i in range(n_steps):
                     ctx.stack_decode(cstack, xs[i % INPUTS], tokens, out)
+                ctx.finish()
                 dt = (time.perf_counter() - t0) / n_steps
-                ctx.moe_check()
+                ctx.moe_check(); ctx.stack_settle(cstack)
                 seen, st = capped.store.table_stats(), capped.store.stats()
                 report[f"batch{tokens}"] = {
                     "ms_per_step": dt * 1e3, "us_per_layer": dt / CL * 1e6, "tokens_per_s": tokens / dt * CL / 48 * 48 / CL,
                     "first_step_ms": cold * 1e3, "slot_hit_rate": (seen.slot_reads - slot0) / max(1, seen.reads - reads0),
                     "bytes_read_from_home_per_token": (seen.home_read_bytes - home0) / n_steps / tokens,
                     "bytes_filled_into_slots_per_token": (st.bytes - fill0) / n_steps / tokens,
-                    "evictions_per_step": (st.evictions - evict0) / n_steps}
+                    "evictions_per_step": (st.evictions - evict0) / n_steps,
+                    "fills_joined_by_a_launch_per_step": (seen.joined - joined0) / n_steps}
                 for b in xs + [out]:
                     ctx.free(b)
-            extra["capped_hbm"][f"{slots}_slots"] = report
+            extra["capped_hbm"][name] = report
             ctx.stack_destroy(cstack)
             capped.close()
-        # Single-layer configurations: decode batches through the exact operator path, and batches through the
-        # sorted-token grouped product on the bf16 matrix cores.
-        # BASELINE configs[1]: continuous-batching decode of the single-layer shape behind N(0, 0.5) router offsets: GEMV
-        # bandwidth over the distinct records of a step, and the expert dedup across its tokens (slots per distinct expert)
-        extra["single_layer_q4_one_launch_normal_0.5"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50, skew=("normal", 0.5)) for t in (1, 8, 32, 64)]
-        extra["single_layer_q4_one_launch"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50) for t in (1, 8, 32, 64)]
-        # raw random inputs behind an unskewed router share next to no experts from one step to the next: every guess of
-        # the one-token kernel misses, which prices the guessing at its worst
-        extra["single_layer_q4_one_launch_all_guesses_miss"] = [one_launch_layer(ctx, "S", 1, 200, skew=None, speculate=on) for on in (True, False)]
-        extra["single_layer_q4_normal_0.5"] = [single_layer(ctx, "S", t, False, 30, skew=("normal", 0.5)) for t in (1, 8, 32, 64)]
-        extra["single_layer_q4"] = [single_layer(ctx, "S", t, False, 50) for t in (1, 8, 32, 64)]
-        extra["single_layer_mixed_one_launch"] = [one_launch_layer(ctx, "S-mixed", t, 100) for t in (1, 8, 16)]
-        extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8, 16)]
-        extra["prefill_q4"] = [single_layer(ctx, "S", t, True, 20) for t in (32, 64, 256, 2048)]
-        extra["prefill_mixed"] = [single_layer(ctx, "S-mixed", t, True, 20, skew=None) for t in (256, 2048)]
+        if not args.capped_only:
+            # Single-layer configurations: decode batches through the exact operator path, and batches through the
+            # sorted-token grouped product on the bf16 matrix cores.
+            # BASELINE configs[1]: continuous-batching decode of the single-layer shape behind N(0, 0.5) router offsets: GEMV
+            # bandwidth over the distinct records of a step, and the expert dedup across its tokens (slots per distinct expert)
+            extra["single_layer_q4_one_launch_normal_0.5"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50, skew=("normal", 0.5)) for t in (1, 8, 32, 64)]
+            extra["single_layer_q4_one_launch"] = [one_launch_layer(ctx, "S", t, 200 if t <= 8 else 50) for t in (1, 8, 32, 64)]
+            # raw random inputs behind an unskewed router share next to no experts from one step to the next: every guess of
+            # the one-token kernel misses, which prices the guessing at its worst
+            extra["single_layer_q4_one_launch_all_guesses_miss"] = [one_launch_layer(ctx, "S", 1, 200, skew=None, speculate=on) for on in (True, False)]
+            extra["single_layer_q4_normal_0.5"] = [single_layer(ctx, "S", t, False, 30, skew=("normal", 0.5)) for t in (1, 8, 32, 64)]
+            extra["single_layer_q4"] = [single_layer(ctx, "S", t, False, 50) for t in (1, 8, 32, 64)]
+            extra["single_layer_mixed_one_launch"] = [one_launch_layer(ctx, "S-mixed", t, 100) for t in (1, 8, 16)]
+            extra["single_layer_mixed"] = [single_layer(ctx, "S-mixed", t, False, 50) for t in (1, 8, 16)]
+            extra["prefill_q4"] = [single_layer(ctx, "S", t, True, 20) for t in (32, 64, 256, 2048)]
+            extra["prefill_mixed"] = [single_layer(ctx, "S-mixed", t, True, 20, skew=None) for t in (256, 2048)]
         result["extra"] = extra
 
     print(json.dumps(result))

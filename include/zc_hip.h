@@ -308,11 +308,16 @@ typedef struct {
     uint64_t slot_reads;       /* ... from an HBM slot */
     uint64_t home_reads;       /* ... from the record's home over the host link */
     uint64_t home_read_bytes;
-    uint64_t switched;         /* finished fills whose table entry moved to the slot */
+    uint64_t switched;         /* fills whose table entry moved to the slot (finished, or joined) */
+    uint64_t joined;           /* ... of which the next launch was made to wait for the fill (zc_hip_store_table_refresh_joining) */
     uint64_t not_admitted;     /* misses that found every slot still loading */
 } zc_store_table_stats;
 zc_status zc_hip_store_table(zc_hip_store* store, const void* const** table);
 zc_status zc_hip_store_table_refresh(zc_hip_store* store);
+/* The same, and the entries of fills still in flight switch to their slots too: whatever the context's stream runs next
+ * waits for those fills on the device (ExpertCache::acquire's "loading join", storage.cpp:636-641, for a whole launch), so a
+ * record that an earlier launch read over the host link is not read over it a second time.  zc_hip_stack_decode uses this. */
+zc_status zc_hip_store_table_refresh_joining(zc_hip_store* store);
 zc_status zc_hip_store_table_observe(zc_hip_store* store, uint32_t layer, const int32_t* ids, uint32_t count);
 /* The same for a launch that ran every layer: ids [layers][per_layer].  All records that the launch read from slots are touched
  * before any record read from home is admitted, whatever their layers, so a miss never takes the slot of a record the same
@@ -323,12 +328,19 @@ zc_status zc_hip_store_geometry(const zc_hip_store* store, uint32_t* layers, uin
 /* A decode stack whose routed records live in an expert store (the capped-HBM run: model.cpp:431-557 with the cache of
  * storage.cpp:525-725 in the loop).  host_layers[l].expert_records is ignored; the store must have n_layers layers of
  * cfg's records, and max_tokens <= 64.  zc_hip_stack_decode on such a stack is ONE launch that reads every record
- * through the store's table (zc_hip_store_table), then waits for the launch on the host, copies the routes back and
- * hands them to zc_hip_store_table_observe, so that the records this step read from their homes are in HBM slots for
- * the steps to come.  Output bytes are those of a stack with all records resident.  flags bit 0 (layer by layer) is
- * refused with ZC_INVALID_ARGUMENT. */
+ * through the store's table (zc_hip_store_table).  Before the launch the fills that earlier launches caused switch to
+ * their slots, and the launch waits for the unfinished ones on the device (zc_hip_store_table_refresh_joining); after it
+ * the routes are copied back and handed to zc_hip_store_table_observe_layers, so that the records this step read from
+ * their homes are in HBM slots for the steps to come (the previous step's experts, which the next step is most likely to
+ * pick again -- the reference's prefetch on predicted experts, model.cpp:438-445, 489-500 -- are therefore in their slots
+ * before the launch that needs them).  While launches read nothing from a home, the host looks at a launch's routes only
+ * after the next launch has been enqueued and never waits for the GPU; a launch that read from a home is observed at once
+ * until that stops.  zc_hip_stack_settle observes a launch that is still waiting to be looked at (before reading the
+ * store's statistics, say).  Output bytes are those of a stack with all records resident.  flags bit 0 (layer by layer)
+ * is refused with ZC_INVALID_ARGUMENT. */
 zc_status zc_hip_stack_create_with_store(zc_hip_ctx* ctx, const zc_moe_config* cfg, const zc_moe_layer* host_layers,
                                          uint32_t n_layers, uint32_t max_tokens, zc_hip_store* store, zc_hip_stack** out);
+zc_status zc_hip_stack_settle(zc_hip_ctx* ctx, zc_hip_stack* stack);
 /* ---- Statistics and stage labels (Metal::label, metal.mm:267-270; KernelConfig::profile; Model::stats, model.cpp:706-732)
  * zc_hip_profile(on != 0) starts a recording: from then on every operator call through the context adds one row -- the
  * label current at the call, the operator's name, and the GPU time between two events placed around its launches (an

@@ -224,6 +224,27 @@ def test_record_table_shows_a_slot_only_while_it_holds_the_finished_record():
     assert table[8 + 3] != homes[8 + 3]
     check_every_entry()
 
+    # The joining refresh (the "loading join" of a whole launch): the entry of a fill still in flight moves to its slot at
+    # once and the fill is waited for -- on a GPU by the stream, here by finishing it; a fill that the test still holds
+    # cannot be joined.
+    s.hold(1, 5)
+    s.table_observe(1, [5])
+    s.table_refresh()
+    assert table[8 + 5] == homes[8 + 5]
+    with pytest.raises(z.ZcError):
+        s.table_refresh_joining()
+    s.hold(1, 5, False)                        # (letting go of the hold finishes the fill)
+    s.hold(1, 6)
+    s.table_observe(1, [6])
+    s.hold(1, 6, False)
+    before = s.table_stats()
+    s.table_refresh_joining()
+    after = s.table_stats()
+    assert table[8 + 5] != homes[8 + 5] and table[8 + 6] != homes[8 + 6] and after.switched == before.switched + 2
+    check_every_entry()
+    s.table_observe_layers(np.array([[-1, -1], [5, -1]], np.int32))   # the router's padding id is no record
+    assert s.table_stats().reads == after.reads + 1
+
     s.table_observe(0, [4, 5, 6])               # three slots, three more records: earlier ones lose their slots at once
     assert sum(table[k] != homes[k] for k in range(16)) <= 3
     check_every_entry()                         # entries of evicted records are back at home before the slot is overwritten

@@ -294,7 +294,7 @@ zc_status zc_hip_stats(zc_hip_ctx* ctx, const zc_hip_store* store, char* json, u
                ", \"prefetch_claims\": " + std::to_string(c.prefetch_claims) + ", \"prefetch_unclaimed\": " + std::to_string(c.prefetch_unclaimed) +
                ", \"record_table\": {\"reads\": " + std::to_string(t.reads) + ", \"slot_reads\": " + std::to_string(t.slot_reads) +
                ", \"home_reads\": " + std::to_string(t.home_reads) + ", \"home_read_bytes\": " + std::to_string(t.home_read_bytes) +
-               ", \"switched\": " + std::to_string(t.switched) + ", \"not_admitted\": " + std::to_string(t.not_admitted) + "}}";
+               ", \"switched\": " + std::to_string(t.switched) + ", \"joined\": " + std::to_string(t.joined) + ", \"not_admitted\": " + std::to_string(t.not_admitted) + "}}";
     }
     out += "}";
     if (needed) *needed = out.size() + 1;
@@ -833,8 +833,13 @@ struct zc_hip_stack {
     void* workspace = nullptr; float *xa = nullptr, *xb = nullptr;
     // routed records behind an expert store: the kernels take every record's address from the store's table
     zc_hip_store* store = nullptr;
-    int32_t* route_ids = nullptr; float* route_weights = nullptr;   // [L][tokens][topk] device copies of every launch's routes
-    int32_t* route_ids_host = nullptr;                               // pinned
+    // [L][tokens][topk] device copies of a launch's routes and pinned host copies (+ one status word each), two of each: the
+    // host may look at one launch's routes while the next launch runs
+    int32_t* route_ids[2] = {nullptr, nullptr}; float* route_weights = nullptr;
+    int32_t* route_ids_host[2] = {nullptr, nullptr};
+    hipEvent_t routes_copied[2] = {nullptr, nullptr};
+    uint32_t turn = 0; int pending = -1; uint32_t pending_per_layer = 0;   // pending: the turn whose routes the store has not seen yet
+    bool defer = true;                 // the last observed launch read nothing from a record's home: the next one is observed late
 };
 
 namespace {
@@ -926,11 +931,14 @@ static zc_status create_stack(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_
         if (!st->persistent_ok) return cleanup(fail(ZC_INVALID_ARGUMENT, "a stack behind an expert store needs a shape the single-launch kernels take"));
         const uint64_t routes = uint64_t(n_layers) * max_tokens * k * 4;
         if (zc_hip_alloc(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
-        st->route_ids = static_cast<int32_t*>(p);
-        if (zc_hip_alloc(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
         st->route_weights = static_cast<float*>(p);
-        if (zc_hip_alloc_host(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
-        st->route_ids_host = static_cast<int32_t*>(p);
+        for (int t = 0; t < 2; ++t) {
+            if (zc_hip_alloc(ctx, routes, &p)) return cleanup(ZC_BUDGET_EXCEEDED);
+            st->route_ids[t] = static_cast<int32_t*>(p);
+            if (zc_hip_alloc_host(ctx, routes + 4, &p)) return cleanup(ZC_BUDGET_EXCEEDED);   // the last word: the status at the end of the launch
+            st->route_ids_host[t] = static_cast<int32_t*>(p);
+            if (hipEventCreateWithFlags(&st->routes_copied[t], hipEventDisableTiming) != hipSuccess) return cleanup(fail(ZC_RUNTIME_ERROR, "HIP execution: cannot create an event"));
+        }
     }
     *out = st;
     return ZC_OK;
@@ -948,8 +956,10 @@ zc_status zc_hip_stack_destroy(zc_hip_ctx* ctx, zc_hip_stack* st) {
     if (!st) return ZC_OK;
     ZC_REQUIRE(ctx, "null context");
     for (void* p : {static_cast<void*>(st->workspace), static_cast<void*>(st->xa), static_cast<void*>(st->xb), static_cast<void*>(st->arena),
-                    static_cast<void*>(st->route_ids), static_cast<void*>(st->route_weights), static_cast<void*>(st->route_ids_host)})
+                    static_cast<void*>(st->route_ids[0]), static_cast<void*>(st->route_ids[1]), static_cast<void*>(st->route_weights),
+                    static_cast<void*>(st->route_ids_host[0]), static_cast<void*>(st->route_ids_host[1])})
         if (p) zc_hip_free(ctx, p);
+    for (hipEvent_t e : st->routes_copied) if (e) (void)hipEventDestroy(e);
     delete st;
     return ZC_OK;
 }
@@ -1024,7 +1034,7 @@ static zc_status launch_piece(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
         p.ids_trace = trace && trace->ids ? trace->ids + uint64_t(first) * k : nullptr;
         p.weights_trace = trace && trace->weights ? trace->weights + uint64_t(first) * k : nullptr;
         p.out_trace = trace && trace->outputs ? trace->outputs + uint64_t(first) * H : nullptr;
-        if (st->store && !p.ids_trace) { p.ids_trace = st->route_ids + uint64_t(first) * k; p.weights_trace = st->route_weights + uint64_t(first) * k; }
+        if (st->store && !p.ids_trace) { p.ids_trace = st->route_ids[st->turn] + uint64_t(first) * k; p.weights_trace = st->route_weights + uint64_t(first) * k; }
         p.clocks = trace && first == 0 ? reinterpret_cast<unsigned long long*>(trace->clocks) : nullptr;
         p.sync = st->sync; p.epoch = st->epoch; p.status = ctx->moe_status; p.spin_limit = st->wait_limit;
         st->epoch += 5 * L + 16;   // at most five barriers per layer; wraps modulo 2^32, the barrier compares epochs as signed differences
@@ -1055,6 +1065,29 @@ int zc_hip_stack_is_persistent(zc_hip_ctx* ctx, zc_hip_stack* st, uint32_t token
     if (st->store && tokens > 64) return 0;
     return launch_unit(ctx, st, tokens) ? 1 : 0;
 }
+// Waits for the routes of the launch that the store has not seen yet, and shows them to the store.
+static zc_status observe_pending(zc_hip_ctx* ctx, zc_hip_stack* st) {
+    (void)ctx;
+    if (st->pending < 0) return ZC_OK;
+    const int turn = st->pending;
+    st->pending = -1;
+    ZC_HIP(hipEventSynchronize(st->routes_copied[turn]));
+    const int32_t status = st->route_ids_host[turn][uint64_t(st->layers.size()) * st->max_tokens * st->cfg.topk];
+    // Only a launch that gave up waiting (bit 2) has no routes to observe; the other bits (an unroutable row, an input that is
+    // not BF16-valued) are sticky reports of this or an earlier call, and the router's padding id -1 is skipped one by one
+    // inside the observation.
+    if (status & 2) return ZC_OK;
+    zc_store_table_stats before{}, after{};
+    if (const zc_status s = zc_hip_store_table_stats(st->store, &before)) return s;
+    if (const zc_status s = zc_hip_store_table_observe_layers(st->store, st->route_ids_host[turn], st->pending_per_layer)) return s;
+    if (const zc_status s = zc_hip_store_table_stats(st->store, &after)) return s;
+    st->defer = after.home_reads == before.home_reads;
+    return ZC_OK;
+}
+zc_status zc_hip_stack_settle(zc_hip_ctx* ctx, zc_hip_stack* st) {
+    ZC_REQUIRE(ctx && st, "null argument");
+    return st->store ? observe_pending(ctx, st) : ZC_OK;
+}
 zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x, uint32_t tokens, float* out,
                               const zc_stack_trace* trace, uint32_t flags) {
     Timed timed(ctx, "stack_decode");
@@ -1066,7 +1099,7 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
     const uint32_t unit = (flags & 1u) ? 0u : launch_unit(ctx, st, tokens);
     if (st->store) {
         ZC_REQUIRE(unit && tokens <= unit, "a stack behind an expert store runs as one launch only");
-        if (const zc_status s = zc_hip_store_table_refresh(st->store)) return s;
+        if (const zc_status s = zc_hip_store_table_refresh_joining(st->store)) return s;
     }
     // More than eight tokens go through the single-launch kernels sixty-four (or eight) at a time, one launch per piece (tokens
     // do not interact inside a layer); every piece stays on the device from the first layer to the last.
@@ -1078,19 +1111,21 @@ zc_status zc_hip_stack_decode(zc_hip_ctx* ctx, zc_hip_stack* st, const float* x,
             if (const zc_status s = launch_piece(ctx, st, x + uint64_t(first) * H, piece, out + uint64_t(first) * H, trace, first, tokens, plan)) return s;
         }
         if (st->store) {
-            // The launch has read every record through the store's table.  Once it has finished, the store learns which
-            // records those were: hits are touched, misses are admitted and their fills start on the side stream.
+            // The launch reads every record through the store's table; afterwards the store learns which records those were:
+            // hits are touched, misses are admitted and their fills start on the side stream (the next launch waits for them on
+            // the device, see zc_hip_store_table_refresh_joining).  While launches read nothing from a record's home the routes
+            // of one launch are looked at only after the next one has been enqueued, so the host never waits for the GPU; once a
+            // launch has read from a home, launches are observed at once again: the sooner a fill starts, the fewer launches read
+            // that record over the host link.
             const uint64_t per_layer = uint64_t(tokens) * k;
-            const int32_t* routes = trace && trace->ids ? trace->ids : st->route_ids;
-            ZC_HIP(hipMemcpyAsync(st->route_ids_host, routes, L * per_layer * 4, hipMemcpyDeviceToHost, ctx->stream));
-            ZC_HIP(hipStreamSynchronize(ctx->stream));
-            int32_t status = 0;
-            ZC_HIP(hipMemcpy(&status, ctx->moe_status, 4, hipMemcpyDeviceToHost));
-            // Only a launch that gave up waiting (bit 2) has no routes to observe; the other bits (an unroutable row, an
-            // input that is not BF16-valued) are sticky reports of this or an earlier call, and an id outside the
-            // expert range is skipped one by one inside the observation.
-            if (!(status & 2))
-                if (const zc_status s = zc_hip_store_table_observe_layers(st->store, st->route_ids_host, uint32_t(per_layer))) return s;
+            const uint32_t turn = st->turn;
+            const int32_t* routes = trace && trace->ids ? trace->ids : st->route_ids[turn];
+            ZC_HIP(hipMemcpyAsync(st->route_ids_host[turn], routes, L * per_layer * 4, hipMemcpyDeviceToHost, ctx->stream));
+            ZC_HIP(hipMemcpyAsync(st->route_ids_host[turn] + uint64_t(L) * st->max_tokens * k, ctx->moe_status, 4, hipMemcpyDeviceToHost, ctx->stream));
+            ZC_HIP(hipEventRecord(st->routes_copied[turn], ctx->stream));
+            if (st->pending >= 0) { if (const zc_status s = observe_pending(ctx, st)) return s; }
+            st->pending = int(turn); st->pending_per_layer = uint32_t(per_layer); st->turn = turn ^ 1u;
+            if (!st->defer) { if (const zc_status s = observe_pending(ctx, st)) return s; }
         }
         return ZC_OK;
     }

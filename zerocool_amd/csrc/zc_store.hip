@@ -304,13 +304,23 @@ zc_status zc_hip_store_table(zc_hip_store* s, const void* const** table) {
         return ZC_OK;
     });
 }
-zc_status zc_hip_store_table_refresh(zc_hip_store* s) {
+static zc_status table_refresh(zc_hip_store* s, bool join) {
     if (!s || !s->mirror) return zc_fail(ZC_LOGIC_ERROR, "the store has no record table");
     return guarded([&] {
         size_t kept = 0;
         for (const size_t slot : s->in_flight) {
             const uint64_t key = s->arriving[slot];
-            const bool done = s->ctx ? hipEventQuery(s->filled[slot]) == hipSuccess : s->pending[slot] == kNone;
+            bool done = s->ctx ? hipEventQuery(s->filled[slot]) == hipSuccess : s->pending[slot] == kNone;
+            if (!done && join && s->cache->key_of(slot) == int64_t(key)) {
+                // ExpertCache::acquire's "loading join" for a whole launch: what the context's stream runs next waits, on the
+                // device, for the fill; the entry can point at the slot at once
+                if (s->ctx) ZC_STORE_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(zc_hip_stream(s->ctx)), s->filled[slot], 0));
+                else {
+                    if (s->held.count(s->pending[slot])) throw std::logic_error("waiting for a fill that the test still holds");
+                    finish_host_fill(s, slot);
+                }
+                done = true; ++s->seen.joined;
+            }
             if (!done) { s->in_flight[kept++] = slot; continue; }
             s->arriving[slot] = kNone;
             if (s->cache->key_of(slot) != int64_t(key)) continue;   // replaced before it was ever shown
@@ -324,6 +334,8 @@ zc_status zc_hip_store_table_refresh(zc_hip_store* s) {
         return ZC_OK;
     });
 }
+zc_status zc_hip_store_table_refresh(zc_hip_store* s) { return table_refresh(s, false); }
+zc_status zc_hip_store_table_refresh_joining(zc_hip_store* s) { return table_refresh(s, true); }
 // What one finished launch read: per layer the distinct valid experts, each classified by what the table showed AT THE LAUNCH
 // (nothing below has changed it yet).  First every record that was read from a slot is leased, then the records read from
 // home are admitted, then all leases go: a miss can only take the slot of a record that this launch did not use.

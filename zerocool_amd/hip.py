@@ -73,7 +73,7 @@ class StoreStats(C.Structure):
 
 
 class StoreTableStats(C.Structure):
-    _fields_ = [(n, C.c_uint64) for n in ("reads", "slot_reads", "home_reads", "home_read_bytes", "switched", "not_admitted")]
+    _fields_ = [(n, C.c_uint64) for n in ("reads", "slot_reads", "home_reads", "home_read_bytes", "switched", "joined", "not_admitted")]
 
 
 class StoreLease(C.Structure):
@@ -182,6 +182,9 @@ class Store:
 
     def table_refresh(self):
         self._check(self.lib.zc_hip_store_table_refresh(self.handle))
+
+    def table_refresh_joining(self):
+        self._check(self.lib.zc_hip_store_table_refresh_joining(self.handle))
 
     def table_observe(self, layer, ids):
         ids = np.ascontiguousarray(ids, np.int32)
@@ -451,6 +454,9 @@ class Context:
 
     def stack_set_speculation(self, stack, on):
         self._call("zc_hip_stack_set_speculation", stack, C.c_int(int(on)))
+
+    def stack_settle(self, stack):
+        self._call("zc_hip_stack_settle", stack)
 
     def stack_set_wait_limit(self, stack, polls):
         self._call("zc_hip_stack_set_wait_limit", stack, C.c_uint32(polls))

@@ -55,6 +55,9 @@ struct zc_hip_ctx {
     uint64_t retired = 0;              // tickets known complete and destroyed
     int32_t* moe_status = nullptr;     // device flag: an id outside [0,E) was seen
     hipEvent_t timer[2] = {nullptr, nullptr};
+    // The prefill layer runs its shared expert beside the router, the selection and the dispatch sort, which are chains of
+    // small kernels: a second stream of default priority, forked from and joined to `stream` by two events per call.
+    hipStream_t beside = nullptr; hipEvent_t fork = nullptr, join = nullptr;
     uint32_t affine_policy = 1;        // 0 literal lane kernels, 1 exact-integer matrix-core kernels where possible
     void* static_scratch = nullptr;    // this device's copy of the static scratch array
     std::mutex mutex;
@@ -145,6 +148,9 @@ zc_status zc_hip_destroy(zc_hip_ctx* ctx) {
     for (auto& b : ctx->blocks) hipFree(b.first);
     for (auto& b : ctx->host_blocks) hipHostFree(b.first);
     hipFree(ctx->moe_status);
+    if (ctx->beside) { hipStreamSynchronize(ctx->beside); hipStreamDestroy(ctx->beside); }
+    if (ctx->fork) hipEventDestroy(ctx->fork);
+    if (ctx->join) hipEventDestroy(ctx->join);
     hipStreamDestroy(ctx->stream);
     delete ctx;
     return ZC_OK;
@@ -656,6 +662,7 @@ struct PrefillSpace {
     int32_t *tile_expert, *tile_first, *tile_rows, *tile_count, *stile_expert, *stile_first, *stile_rows, *stile_count;
     uint32_t max_tiles, max_shared_tiles;
     uint32_t* near_bits;      // one bit per product element: recompute exactly
+    uint32_t* shared_near_bits;   // the same for the shared expert's products, which run beside the routed ones
     float* norms;             // |row| of the inputs and of the router's rows (the fast router's bound)
     uint64_t bytes;
 };
@@ -678,6 +685,7 @@ PrefillSpace carve_prefill(const zc_moe_config* c, uint32_t T, void* base) {
     w.ssum16 = (float*)take(uint64_t(T) * (c->inter / 16) * 4);
     w.norms = (float*)take((uint64_t(T) + c->experts) * 4);
     w.xplain = (float*)take(uint64_t(T) * (c->hidden / 64) * 4);
+    w.shared_near_bits = (uint32_t*)take(uint64_t(T) * std::max(c->hidden, c->inter) / 8);
     w.bytes = at;
     return w;
 }
@@ -713,17 +721,23 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     // whose logits nobody asks for gets exact logits only where the selection can see the difference (launch_prefill_router)
     const bool x_q4 = c->bits_gate_up == 4 || c->shared_bits_gate_up == 4, x_q8 = c->bits_gate_up == 8 || c->shared_bits_gate_up == 8;
     zc::launch_prefill_rows(s, x, T, H, w.xb, x_q4 ? w.xsum : nullptr, x_q4 ? w.xsum16 : nullptr, x_q8 ? w.xplain : nullptr, ctx->moe_status);
+    // the shared expert needs the bf16 rows and nothing of the routing: it runs on a stream of its own from here to the combine
+    if (!ctx->beside) {
+        ZC_HIP(hipStreamCreateWithFlags(&ctx->beside, hipStreamNonBlocking));
+        ZC_HIP(hipEventCreateWithFlags(&ctx->fork, hipEventDisableTiming)); ZC_HIP(hipEventCreateWithFlags(&ctx->join, hipEventDisableTiming));
+    }
+    hipStream_t s2 = ctx->beside;
+    ZC_HIP(hipEventRecord(ctx->fork, s)); ZC_HIP(hipStreamWaitEvent(s2, ctx->fork, 0));
     if (T >= 128 && !(trace && trace->logits)) zc::launch_prefill_router(s, x, w.xb, l->router, l->router_offsets, T, H, E, k, w.norms, w.base.logits);
     else zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
     zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
     zc::launch_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, w.base.selected, w.base.count, ctx->moe_status);
-    zc::launch_plain(s, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
+    zc::launch_plain(s2, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
     // operands of the matrix cores: bf16 rows and their group sums; work lists
-    const float margin = zc::kPrefillMargin;
     // the per-block chain sums pay where a lane of the recomputation has several blocks of a row (long rows); short rows form them in place
     const bool table_inter = I / 16 >= 128;
     zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
-    zc::launch_prefill_tiles(s, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
+    zc::launch_prefill_tiles(s2, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
     auto offsets_of = [&](const void* record, int shared, uint64_t* off, int first, int count) {
         for (int q = 0; q < count; ++q) {
             zc_linear lin; zc_hip_expert_linear(c, shared, record, first + q, &lin);
@@ -739,7 +753,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         g.records = static_cast<const uint8_t*>(l->expert_records); g.stride = l->record_stride; offsets_of(l->expert_records, 0, g.off, 0, 2);
         g.tile_expert = w.tile_expert; g.tile_first = w.tile_first; g.tile_rows = w.tile_rows; g.tile_count = w.tile_count;
         g.K = H; g.N = I; g.out_b = w.actb;
-        g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(n) * I / 32); g.near_margin = margin; g.ids = w.base.ids; g.slots = w.base.slots;
+        g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(n) * I / 32); g.near_margin = zc::prefill_margin(g.K); g.ids = w.base.ids; g.slots = w.base.slots;
         g.covered = w.base.offsets + E; g.experts = E;
         zc::launch_prefill_gemm(s, g, true, w.max_tiles);
         zc::launch_prefill_patch(s, g, true);
@@ -750,32 +764,33 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
         d.K = I; d.N = H; d.out_f = w.base.expert_out;
-        d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(n) * H / 32); d.near_margin = margin; d.ids = w.base.ids; d.slots = w.base.slots;
+        d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(n) * H / 32); d.near_margin = zc::prefill_margin(d.K); d.ids = w.base.ids; d.slots = w.base.slots;
         d.covered = w.base.offsets + E; d.experts = E;
         zc::launch_prefill_gemm(s, d, false, w.max_tiles);
         zc::launch_prefill_patch(s, d, false);
     }
-    {   // shared expert (model.cpp:482-485): one group of all the tokens
+    {   // shared expert (model.cpp:482-485): one group of all the tokens, beside the routed experts
         zc::PrefillGemm g{};
         g.bits = c->shared_bits_gate_up;
         g.a = w.xb; g.asum = g.bits == 4 ? w.xsum : w.xplain; g.asum16 = g.bits == 4 ? w.xsum16 : nullptr; g.a_rows = nullptr; g.a_div = 1;
         g.records = static_cast<const uint8_t*>(l->shared_record); g.stride = 0; offsets_of(l->shared_record, 1, g.off, 0, 2);
         g.tile_expert = w.stile_expert; g.tile_first = w.stile_first; g.tile_rows = w.stile_rows; g.tile_count = w.stile_count;
         g.K = H; g.N = I; g.out_b = w.sactb;
-        g.near_bits = w.near_bits; g.near_words = uint32_t(uint64_t(T) * I / 32); g.near_margin = margin; g.ids = nullptr; g.slots = nullptr;
-        zc::launch_prefill_gemm(s, g, true, w.max_shared_tiles);
-        zc::launch_prefill_patch(s, g, true);
+        g.near_bits = w.shared_near_bits; g.near_words = uint32_t(uint64_t(T) * I / 32); g.near_margin = zc::prefill_margin(g.K); g.ids = nullptr; g.slots = nullptr;
+        zc::launch_prefill_gemm(s2, g, true, w.max_shared_tiles);
+        zc::launch_prefill_patch(s2, g, true);
         zc::PrefillGemm d{};
         d.bits = c->shared_bits_down;
-        zc::launch_prefill_sums(s, w.sactb, nullptr, T, I, w.ssum, table_inter && d.bits == 4 ? w.ssum16 : nullptr, d.bits == 8);
+        zc::launch_prefill_sums(s2, w.sactb, nullptr, T, I, w.ssum, table_inter && d.bits == 4 ? w.ssum16 : nullptr, d.bits == 8);
         d.a = w.sactb; d.asum = w.ssum; d.asum16 = table_inter && d.bits == 4 ? w.ssum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = nullptr;
         d.records = g.records; d.stride = 0; offsets_of(l->shared_record, 1, d.off, 2, 1);
         d.tile_expert = w.stile_expert; d.tile_first = w.stile_first; d.tile_rows = w.stile_rows; d.tile_count = w.stile_count;
         d.K = I; d.N = H; d.out_f = w.base.shared;
-        d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(T) * H / 32); d.near_margin = margin; d.ids = nullptr; d.slots = nullptr;
-        zc::launch_prefill_gemm(s, d, false, w.max_shared_tiles);
-        zc::launch_prefill_patch(s, d, false);
+        d.near_bits = w.shared_near_bits; d.near_words = uint32_t(uint64_t(T) * H / 32); d.near_margin = zc::prefill_margin(d.K); d.ids = nullptr; d.slots = nullptr;
+        zc::launch_prefill_gemm(s2, d, false, w.max_shared_tiles);
+        zc::launch_prefill_patch(s2, d, false);
     }
+    ZC_HIP(hipEventRecord(ctx->join, s2)); ZC_HIP(hipStreamWaitEvent(s, ctx->join, 0));
     // weighted combine (model.cpp:553-556)
     zc::launch_moe_sum(s, w.base.expert_out, w.base.weights, w.base.shared, w.base.gate, T, H, k, out);
     ZC_LAUNCHED();

@@ -8,7 +8,7 @@
 // scale group of 64; per group the accumulator is folded as  total += scale * dot + bias * chain_sum  with the chain
 // sums precomputed per (row, group) exactly as the reference rounds them.  Only the order of the fp32 additions
 // differs from the reference, so results agree to a few fp32 steps before the BF16 rounding of the outputs.  Every sum
-// that lands within kPrefillMargin fp32 steps of a BF16 rounding boundary is then recomputed with the reference's exact
+// that lands within prefill_margin(K) of its term magnitudes of a BF16 rounding boundary is then recomputed with the reference's exact
 // lane arithmetic (about 2-3 % of the elements), which removes the rounding flips in practice; the path is still
 // specified by a tolerance (max relative error 2e-3 of the layer output), not as bit-exact.  Routing, dispatch and the
 // combine use the exact kernels.

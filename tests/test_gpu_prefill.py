@@ -67,7 +67,12 @@ def test_prefill_matches_the_exact_path(ctx, shape, tokens):
     assert rel(fast["out"], exact["out"]) <= TOLERANCE
     same = np.mean(fast["out"].view(np.uint32) == exact["out"].view(np.uint32))
     assert same > 0.9999, same
-    for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, x):
+    # a call that asks for no intermediates hands the slots' outputs to the combine as bf16: the same values, the same output
+    out, ws = ctx.alloc(tokens * cfg.hidden * 4), ctx.alloc(ctx.moe_prefill_workspace_bytes(cfg, tokens))
+    ctx.moe_prefill(cfg, weights.layer, x, tokens, out, ws)
+    ctx.moe_check()
+    assert out.numpy(f32).tobytes() == fast["out"].tobytes()
+    for b in (weights.router, weights.shared_gate, weights.shared_record, weights.records, x, out, ws):
         ctx.free(b)
 
 

@@ -717,6 +717,7 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     hipStream_t s = ctx->stream;
     const uint32_t H = c->hidden, I = c->inter, E = c->experts, k = c->topk;
     const uint64_t n = uint64_t(T) * k;
+    const bool half_out = !(trace && trace->expert_out) && reinterpret_cast<uintptr_t>(out) % 16 == 0;
     // router logits, top-k + softmax, dispatch (model.cpp:434-479), shared gate: the exact kernels, except that a long batch
     // whose logits nobody asks for gets exact logits only where the selection can see the difference (launch_prefill_router)
     const bool x_q4 = c->bits_gate_up == 4 || c->shared_bits_gate_up == 4, x_q8 = c->bits_gate_up == 8 || c->shared_bits_gate_up == 8;
@@ -731,12 +732,14 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     if (T >= 128 && !(trace && trace->logits)) zc::launch_prefill_router(s, x, w.xb, l->router, l->router_offsets, T, H, E, k, w.norms, w.base.logits);
     else zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
     zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
-    zc::launch_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, w.base.selected, w.base.count, ctx->moe_status);
-    zc::launch_plain(s2, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);
+    // dispatch sort and the routed experts' tile list: one launch for a long batch
+    const bool one_dispatch = zc::prefill_dispatch_fits(w.base.ids, T, k, E);
+    if (one_dispatch) zc::launch_prefill_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, ctx->moe_status, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
+    else zc::launch_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, w.base.selected, w.base.count, ctx->moe_status);
     // operands of the matrix cores: bf16 rows and their group sums; work lists
     // the per-block chain sums pay where a lane of the recomputation has several blocks of a row (long rows); short rows form them in place
     const bool table_inter = I / 16 >= 128;
-    zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
+    if (!one_dispatch) zc::launch_prefill_tiles(s, w.base.offsets, E, 0, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);
     zc::launch_prefill_tiles(s2, nullptr, 1, T, w.stile_expert, w.stile_first, w.stile_rows, w.stile_count);
     auto offsets_of = [&](const void* record, int shared, uint64_t* off, int first, int count) {
         for (int q = 0; q < count; ++q) {
@@ -763,7 +766,9 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         d.a = w.actb; d.asum = w.asum; d.asum16 = table_inter && d.bits == 4 ? w.asum16 : nullptr; d.a_rows = nullptr; d.a_div = 1; d.out_rows = w.base.slots;
         d.records = g.records; d.stride = g.stride; offsets_of(l->expert_records, 0, d.off, 2, 1);
         d.tile_expert = w.tile_expert; d.tile_first = w.tile_first; d.tile_rows = w.tile_rows; d.tile_count = w.tile_count;
-        d.K = I; d.N = H; d.out_f = w.base.expert_out;
+        d.K = I; d.N = H;
+        // nobody asks for the slots' outputs: they go to the combine as bf16 (BF16 values either way), in the same space
+        if (half_out) d.out_h = reinterpret_cast<uint16_t*>(w.base.expert_out); else d.out_f = w.base.expert_out;
         d.near_bits = w.near_bits; d.near_words = uint32_t(uint64_t(n) * H / 32); d.near_margin = zc::prefill_margin(d.K); d.ids = w.base.ids; d.slots = w.base.slots;
         d.covered = w.base.offsets + E; d.experts = E;
         zc::launch_prefill_gemm(s, d, false, w.max_tiles);
@@ -789,10 +794,12 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
         d.near_bits = w.shared_near_bits; d.near_words = uint32_t(uint64_t(T) * H / 32); d.near_margin = zc::prefill_margin(d.K); d.ids = nullptr; d.slots = nullptr;
         zc::launch_prefill_gemm(s2, d, false, w.max_shared_tiles);
         zc::launch_prefill_patch(s2, d, false);
+        zc::launch_plain(s2, l->shared_gate, 0, x, H, 1, T, w.base.gate, false);   // the gate dot of the combine: last, it is short
     }
     ZC_HIP(hipEventRecord(ctx->join, s2)); ZC_HIP(hipStreamWaitEvent(s, ctx->join, 0));
     // weighted combine (model.cpp:553-556)
-    zc::launch_moe_sum(s, w.base.expert_out, w.base.weights, w.base.shared, w.base.gate, T, H, k, out);
+    if (half_out) zc::launch_moe_sum_half(s, reinterpret_cast<const uint16_t*>(w.base.expert_out), w.base.weights, w.base.shared, w.base.gate, T, H, k, out);
+    else zc::launch_moe_sum(s, w.base.expert_out, w.base.weights, w.base.shared, w.base.gate, T, H, k, out);
     ZC_LAUNCHED();
     if (trace) {
         if (trace->logits) ZC_HIP(hipMemcpyAsync(trace->logits, w.base.logits, uint64_t(T) * E * 4, hipMemcpyDeviceToDevice, s));

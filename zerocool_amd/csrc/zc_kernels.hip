@@ -676,20 +676,27 @@ void launch_scatter(hipStream_t s, const float* x, const int32_t* positions, uin
 }
 // General top-k keeps the reference's eight strided partials: partial j takes
 // k = j, j+8, ...; partials are then added 0..7.  top-k 10 is the reference expression.
-template <int V>
-__global__ __launch_bounds__(256) void moe_sum_kernel(const float* __restrict__ experts, const float* __restrict__ weights, const float* __restrict__ shared,
+template <int V, bool HALF = false>
+__global__ __launch_bounds__(256) void moe_sum_kernel(const void* __restrict__ experts_in, const float* __restrict__ weights, const float* __restrict__ shared,
                                                       const float* __restrict__ gate, uint32_t T, uint32_t H, uint32_t topk, float* __restrict__ out) {
-    // V neighbouring columns per thread (one 16-byte load per slot when V is 4); every column keeps the scalar arithmetic
+    // V neighbouring columns per thread (one 16-byte load per slot when V is 4); every column keeps the scalar arithmetic.
+    // HALF: the expert outputs are stored as bf16 (they are BF16 values: the same numbers, half the bytes; V is 4 then).
     typedef float row_t __attribute__((ext_vector_type(V)));
     const uint32_t c = (blockIdx.x * blockDim.x + threadIdx.x) * V, t = blockIdx.y;
     if (c >= H || t >= T) return;
+    auto row_of = [&](uint64_t slot) {
+        if constexpr (HALF) {
+            const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(experts_in) + slot * H + c);
+            return row_t{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u)};
+        } else return *reinterpret_cast<const row_t*>(static_cast<const float*>(experts_in) + slot * H + c);
+    };
     row_t partial[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) partial[k] = row_t(0);
     if (topk == 10) {   // the reference's shape: all ten rows requested before the first is used
         row_t value[10]; float weight[10];
 #pragma unroll
-        for (int k = 0; k < 10; ++k) { value[k] = *reinterpret_cast<const row_t*>(experts + (uint64_t(t) * 10 + k) * H + c); weight[k] = weights[uint64_t(t) * 10 + k]; }
+        for (int k = 0; k < 10; ++k) { value[k] = row_of(uint64_t(t) * 10 + k); weight[k] = weights[uint64_t(t) * 10 + k]; }
 #pragma unroll
         for (int k = 0; k < 10; ++k) {
             const row_t product = value[k] * weight[k];
@@ -697,7 +704,7 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const float* __restrict__ 
         }
     } else
     for (uint32_t k = 0; k < topk; ++k) {
-        const row_t product = *reinterpret_cast<const row_t*>(experts + (uint64_t(t) * topk + k) * H + c) * weights[uint64_t(t) * topk + k];
+        const row_t product = row_of(uint64_t(t) * topk + k) * weights[uint64_t(t) * topk + k];
         if (k < 8) partial[k] = product; else partial[k % 8] = partial[k % 8] + product;
     }
     row_t sum = partial[0];
@@ -715,8 +722,13 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const float* __restrict__ 
 void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, const float* shared, const float* gate,
                     uint32_t T, uint32_t H, uint32_t topk, float* out) {
     const bool wide = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(experts) | reinterpret_cast<uintptr_t>(shared) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
-    if (wide) hipLaunchKernelGGL(moe_sum_kernel<4>, dim3((H / 4 + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
-    else hipLaunchKernelGGL(moe_sum_kernel<1>, dim3((H + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
+    if (wide) hipLaunchKernelGGL((moe_sum_kernel<4>), dim3((H / 4 + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
+    else hipLaunchKernelGGL((moe_sum_kernel<1>), dim3((H + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
+}
+// The same with the expert outputs as bf16 rows (H a multiple of four, every array sixteen-byte aligned).
+void launch_moe_sum_half(hipStream_t s, const uint16_t* experts, const float* weights, const float* shared, const float* gate,
+                         uint32_t T, uint32_t H, uint32_t topk, float* out) {
+    hipLaunchKernelGGL((moe_sum_kernel<4, true>), dim3((H / 4 + 255) / 256, T), dim3(256), 0, s, experts, weights, shared, gate, T, H, topk, out);
 }
 // Stand-in glue between stacked layers: x_next = bf(y * (1 / max|y|)) per token.
 __global__ __launch_bounds__(256) void stack_glue_kernel(const float* y, uint32_t H, float* out) {

@@ -46,6 +46,8 @@ void launch_hc_add(hipStream_t s, const float* hyper, const float* x, const floa
 void launch_norm(hipStream_t s, const float* x, const void* w, uint32_t dtype, uint32_t D, uint32_t width, uint32_t tokens, float* out);
 void launch_moe_sum(hipStream_t s, const float* experts, const float* weights, const float* shared, const float* gate,
                     uint32_t T, uint32_t H, uint32_t topk, float* out);
+void launch_moe_sum_half(hipStream_t s, const uint16_t* experts, const float* weights, const float* shared, const float* gate,
+                         uint32_t T, uint32_t H, uint32_t topk, float* out);
 void launch_stack_glue(hipStream_t s, const float* y, uint32_t T, uint32_t H, float* out);
 void launch_synth_words(hipStream_t s, uint32_t* dst, uint64_t count, uint64_t seed);
 void launch_synth_scales(hipStream_t s, uint16_t* sc, uint16_t* bi, uint64_t count, uint64_t seed, float lo, float span, float factor);
@@ -126,6 +128,7 @@ struct PrefillGemm {
     uint32_t bits;            // 4: nibble codes, asum = the Q4 lanes' BF16-rounded sum-of-four chains; 8: byte codes, asum = the Q8 lanes' plain sums
     uint16_t* out_b;          // gate/up: SwiGLU activations as bf16 [sorted position][N]
     float* out_f;             // down: BF16-rounded fp32 [output row][N]
+    uint16_t* out_h;          // down, instead of out_f when not null: the same values as bf16 (what the combine reads is half as long)
     // Sums that land within near_margin * (sum of term magnitudes) of a BF16 rounding boundary are marked in a bit map
     // (bit sorted position * N + row; near_words 32-bit words, all written by the product kernel)
     // and recomputed afterwards with the reference's exact lane arithmetic (launch_prefill_patch).
@@ -146,6 +149,9 @@ void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t 
 void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, const void* w, const float* offsets, uint32_t T, uint32_t K,
                            uint32_t E, uint32_t topk, float* norms, float* logits);
 void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16, bool plain);
+void launch_prefill_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets, int32_t* slots, int32_t* rows,
+                             int32_t* status, int32_t* tile_expert, int32_t* tile_first, int32_t* tile_rows, int32_t* tile_count);
+bool prefill_dispatch_fits(const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E);
 void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t experts, uint32_t rows, int32_t* tile_expert, int32_t* tile_first,
                           int32_t* tile_rows, int32_t* tile_count);
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles);

@@ -124,6 +124,123 @@ __global__ __launch_bounds__(1024) void prefill_tiles_kernel(const int32_t* offs
     if (e == 1023) *tile_count = scan[1023];
 }
 
+// The dispatch sort of a long batch and the routed experts' work list in ONE launch (the decode path's three dispatch
+// kernels and prefill_tiles_kernel hold the same steps as four launches in a row, each of them short: what they cost was
+// the four launches).  A workgroup = four experts (one per wave) x one of kDispatchParts stretches of the slots.  Every
+// workgroup counts ALL the slots' experts, per stretch, into a table in LDS and keeps its own stretch of the ids there;
+// it scans the table (sorted offsets and tile counts of every expert), and each wave then places its expert's slots of
+// the workgroup's stretch in ascending slot order, starting where the earlier stretches' slots of that expert end.  The
+// workgroups of the first stretch also write their experts' tiles, workgroup (0, 0) the offsets.  Same results as
+// launch_dispatch followed by launch_prefill_tiles; the list of selected experts is not written (nothing here reads it).
+// ids sixteen-byte aligned; stretch: slots per stretch, a multiple of 1024.
+constexpr uint32_t kDispatchParts = 4;
+__global__ __launch_bounds__(256) void prefill_dispatch_kernel(const int32_t* __restrict__ ids, uint32_t n, uint32_t topk, uint32_t E, uint32_t stretch,
+                                                               int32_t* __restrict__ offsets, int32_t* __restrict__ slots, int32_t* __restrict__ rows, int32_t* status,
+                                                               int32_t* tile_expert, int32_t* tile_first, int32_t* tile_rows, int32_t* tile_count) {
+    extern __shared__ __align__(16) int32_t table[];   // [parts][E] counts, [E + 1] offsets, [E + 1] tiles before, then the stretch's ids
+    __shared__ int32_t wave_sum[2][4];
+    int32_t* cnt = table; int32_t* off = table + kDispatchParts * E; int32_t* tiles_before = off + E + 1;
+    int32_t* copy = table + ((kDispatchParts + 2) * E + 2 + 3) / 4 * 4;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, part = blockIdx.y, first = part * stretch;
+    for (uint32_t i = tid; i < kDispatchParts * E; i += 256) cnt[i] = 0;
+    __syncthreads();
+    {
+        int bad = 0;
+        uint32_t at = 0, until = stretch;   // the stretch of slot p: counted up as p goes
+        for (uint32_t b0 = 0; b0 < n; b0 += 8 * 1024) {   // eight steps' loads in flight
+            int4 batch[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t p = b0 + u * 1024 + 4 * tid;
+                int4 v = make_int4(-1, -1, -1, -1);   // (-1: past the end)
+                if (p + 3 < n) v = *reinterpret_cast<const int4*>(ids + p);
+                else { if (p < n) v.x = ids[p]; if (p + 1 < n) v.y = ids[p + 1]; if (p + 2 < n) v.z = ids[p + 2]; }
+                batch[u] = v;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t p0 = b0 + u * 1024, p = p0 + 4 * tid;
+                if (p0 >= n) break;
+                if (p0 >= until) { ++at; until += stretch; }
+                const int32_t four[4] = {batch[u].x, batch[u].y, batch[u].z, batch[u].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (p + j >= n) continue;
+                    if (four[j] < 0 || four[j] >= int32_t(E)) bad = 1; else atomicAdd(&cnt[at * E + uint32_t(four[j])], 1);
+                }
+                if (at == part) *reinterpret_cast<int4*>(copy + (p - first)) = batch[u];
+            }
+        }
+        if (bad && blockIdx.x == 0 && part == 0) atomicOr(status, 1);
+    }
+    __syncthreads();
+    auto count_of = [&](uint32_t e) { int32_t c = 0; for (uint32_t q = 0; q < kDispatchParts; ++q) c += cnt[q * E + e]; return c; };
+    {   // exclusive scans over the experts: thread t owns experts t * per .. t * per + per - 1
+        const uint32_t per = (E + 255) / 256;
+        auto tiles_of = [](int32_t count) {
+            const int32_t whole = count / int32_t(kTileRows), left = count % int32_t(kTileRows);
+            return count == 0 ? 0 : (whole == 0 ? 1 : whole + (left > int32_t(kTileRowsMax - kTileRows) ? 1 : 0));
+        };
+        int32_t mine[2] = {0, 0};
+        for (uint32_t i = 0; i < per; ++i) { const uint32_t e = tid * per + i; if (e < E) { const int32_t c = count_of(e); mine[0] += c; mine[1] += tiles_of(c); } }
+        int32_t incl[2] = {mine[0], mine[1]};
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1)
+#pragma unroll
+            for (int v = 0; v < 2; ++v) { const int32_t up = __shfl_up(incl[v], o); if (int(lane) >= o) incl[v] += up; }
+        if (lane == 63) { wave_sum[0][wave] = incl[0]; wave_sum[1][wave] = incl[1]; }
+        __syncthreads();
+        int32_t at[2];
+#pragma unroll
+        for (int v = 0; v < 2; ++v) { at[v] = incl[v] - mine[v]; for (uint32_t w = 0; w < wave; ++w) at[v] += wave_sum[v][w]; }
+        for (uint32_t i = 0; i < per; ++i) {
+            const uint32_t e = tid * per + i;
+            if (e < E) { const int32_t c = count_of(e); off[e] = at[0]; tiles_before[e] = at[1]; at[0] += c; at[1] += tiles_of(c); }
+        }
+        if (tid == 255) { off[E] = at[0]; tiles_before[E] = at[1]; }
+        __syncthreads();
+    }
+    if (blockIdx.x == 0 && part == 0) {
+        for (uint32_t e = tid; e <= E; e += 256) offsets[e] = off[e];
+        if (tid == 0) *tile_count = tiles_before[E];
+    }
+    const uint32_t e = blockIdx.x * 4 + wave;
+    if (e >= E) return;
+    const int32_t count = count_of(e);
+    if (count == 0) return;
+    if (part == 0) {   // the expert's tiles: whole tiles of 32 rows, the last one takes what is left (at most 48)
+        const int32_t tiles = tiles_before[e + 1] - tiles_before[e], begin = tiles_before[e];
+        for (int32_t t = int32_t(lane); t < tiles; t += 64) {
+            tile_expert[begin + t] = int32_t(e); tile_first[begin + t] = off[e] + t * int32_t(kTileRows);
+            tile_rows[begin + t] = t + 1 < tiles ? int32_t(kTileRows) : count - t * int32_t(kTileRows);
+        }
+    }
+    int32_t pos = off[e];
+    for (uint32_t q = 0; q < part; ++q) pos += cnt[q * E + e];
+    const int32_t end = pos + cnt[part * E + e];
+    const uint64_t below = (1ull << lane) - 1;
+    const float inverse = 1.0f / float(topk);
+    // 256 slots per step, in order: four neighbouring slots per lane, slots of lower lanes first, then the lane's own
+    for (uint32_t q0 = first; q0 < n && q0 < first + stretch && pos < end; q0 += 256) {
+        const uint32_t p = q0 + 4 * lane;
+        const int4 v = *reinterpret_cast<const int4*>(copy + (p - first));
+        const bool m[4] = {v.x == int32_t(e), v.y == int32_t(e), v.z == int32_t(e), v.w == int32_t(e)};
+        const uint64_t mask[4] = {__ballot(m[0]), __ballot(m[1]), __ballot(m[2]), __ballot(m[3])};
+        if ((mask[0] | mask[1] | mask[2] | mask[3]) == 0) continue;   // uniform: none of these 256 slots is the expert's
+        int32_t at = pos + __popcll(mask[0] & below) + __popcll(mask[1] & below) + __popcll(mask[2] & below) + __popcll(mask[3] & below);
+        // token and rank of slot p (p < 2^24: the rounded quotient is off by one at most)
+        uint32_t token = uint32_t(float(p) * inverse);
+        int32_t rest = int32_t(p) - int32_t(token * topk);
+        if (rest < 0) { --token; rest += int32_t(topk); } else if (rest >= int32_t(topk)) { ++token; rest -= int32_t(topk); }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (m[j]) { slots[at] = int32_t(p + j); if (rows) rows[at] = int32_t(token); ++at; }
+            if (++rest == int32_t(topk)) { rest = 0; ++token; }
+        }
+        pos += __popcll(mask[0]) + __popcll(mask[1]) + __popcll(mask[2]) + __popcll(mask[3]);
+    }
+}
+
 // BITS: 4 (nibble codes, eight bytes of a row per lane and step) or 8 (byte codes, sixteen bytes; the chain sums are then
 // the plain ones of the Q8 lanes).  A byte code is exact in bf16 like a nibble code, and its product with a BF16 value is
 // exact in fp32.
@@ -357,7 +474,10 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(PrefillGemm p) {
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
                     const uint32_t n = n0 + (2 * wave + uint32_t(q)) * 16 + j;
-                    if (live) p.out_f[uint64_t(out_row) * N + n] = bf(total[rb][q][r]);
+                    if (live) {
+                        if (p.out_h) p.out_h[uint64_t(out_row) * N + n] = uint16_t(__float_as_uint(bf(total[rb][q][r])) >> 16);
+                        else p.out_f[uint64_t(out_row) * N + n] = bf(total[rb][q][r]);
+                    }
                     const uint64_t marks = __ballot(near_boundary(total[rb][q][r], mag[rb][q][r]));
                     if (live && j == 0) bits[(uint64_t(pos) * N + n) / 16] = uint16_t(marks >> (16 * g4));
                 }
@@ -478,7 +598,10 @@ __global__ __launch_bounds__(256) void prefill_patch_kernel(PrefillGemm p, uint3
     if constexpr (GATED) result[1] = lane_sum32(result[1]);
     if (lane == 0) {
         if constexpr (GATED) p.out_b[uint64_t(pos) * N + n] = uint16_t(__float_as_uint(swiglu_bf(result[0], result[1])) >> 16);
-        else p.out_f[uint64_t(p.out_rows ? uint32_t(p.out_rows[pos]) : pos) * N + n] = bf(result[0]);
+        else {
+            const uint64_t at = uint64_t(p.out_rows ? uint32_t(p.out_rows[pos]) : pos) * N + n;
+            if (p.out_h) p.out_h[at] = uint16_t(__float_as_uint(bf(result[0])) >> 16); else p.out_f[at] = bf(result[0]);
+        }
     }
   }
 }
@@ -692,6 +815,19 @@ void launch_prefill_tiles(hipStream_t s, const int32_t* offsets, uint32_t expert
 }
 // LDS beyond the kernel's fixed arrays: the scales and biases of 128 weight rows and the chain sums of 48 token rows for
 // every step of K.
+void launch_prefill_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets, int32_t* slots, int32_t* rows,
+                             int32_t* status, int32_t* tile_expert, int32_t* tile_first, int32_t* tile_rows, int32_t* tile_count) {
+    const uint32_t n = tokens * topk, stretch = ((n + kDispatchParts - 1) / kDispatchParts + 1023) / 1024 * 1024;
+    const size_t lds = size_t(((kDispatchParts + 2) * E + 2 + 3) / 4 * 4 + stretch) * 4;
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_dispatch_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    hipLaunchKernelGGL(prefill_dispatch_kernel, dim3((E + 3) / 4, kDispatchParts), dim3(256), lds, s, ids, n, topk, E, stretch, offsets, slots, rows, status,
+                       tile_expert, tile_first, tile_rows, tile_count);
+}
+// whether launch_prefill_dispatch takes this batch (else: launch_dispatch and launch_prefill_tiles)
+bool prefill_dispatch_fits(const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E) {
+    const uint64_t n = uint64_t(tokens) * topk;
+    return reinterpret_cast<uintptr_t>(ids) % 16 == 0 && n > 1024 && n < (1u << 24) && E <= 1024 && n / kDispatchParts + 1024 <= 24 * 1024;
+}
 static uint32_t prefill_gemm_lds(uint32_t K) { const uint32_t groups = K / 64; return 2 * kTileCols * (groups + 2) * 2 + groups * kTileRowsMax * 4; }
 void launch_prefill_gemm(hipStream_t s, const PrefillGemm& p, bool gated, uint32_t max_tiles) {
     const dim3 grid(gated ? p.N / 64 : p.N / 128, max_tiles);

@@ -109,24 +109,32 @@ __global__ __launch_bounds__(kMultiThreads) void decode_multi_kernel(DecodeParam
         const bool ahead = H / 128 <= uint32_t(kPieces);
         {
             const bool glue = layer != 0;
-            // the glue's scale per token: 1 / max|y| of the previous layer
-            if (glue) {   // the largest magnitude of every row: the combine left one candidate per 64 columns
-                const uint32_t groups = H / 64;
-                uint32_t m = 0;
-                for (uint32_t g = lane; g < groups; g += 64) if (wave < T) m = max(m, ZC_LD(p.maxabs + wave * groups + g));
-                m = __float_as_uint(wave_max_f32(__uint_as_float(m)));
-                if (wave < T && lane == 0) {
-                    const float v = __uint_as_float(m);
-                    gatev[wave] = (v > 0.0f && v < __uint_as_float(0x7f800000u)) ? 1.0f / v : 1.0f;
+            // Everything the staging needs is requested in one go -- the input rows, then the candidates of the glue's scale
+            // per token (1 / max|y| of the previous layer: the combine left one candidate per 64 columns) and the shared gate's
+            // weights -- so that the three fetches cost one trip to the L2, not three in a row.
+            auto ready = [&]() {
+                uint4 gw[2];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) { const uint32_t i = tid + q * kMultiThreads; gw[q] = i < H / 8 ? ldg_u4(L.shared_gate, i) : make_uint4(0, 0, 0, 0); }
+                if (glue) {
+                    const uint32_t groups = H / 64;
+                    uint32_t m = 0;
+                    for (uint32_t g = lane; g < groups; g += 64) if (wave < T) m = max(m, ZC_LD(p.maxabs + wave * groups + g));
+                    m = __float_as_uint(wave_max_f32(__uint_as_float(m)));
+                    if (wave < T && lane == 0) {
+                        const float v = __uint_as_float(m);
+                        gatev[wave] = (v > 0.0f && v < __uint_as_float(0x7f800000u)) ? 1.0f / v : 1.0f;
+                    }
                 }
-            }
-            __syncthreads();
-            const int bad = stage_bf16<24>(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), []() {},
+#pragma unroll
+                for (int q = 0; q < 2; ++q) { const uint32_t i = tid + q * kMultiThreads; if (i < H / 8) reinterpret_cast<uint4*>(lds + lp.gatew)[i] = gw[q]; }
+                __syncthreads();
+            };
+            const int bad = stage_bf16<24>(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh), ready,
                 [&](uint32_t i, float& a, float& b) {
                     if (glue) { const float scale = gatev[(2 * i) / H]; a = bf(a * scale); b = bf(b * scale); }
                 });
             if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
-            for (uint32_t i = tid; i < H / 8; i += kMultiThreads) reinterpret_cast<uint4*>(lds + lp.gatew)[i] = ldg_u4(L.shared_gate, i);
         }
         xint_prepare_begin(LH, lds + lp.img_x, T);
         __syncthreads();

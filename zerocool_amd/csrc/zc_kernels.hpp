@@ -140,11 +140,11 @@ struct PrefillGemm {
     const int32_t* covered; uint32_t experts;
 };
 // Margin of the recomputation, as a fraction of the summed term magnitudes (those of the scale groups' sums: what cancels
-// inside a group is not seen).  Rows of fewer than 32 groups keep 2^-22, four fp32 steps: with few groups the additions
-// inside a group weigh most, and a flip was seen at two groups with half of that.  From 32 groups on the margin is 2^-28 per
-// group (2^-23 at 32 groups, where the largest distance seen between the two orders of additions is a quarter of it; 2^-22
-// again at 64): the distance grows with the number of additions.
-constexpr float prefill_margin(uint32_t K) { return K / 64 < 32 ? 0x1p-22f : float(K / 64) * 0x1p-28f; }
+// inside a group is not seen).  Rows of fewer than 8 groups keep 2^-22, four fp32 steps: with few groups the additions
+// inside a group weigh most, and a flip was seen at two groups with half of that.  From 8 to 32 groups the margin is
+// 2^-23 (the largest distance seen between the two orders of additions, on rows of 8 and of 32 groups, is a quarter of it),
+// beyond that 2^-28 per group (2^-22 again at 64): the distance grows with the number of additions.
+constexpr float prefill_margin(uint32_t K) { return K / 64 < 8 ? 0x1p-22f : (K / 64 <= 32 ? 0x1p-23f : float(K / 64) * 0x1p-28f); }
 void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, float* plain, int32_t* status);
 void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, const void* w, const float* offsets, uint32_t T, uint32_t K,
                            uint32_t E, uint32_t topk, float* norms, float* logits);

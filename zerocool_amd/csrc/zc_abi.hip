@@ -729,9 +729,14 @@ zc_status zc_hip_moe_prefill(zc_hip_ctx* ctx, const zc_moe_config* c, const zc_m
     }
     hipStream_t s2 = ctx->beside;
     ZC_HIP(hipEventRecord(ctx->fork, s)); ZC_HIP(hipStreamWaitEvent(s2, ctx->fork, 0));
-    if (T >= 128 && !(trace && trace->logits)) zc::launch_prefill_router(s, x, w.xb, l->router, l->router_offsets, T, H, E, k, w.norms, w.base.logits);
-    else zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
-    zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
+    if (T >= 128 && !(trace && trace->logits)) {
+        const bool select = k <= 64;   // the refinement's wavefront selects its token's experts too
+        zc::launch_prefill_router(s, x, w.xb, l->router, l->router_offsets, T, H, E, k, w.norms, w.base.logits, select ? w.base.ids : nullptr, select ? w.base.weights : nullptr);
+        if (!select) zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
+    } else {
+        zc::launch_router(s, l->router, x, T, H, E, l->router_offsets, w.base.logits);
+        zc::launch_route(s, w.base.logits, T, E, k, w.base.ids, w.base.weights);
+    }
     // dispatch sort and the routed experts' tile list: one launch for a long batch
     const bool one_dispatch = zc::prefill_dispatch_fits(w.base.ids, T, k, E);
     if (one_dispatch) zc::launch_prefill_dispatch(s, w.base.ids, T, k, E, w.base.offsets, w.base.slots, w.base.rows, ctx->moe_status, w.tile_expert, w.tile_first, w.tile_rows, w.tile_count);

@@ -146,8 +146,9 @@ struct PrefillGemm {
 // beyond that 2^-28 per group (2^-22 again at 64): the distance grows with the number of additions.
 constexpr float prefill_margin(uint32_t K) { return K / 64 < 8 ? 0x1p-22f : (K / 64 <= 32 ? 0x1p-23f : float(K / 64) * 0x1p-28f); }
 void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, float* plain, int32_t* status);
+// ids / weights not null (topk <= 64): the selection runs in the same launch and the logits are not written
 void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, const void* w, const float* offsets, uint32_t T, uint32_t K,
-                           uint32_t E, uint32_t topk, float* norms, float* logits);
+                           uint32_t E, uint32_t topk, float* norms, float* logits, int32_t* ids, float* weights);
 void launch_prefill_sums(hipStream_t s, const uint16_t* xb, const int32_t* rows_ptr, uint32_t rows_max, uint32_t K, float* sums, float* sums16, bool plain);
 void launch_prefill_dispatch(hipStream_t s, const int32_t* ids, uint32_t tokens, uint32_t topk, uint32_t E, int32_t* offsets, int32_t* slots, int32_t* rows,
                              int32_t* status, int32_t* tile_expert, int32_t* tile_first, int32_t* tile_rows, int32_t* tile_count);

@@ -23,6 +23,7 @@
 // forty rows per expert -- an unskewed router at 2048 tokens -- every expert's codes are then expanded once, not twice.
 #include "zc_kernels.hpp"
 #include "zc_device.hpp"
+#include "zc_decode_common.hpp"   // route_token: top-k + softmax of one token by one wavefront
 
 namespace zc {
 
@@ -692,11 +693,17 @@ __global__ __launch_bounds__(256) void router_product_kernel(const uint16_t* a, 
 }
 // One wavefront per token: bounds, the experts that can be among the top k, their exact logits; everything else -inf.
 // (A whole workgroup per token, each wavefront taking a quarter of the list, measured slower: 35 against 29 us.)
+// ids / weights not null (topk <= 64): the wavefront also selects its token's top k and forms the softmax weights from the
+// row it holds in LDS (route_token, the selection of the decode kernels: the same ids and weights as route_kernel's), and
+// the row itself is not written out.
 constexpr int kRefinePerLane = 16;   // experts <= 1024
 __global__ __launch_bounds__(256) void router_refine_kernel(const uint16_t* xb, const uint16_t* w, const float* offsets, const float* norms,
-                                                            uint32_t T, uint32_t E, uint32_t K, uint32_t topk, float* logits) {
+                                                            uint32_t T, uint32_t E, uint32_t K, uint32_t topk, float* logits,
+                                                            int32_t* ids, float* weights) {
     __shared__ float row_s[4][1024];
     __shared__ uint16_t list_s[4][1024];
+    __shared__ uint32_t pick_s[4][128];                      // route_token's scratch
+    __shared__ int32_t ids_s[4][64]; __shared__ float weights_s[4][64];
     extern __shared__ __align__(16) uint16_t x_s[];   // the four tokens' input rows (BF16-valued, so the bf16 copy is the input)
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x & 63u, t = blockIdx.x * 4 + wave;
     if (t >= T) return;
@@ -789,16 +796,30 @@ __global__ __launch_bounds__(256) void router_refine_kernel(const uint16_t* xb, 
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    for (uint32_t e = lane; e < E; e += 64) row[e] = row_s[wave][e];
+    if (!ids) { for (uint32_t e = lane; e < E; e += 64) row[e] = row_s[wave][e]; return; }
+    auto fetch = [&](auto& cand, uint32_t per) {
+        constexpr int PER = int(sizeof(cand) / sizeof(float));
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const uint32_t e = lane * per + uint32_t(i);
+            cand[i] = (uint32_t(i) < per && e < E) ? row_s[wave][e] : ninf;
+        }
+    };
+    if (E == 512) route_token<8>(fetch, E, topk, lane, ids_s[wave], weights_s[wave], pick_s[wave], []() {}, []() {});
+    else route_token<16>(fetch, E, topk, lane, ids_s[wave], weights_s[wave], pick_s[wave], []() {}, []() {});
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (lane < topk) { ids[uint64_t(t) * topk + lane] = ids_s[wave][lane]; weights[uint64_t(t) * topk + lane] = weights_s[wave][lane]; }
 }
 // Router logits for the selection that follows: exact where it can matter, -inf elsewhere.  xb: the inputs as bf16 rows;
 // norms: rows + experts floats of scratch.  K % 128 == 0, experts <= 1024.
 void launch_prefill_router(hipStream_t s, const float* x, const uint16_t* xb, const void* w, const float* offsets, uint32_t T, uint32_t K,
-                           uint32_t E, uint32_t topk, float* norms, float* logits) {
+                           uint32_t E, uint32_t topk, float* norms, float* logits, int32_t* ids, float* weights) {
     const uint16_t* wb = static_cast<const uint16_t*>(w);
     hipLaunchKernelGGL(row_norms_kernel, dim3((T + E + 3) / 4), dim3(256), 0, s, xb, T, wb, E, K, norms);
     hipLaunchKernelGGL(router_product_kernel, dim3((E + 63) / 64, (T + 63) / 64), dim3(256), 0, s, xb, wb, T, E, K, offsets, logits);
-    hipLaunchKernelGGL(router_refine_kernel, dim3((T + 3) / 4), dim3(256), 4 * K * 2, s, xb, wb, offsets, norms, T, E, K, topk, logits);
+    hipLaunchKernelGGL(router_refine_kernel, dim3((T + 3) / 4), dim3(256), 4 * K * 2, s, xb, wb, offsets, norms, T, E, K, topk, logits, ids, weights);
 }
 
 void launch_prefill_rows(hipStream_t s, const float* x, uint32_t rows, uint32_t K, uint16_t* xb, float* sums, float* sums16, float* plain, int32_t* status) {

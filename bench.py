@@ -76,7 +76,7 @@ def write_traffic_file(fetch_dir, write_dir):
     write, write_copy, _ = averages(write_dir, "WRITE_SIZE")
     read_bytes = fetch * (1048576.0 / fetch_copy) * 1024
     written_bytes = write * (1048576.0 / write_copy) * 1024
-    record = {"kernel": "zc::decode_stack_kernel<1, false>", "workload": "48 F-shape layers, batch 1 (the default run of bench.py)",
+    record = {"kernel": "zc::decode_stack_kernel<false>", "workload": "48 F-shape layers, batch 1 (the default run of bench.py)",
               "dispatches_averaged": calls, "FETCH_SIZE_KiB": fetch, "FETCH_SIZE_KiB_of_1GiB_copy": fetch_copy,
               "WRITE_SIZE_KiB": write, "WRITE_SIZE_KiB_of_1GiB_copy": write_copy,
               "hbm_bytes_read": int(read_bytes), "hbm_bytes_written": int(written_bytes),

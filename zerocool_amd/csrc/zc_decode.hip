@@ -1,4 +1,5 @@
-// Persistent decode kernel: a whole stack of MoE layers for a few tokens in ONE launch.
+// Persistent decode kernel for ONE token: a whole stack of MoE layers in ONE launch (two to eight tokens:
+// zc_decode_multi.hip; nine to sixty-four: zc_decode_wide.hip).
 //
 // One workgroup per compute unit stays resident for all layers.  A layer is three phases:
 //   R  router logits (16-split chains), shared-expert gate dot
@@ -13,8 +14,7 @@
 // memory; no cache write-back or invalidate is needed, only wait counters.
 // Weights are read with ordinary cached loads: nothing writes them.
 //
-// Several tokens (NT = 8) separate the phases with grid barriers (Barrier::wait).  One token (NT = 1) has none on its
-// path: every exchanged value carries a tag (a 16-bit number that advances with every layer of every launch) and its
+// There is no grid barrier on the path: every exchanged value carries a tag (a 16-bit number that advances with every layer of every launch) and its
 // reader polls the data itself until the tag is the expected one (Barrier::until); one flag per workgroup and layer,
 // stored without waiting and checked a layer later (Barrier::arrive), keeps a buffer from being overwritten before
 // every workgroup has read it.  Inside a workgroup, waves hand work on through flag words in LDS where a workgroup
@@ -28,16 +28,14 @@ namespace zc {
 
 constexpr int kRing = 8;         // sixteen-byte pieces of a router partition in flight per lane; tiles keep eight 128-element spans
                                  // in flight with one wave per SIMD and four with two
-#define ZC_RUN_TILE(SPANS, ...) do { if (NT != 1 && (SPANS) % 8 == 0) xint_run_tile<PT, 8>(__VA_ARGS__); else xint_run_tile<PT, 4>(__VA_ARGS__); } while (0)
 
-// NT = 1: single-token decode.  NT = 8: up to eight tokens, tiles take four at a time.
 // MIXED: the down projection and/or the shared expert are affine Q8 and run on literal lanes; that variant leaves out the
 // wave-local down phase (whose tile engine is the largest single piece of the kernel), so that both variants fit the
 // register file without scratch memory and the all-Q4 variant is exactly what it was.
-template <int NT, bool MIXED>
-__global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
-    constexpr int PT = NT < 4 ? NT : 4;   // tokens per tile pass
-    constexpr uint32_t kDecodeThreads = decode_threads(NT), kDecodeWaves = kDecodeThreads / 64;
+template <bool MIXED>
+__global__ __launch_bounds__(decode_threads(1)) void decode_stack_kernel(DecodeParams p, DecodeLdsPlan lp) {
+    constexpr int PT = 1;   // tokens per tile pass
+    constexpr uint32_t kDecodeThreads = decode_threads(1), kDecodeWaves = kDecodeThreads / 64;
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, col = lane & 15u, G = lane >> 4;
     const uint32_t wg = blockIdx.x, nwg = gridDim.x;
@@ -45,10 +43,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
     int32_t* ids = reinterpret_cast<int32_t*>(lds + lp.ids);
     float* weights = reinterpret_cast<float*>(lds + lp.weights);
     float* gatev = reinterpret_cast<float*>(lds + lp.gatev);
-    int32_t* head = reinterpret_cast<int32_t*>(lds + lp.head);
-    int32_t* next = reinterpret_cast<int32_t*>(lds + lp.next);
     int32_t* experts = reinterpret_cast<int32_t*>(lds + lp.experts);
-    int32_t* misc = reinterpret_cast<int32_t*>(lds + lp.misc);   // [0] U, [1..8] wave counts
+    int32_t* misc = reinterpret_cast<int32_t*>(lds + lp.misc);   // [1..8] wave maxima, [10..14] hand-off and ready words
     const uint16_t* xh_all = reinterpret_cast<const uint16_t*>(lds + lp.xh);
     const XintLayout LH{H}, LI{I};
     Barrier bar{p.sync, p.epoch, p.spin_limit, p.status, p.epoch};
@@ -60,16 +56,6 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
 
     if (wg == 0) for (uint32_t i = tid; i < p.L * T; i += blockDim.x) ZC_ST(p.maxabs + i, 0u);
     if (tid == 0) { misc[10] = 0; misc[11] = 0; misc[12] = 0; misc[13] = 0; misc[14] = 0; }   // the router chain's hand-off word, the ids-ready word, the staging waves' image-ready words: no tag is 0
-    // SwiGLU of a finished gate/up tile (gate rows in columns 0-7, up rows in 8-15), stored as packed BF16 pairs:
-    // the lane of an even row writes rows r and r+1 of activation row `slot_row` as one word.
-    auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {
-        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
-        const uint32_t a = __float_as_uint(swiglu_bf(v, up));
-        const uint32_t other = uint32_t(__shfl_xor(int(a), 1));
-        if (lane < 8 && !(lane & 1u))
-            ZC_ST(reinterpret_cast<uint32_t*>(buffer) + (uint64_t(slot_row) * I + row) / 2, (a >> 16) | (other & 0xffff0000u));
-    };
-
     for (uint32_t layer = 0; layer < p.L; ++layer) {
         const DecodeLayer L = p.layers[layer];
         // Per-lane addresses and predicates derived from the thread index are recomputed in every layer: hoisted out of
@@ -86,7 +72,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         const uint32_t tag = tag_of(layer);
         auto st_logit = [&](uint32_t index, float v) { ZC_ST(p.tlogits + index, (uint64_t(tag) << 32) | __float_as_uint(v)); };
         // one token: the experts this layer picked at the previous step (null: no guess), and where every slot's activations are
-        const int32_t* pred = (NT == 1 && p.pred_in) ? p.pred_in + uint64_t(layer) * k : nullptr;
+        const int32_t* pred = p.pred_in ? p.pred_in + uint64_t(layer) * k : nullptr;
         int32_t* spec = reinterpret_cast<int32_t*>(lds + lp.spec);   // [k + 1] source rows, [k + 1] miss list, [1] misses
         // ---------------- phase R: input images, router, shared gate/up, shared gate ----------------
         __syncthreads();
@@ -99,7 +85,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         // latency instead of one per ring.  The shared gate dot goes to the next workgroup, all of whose threads form the
         // products before one half-wave adds them in the reference's order.
         const uint32_t router_pieces = H / 128, router_segments = router_pieces / kRing;
-        const bool segmented = NT == 1 && router_pieces % kRing == 0 && router_segments <= kDecodeWaves && (E + 3) / 4 < nwg;
+        const bool segmented = router_pieces % kRing == 0 && router_segments <= kDecodeWaves && (E + 3) / 4 < nwg;
         uint4 early[kRing];
 #pragma unroll
         for (int i = 0; i < kRing; ++i) early[i] = make_uint4(0, 0, 0, 0);
@@ -107,9 +93,9 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         // router's (the staging waves and the ones behind them), which start them as soon as the image is complete -- told
         // so through flag words in LDS, not by a workgroup barrier, for which the router's waves would have to finish their
         // chains first (a tile is then 2.6 us late, and the layer with it: the gate/up burst is what the routing waits for).
-        const bool apart = NT == 1 && !MIXED && pred != nullptr && segmented && wg < (E + 3) / 4 && 64 * router_segments + H / 16 <= kDecodeThreads &&
+        const bool apart = !MIXED && pred != nullptr && segmented && wg < (E + 3) / 4 && 64 * router_segments + H / 16 <= kDecodeThreads &&
                            (k * (I / 8)) % nwg == 0 && (E + 3) / 4 + I / 8 <= nwg && kDecodeWaves - router_segments >= k * (I / 8) / nwg && (H / 16 + 63) / 64 <= 3;
-        if constexpr (NT == 1) {
+        {
             // One token: thread b fetches the sixteen values of block b, applies the glue's scale, writes the BF16 copy and
             // builds the block's image pieces straight from registers; the shared gate row rides along.  After the first
             // layer the values are the previous layer's tagged words: the thread fetches them again until every tag is that
@@ -240,57 +226,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                 if (lane == 0) __hip_atomic_store(misc + 12 + (wave - router_segments), int32_t(tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
-        } else {
-            {
-                uint16_t* xh = reinterpret_cast<uint16_t*>(lds + lp.xh);
-                const bool glue = layer != 0;
-                // the glue's scale per token, 1 / max|y| of the previous layer: one token fetches it together with the row,
-                // several tokens go through LDS (one more round trip, fewer registers)
-                uint32_t peak = 0; float inv = 1.0f;
-                if constexpr (NT == 1) {
-                    if (glue) peak = ZC_LD(p.maxabs + (layer - 1) * T);
-                } else {
-                    if (glue && tid < T) {
-                        const float m = __uint_as_float(ZC_LD(p.maxabs + (layer - 1) * T + tid));
-                        gatev[tid] = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
-                    }
-                    __syncthreads();
-                }
-                // the shared-expert gate row rides along: coalesced sixteen-byte loads, used from LDS by the gate-dot waves
-                constexpr int kGatePieces = (3072 / 8 + kDecodeThreads - 1) / kDecodeThreads;   // hidden <= 3072
-                uint4 gate_piece[kGatePieces];
-#pragma unroll
-                for (int q = 0; q < kGatePieces; ++q) gate_piece[q] = make_uint4(0, 0, 0, 0);
-                const int bad = stage_bf16(glue ? p.layer_out : p.x_in, T * H / 2, reinterpret_cast<uint32_t*>(xh),
-                    [&]() {
-                        if constexpr (NT == 1) {
-#pragma unroll
-                            for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);
-                            const float m = __uint_as_float(peak); inv = (m > 0.0f && m < __uint_as_float(0x7f800000u)) ? 1.0f / m : 1.0f;
-                        }
-                    },
-                    [&](uint32_t i, float& a, float& b) {
-                        if (glue) {
-                            const float scale = NT == 1 ? inv : gatev[(2 * i) / H];
-                            a = bf(a * scale); b = bf(b * scale);
-                        }
-                    });
-                if (bad) atomicOr(p.status, 4);   // inputs must be BF16-valued
-#pragma unroll
-                for (int q = 0; q < kGatePieces; ++q) if (tid + q * kDecodeThreads < H / 8) {
-                    if constexpr (NT != 1) gate_piece[q] = ldg_u4(L.shared_gate, tid + q * kDecodeThreads);   // several tokens: after the rows, to spare registers
-                    reinterpret_cast<uint4*>(lds + lp.gatew)[tid + q * kDecodeThreads] = gate_piece[q];
-                }
-            }
-            __syncthreads();
-            xint_prepare_batch([&](uint32_t q) { return LdsBf16{xh_all + q * H}; }, T, LH, lds + lp.img_rg);
         }
         clock(1);
         {
             // One token: the shared gate/up tiles run in phase G beside the routed ones, on waves that have no routed tile;
             // this phase then only has the router.
-            const uint32_t router_units = (E + 3) / 4, shared_units = NT == 1 ? 0 : I / 8, gate_units = (T + 1) / 2;
-            const uint32_t units = router_units + shared_units + gate_units;
+            const uint32_t router_units = (E + 3) / 4, gate_units = (T + 1) / 2;
+            const uint32_t units = router_units + gate_units;
             if (segmented) {
                 float* handoff = reinterpret_cast<float*>(lds + lp.gprod);   // 64 chain values; the products table belongs to another workgroup
                 if (wg < router_units) {
@@ -354,17 +296,15 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     constexpr int kRouterRing = kRing;
                     const uint32_t pieces = P / 8;   // sixteen-byte pieces of the partition, kRing in flight
                     uint4 wv[kRouterRing];
-                    if (NT == 1 && u == first_unit) {
+                    if (u == first_unit) {
 #pragma unroll
                         for (int i = 0; i < kRouterRing; ++i) wv[i] = early[i];
                     } else {
 #pragma unroll
                         for (int i = 0; i < kRouterRing; ++i) if (uint32_t(i) < pieces) wv[i] = ldg_u4(wr, i);
                     }
-                    float c[NT];
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) c[t] = 0;
-                    if (NT == 1 && pieces % kRouterRing == 0) {
+                    float c = 0;
+                    if (pieces % kRouterRing == 0) {
                         // one token, whole rings (hidden a multiple of 1024): straight-line bodies of eight pieces, the eight input
                         // pieces read from LDS together so that one wait covers them, the next ring requested before the chain runs
                         for (uint32_t i0 = 0; i0 < pieces; i0 += kRouterRing) {
@@ -380,8 +320,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                                 const uint32_t xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {wc[j].x, wc[j].y, wc[j].z, wc[j].w};
 #pragma unroll
                                 for (int q = 0; q < 4; ++q) {
-                                    c[0] = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c[0]);
-                                    c[0] = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c[0]);
+                                    c = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c);
+                                    c = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c);
                                 }
                             }
                         }
@@ -393,52 +333,25 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                             if (i < pieces) {
                                 const uint32_t ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
                                 if (i + kRouterRing < pieces) wv[j] = ldg_u4(wr, i + kRouterRing);
+                                const uint4 xv = *reinterpret_cast<const uint4*>(xh_all + split * P + i * 8);
+                                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
 #pragma unroll
-                                for (int t = 0; t < NT; ++t) {
-                                    if (t >= int(T)) break;
-                                    const uint4 xv = *reinterpret_cast<const uint4*>(xh_all + uint64_t(t) * H + split * P + i * 8);
-                                    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
-#pragma unroll
-                                    for (int q = 0; q < 4; ++q) {
-                                        c[t] = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c[t]);
-                                        c[t] = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c[t]);
-                                    }
+                                for (int q = 0; q < 4; ++q) {
+                                    c = __builtin_fmaf(__uint_as_float(xw[q] << 16), __uint_as_float(ww[q] << 16), c);
+                                    c = __builtin_fmaf(__uint_as_float(xw[q] & 0xffff0000u), __uint_as_float(ww[q] & 0xffff0000u), c);
                                 }
                             }
                         }
                     }
                     // partials added 0..15: after step s the lane of partition i <= s holds ((c0 + c1) + ..) + ci
                     const float offset = (L.offsets && e < E) ? ldg_f32(L.offsets, e) : 0.0f;
+                    float sum = 0.0f + c;
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        if (t >= int(T)) break;
-                        float sum = 0.0f + c[t];
-#pragma unroll
-                        for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c[t];
-                        if (split == 15 && e < E) {
-                            if constexpr (NT == 1) st_logit(e, L.offsets ? sum + offset : sum);
-                            else st_f32(p.logits + uint64_t(t) * E + e, L.offsets ? sum + offset : sum);
-                        }
-                    }
-                } else if (u < router_units + shared_units) {
-                    const uint32_t tile = u - router_units, row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                    const uint8_t* rec = L.shared_record;
-                    const uint8_t* w_row = rec + p.so[pr] + uint64_t(row) * (H / 2);
-                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 1]) + uint64_t(row) * (H / 64);
-                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.so[pr + 2]) + uint64_t(row) * (H / 64);
-                    for (uint32_t t0 = 0; t0 < T; t0 += PT) {
-                        const uint8_t* img[PT]; LdsBf16 src[PT];
-#pragma unroll
-                        for (int t = 0; t < PT; ++t) {
-                            const uint32_t tt = t0 + t < T ? t0 + t : 0;
-                            img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
-                        }
-                        auto emit = [&](int t, float v) { store_act(p.shared_act, t0 + t, row, v); };
-                        ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, int(min(uint32_t(PT), T - t0)), emit);
-                    }
+                    for (int step = 1; step < 16; ++step) sum = dpp_row_shr1(sum) + c;
+                    if (split == 15 && e < E) st_logit(e, L.offsets ? sum + offset : sum);
                 } else {
                     // shared_expert_gate: reference lane chain k = lane + 32 j (qwen.metal:499-506); two tokens per wave
-                    const uint32_t t = (u - router_units - shared_units) * 2 + (lane >> 5), l32 = lane & 31u;
+                    const uint32_t t = (u - router_units) * 2 + (lane >> 5), l32 = lane & 31u;
                     const uint16_t* gw = reinterpret_cast<const uint16_t*>(lds + lp.gatew);   // staged with the input rows
                     float sum = 0;
                     if (t < T)
@@ -450,9 +363,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                             for (int j = 0; j < 8; ++j) sum += a[j] * g[j];
                         }
                     sum = lane_sum32(sum);
-                    if (t < T && l32 == 0) {
-                        if constexpr (NT == 1) st_logit(E, bf(sum)); else st_f32(p.gate + t, bf(sum));
-                    }
+                    if (t < T && l32 == 0) st_logit(E, bf(sum));
                 }
             }
         }
@@ -470,7 +381,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             }
         } else {
             clock_all(2);
-            if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the routing below polls the logits themselves
+            __syncthreads();   // the routing below polls the logits themselves
         }
         refresh();
         clock(3);
@@ -479,13 +390,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
         {
             uint32_t route_stamp = 4; auto stamp = [&]() { if (t == 0) clock(route_stamp++); };
             // the previous step's ids of this layer, one per lane: requested now, compared when this step's ids are final
-            const int32_t guess = (NT == 1 && pred && lane < k) ? pred[lane] : -1;
-            uint32_t* scratch = reinterpret_cast<uint32_t*>(experts) + 128 * wave;   // the expert list is built later; 128 words per wave fit it for 512 experts
+            const int32_t guess = (pred && lane < k) ? pred[lane] : -1;
+            uint32_t* scratch = reinterpret_cast<uint32_t*>(experts) + 128 * wave;   // the selection's 128 words of scratch per wave
             // the lane's logits: written by other workgroups; one token polls the tagged words until all carry this layer's tag
             auto fetch = [&](auto& cand, uint32_t per) {
                 constexpr int PER = int(sizeof(cand) / sizeof(float));
                 const float ninf = __uint_as_float(0xff800000u);
-                if constexpr (NT == 1) {
+                {
                     // polled with the lanes side by side (word i * 64 + lane: four whole cache lines per load; lane-major, as
                     // the selection wants its candidates, a load touched thirty-two), turned lane-major through LDS
                     uint64_t w[PER];
@@ -512,18 +423,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
 #pragma unroll
                     for (int i = 0; i < PER; ++i) cand[i] = (uint32_t(i) < per && lane * per + i < E) ? turned[lane * per + i] : ninf;
                     wave_order();
-                } else {
-#pragma unroll
-                    for (int i = 0; i < PER; ++i) {
-                        const uint32_t e = lane * per + i;
-                        cand[i] = (uint32_t(i) < per && e < E) ? load_shared_f32(p.logits + uint64_t(t) * E + e) : ninf;
-                    }
                 }
             };
             // One token: the other waves wait for the ids only (a flag word in LDS), not for the softmax weights, which the
             // combine needs much later; the routing wave takes its tiles last.
             auto ready = [&]() {
-                if constexpr (NT == 1) {
+                {
                     // Where every slot's gate/up activations come from: the row of the prediction pass that already ran the same
                     // expert (slot j' of the predicted list), or this layer's own row once the tiles below have run (-1: a miss).
                     // The misses form the tile list of the second pass; without a prediction every slot and the shared expert miss.
@@ -554,46 +459,19 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
             if (E == 512) route_token<8>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp, ready);
             else route_token<16>(fetch, E, k, lane, ids + t * k, weights + t * k, scratch, stamp, ready);
         }
-        if constexpr (NT == 1) {
+        {
             // (the waves other than the routing wave go straight to the prediction pass below and wait for the ids after it)
-        } else {
-            if (tid < T) gatev[tid] = bf(sigmoid_bf(load_shared_f32(p.gate + tid)));   // the combine's gate factor, ready early
-            for (uint32_t e = tid; e < E; e += blockDim.x) head[e] = -1;
-            __syncthreads();
         }
         clock(6);
         if (tid < n) {
             const int32_t e = ids[tid];
-            if (e < 0 || e >= int32_t(E)) { atomicOr(p.status, 1); if constexpr (NT != 1) next[tid] = -1; }
-            else if constexpr (NT != 1) next[tid] = atomicExch(&head[e], int32_t(tid));
+            if (e < 0 || e >= int32_t(E)) atomicOr(p.status, 1);
             if (wg == 0 && p.ids_trace) { st_i32(p.ids_trace + uint64_t(layer) * p.trace_tokens * k + tid, e); st_f32(p.weights_trace + uint64_t(layer) * p.trace_tokens * k + tid, weights[tid]); }
-            if (NT == 1 && wg == 0 && p.pred_out) p.pred_out[uint64_t(layer) * k + tid] = e;   // the next step's guess for this layer
+            if (wg == 0 && p.pred_out) p.pred_out[uint64_t(layer) * k + tid] = e;   // the next step's guess for this layer
         }
-        // One token: slot j belongs to expert ids[j] and no two slots share an expert, so there is nothing to group.
-        uint32_t U = k;
-        if constexpr (NT != 1) {
-        __syncthreads();
-        {   // compact the experts that own at least one slot (any order: slots are independent)
-            uint32_t base = 0;
-            for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
-                const uint32_t e = e0 + tid;
-                const bool used = e < E && head[e] >= 0;
-                const uint64_t m = __ballot(used);
-                if (lane == 0) misc[1 + wave] = __popcll(m);
-                __syncthreads();
-                uint32_t before = base;
-                for (uint32_t w = 0; w < wave; ++w) before += misc[1 + w];
-                if (used) experts[before + __popcll(m & ((1ull << lane) - 1))] = int32_t(e);
-                for (uint32_t w = 0; w < kDecodeWaves; ++w) base += misc[1 + w];
-                __syncthreads();
-            }
-            if (tid == 0) misc[0] = int32_t(base);
-        }
-        __syncthreads();
-        U = uint32_t(uniform(misc[0]));
-        }
+        // (slot j belongs to expert ids[j] and no two slots share an expert, so there is nothing to group)
         clock(7);
-        if constexpr (NT == 1) {
+        {
             // Two passes over gate/up tiles.  Pass 0 runs BEFORE the ids are known, on the seven waves that do not route: the
             // tiles of the experts this layer picked at the previous step (the reference predicts a layer's experts for its
             // prefetcher, model.cpp:438-445; here the guess buys the time of the router, the exchange of the logits and the
@@ -669,7 +547,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         const uint32_t a = __float_as_uint(swiglu_bf(v, up));
                         if (lane < 8) ZC_ST(out_row + row, (a & 0xffff0000u) | tag);
                     };
-                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
+                    xint_run_tile<PT, 4>(w_row, s_row, b_row, H / 128, img, src, LH, lane, 1, emit);
                 }
             }
             if (tid == 64) {   // the combine's gate factor (written by another workgroup)
@@ -677,42 +555,19 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 bar.until([&]() { w = ZC_LD(p.tlogits + E); return uint32_t(w >> 32) == tag; });
                 gatev[0] = bf(sigmoid_bf(__uint_as_float(uint32_t(w))));
             }
-        } else {
-            const uint32_t tiles = I / 8, units = U * tiles;
-            for (uint32_t u = wg + nwg * wave; u < units; u += nwg * kDecodeWaves) {
-                const uint32_t e = uint32_t(uniform(experts[u / tiles])), tile = u % tiles;
-                const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
-                const uint8_t* rec = record_of(L, e);
-                const uint8_t* w_row = rec + p.ro[pr] + uint64_t(row) * (H / 2);
-                const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 1]) + uint64_t(row) * (H / 64);
-                const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + p.ro[pr + 2]) + uint64_t(row) * (H / 64);
-                int32_t s = uniform(head[e]);
-                while (s >= 0) {   // the expert's slots, PT at a time
-                    const uint8_t* img[PT]; LdsBf16 src[PT]; int32_t slot[PT]; int nt = 0;
-#pragma unroll
-                    for (int t = 0; t < PT; ++t) { slot[t] = s; if (s >= 0) { nt = t + 1; s = uniform(next[s]); } }
-#pragma unroll
-                    for (int t = 0; t < PT; ++t) {
-                        const uint32_t tt = t < nt ? uint32_t(slot[t]) / k : 0;
-                        img[t] = lds + lp.img_rg + tt * LH.bytes(); src[t] = LdsBf16{xh_all + tt * H};
-                    }
-                    auto emit = [&](int t, float v) { store_act(p.act, uint32_t(slot[t]), row, v); };
-                    ZC_RUN_TILE(H / 128, w_row, s_row, b_row, H / 128, img, src, LH, lane, nt, emit);
-                }
-            }
         }
         clock_all(8);
-        if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the staging below polls the activations themselves
+        __syncthreads();   // the staging below polls the activations themselves
         refresh();
         clock(9);
         // ---------------- phase D: down tiles per 16 output rows, combine ----------------
         float* otile = reinterpret_cast<float*>(lds + lp.otile);
         const uint32_t slots_total = n + T, SB = lp.slots_per_batch;
         if (wg >= H / 16) { clock(10); clock(11); clock(12); }   // workgroups without a row tile keep the stamp count
-        if constexpr (NT == 1) { if (wg >= H / 16) bar.arrive(); }
+        { if (wg >= H / 16) bar.arrive(); }
         for (uint32_t rt = wg; rt < H / 16; rt += nwg) {
             const uint32_t row = rt * 16 + col;
-            if (!MIXED && NT == 1 && SB >= slots_total && I == 1024) {
+            if (!MIXED && SB >= slots_total && I == 1024) {
                 // One token, all slots' images resident, tiles of two bodies (intermediate 1024): every wave works alone.  It requests the first weights of its slot's
                 // tile, then polls that slot's activations (one 16-element block per lane), builds the slot's image and the
                 // BF16 copy under the latency of those loads, and runs the tile; no workgroup barrier until the combine, and
@@ -785,7 +640,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 __syncthreads();
                 uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
                 auto source_of = [&](uint32_t q) { return LdsBf16{ah + q * I}; };
-                if constexpr (NT == 1) {
+                {
                     // One token: a thread fetches whole 16-element blocks of the activations (32 bytes) and builds their
                     // image pieces straight from registers; the BF16 copy for the literal chain is written on the way.
                     const uint32_t per = I / 16, total = sn * per;
@@ -850,19 +705,8 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                     if (s0 == 0) { clock(10); clock(11); }
                     __syncthreads();
                     if (rt + nwg >= H / 16 && s0 + SB >= slots_total) bar.arrive();   // nothing more to read from other workgroups in this layer
-                } else {
-                    {   // rows s0 .. s0+sn-1 of [act ; shared_act]: contiguous except across the seam between the two buffers
-                        const uint32_t routed = s0 < n ? min(sn, n - s0) : 0;
-                        if (routed) stage_copy<6>(reinterpret_cast<const uint64_t*>(p.act) + uint64_t(s0) * I / 4, routed * I / 4, reinterpret_cast<uint64_t*>(ah));
-                        if (sn > routed) stage_copy<6>(reinterpret_cast<const uint64_t*>(p.shared_act) + uint64_t(s0 + routed - n) * I / 4, (sn - routed) * I / 4,
-                                                       reinterpret_cast<uint64_t*>(ah + routed * I));
-                    }
-                    __syncthreads();
-                    if (s0 == 0) clock(10);
-                    xint_prepare_batch(source_of, sn, LI, lds + lp.img_d);
-                    if (s0 == 0) clock(11);
                 }
-                if constexpr (NT == 1) {
+                {
                     for (uint32_t slot = wave; slot <= k; slot += kDecodeWaves) {   // slot k is the shared expert's
                         if (slot < s0 || slot >= s0 + sn) continue;
                         const uint8_t* rec = L.shared_record; const uint64_t* off = p.so;
@@ -882,40 +726,12 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                         const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
                         const uint8_t* img[PT] = {lds + lp.img_d + (slot - s0) * LI.bytes()}; LdsBf16 src[PT] = {source_of(slot - s0)};
                         auto emit = [&](int, float v) { if (G == 0) otile[slot * 16 + col] = bf(v); };
-                        ZC_RUN_TILE(I / 128, w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit);
-                    }
-                } else
-                for (uint32_t u = wave; u <= U; u += kDecodeWaves) {
-                    const uint8_t* rec; const uint64_t* off; int32_t s;
-                    if (u < U) { const uint32_t e = uint32_t(uniform(experts[u])); s = uniform(head[e]); rec = record_of(L, e); off = p.ro; }
-                    else { s = int32_t(n); rec = L.shared_record; off = p.so; }
-                    const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
-                    const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
-                    const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
-                    while (u < U ? s >= 0 : uint32_t(s) < n + T) {
-                        // next PT slots of this unit that lie in the batch
-                        int32_t slot[PT]; int nt = 0;
-#pragma unroll
-                        for (int t = 0; t < PT; ++t) slot[t] = int32_t(s0);
-                        while (nt < PT && (u < U ? s >= 0 : uint32_t(s) < n + T)) {
-                            if (uint32_t(s) >= s0 && uint32_t(s) < s0 + sn) {
-#pragma unroll
-                                for (int q = 0; q < PT; ++q) if (q == nt) slot[q] = s;
-                                ++nt;
-                            }
-                            s = u < U ? uniform(next[s]) : s + 1;
-                        }
-                        if (!nt) break;
-                        const uint8_t* img[PT]; LdsBf16 src[PT];
-#pragma unroll
-                        for (int t = 0; t < PT; ++t) { img[t] = lds + lp.img_d + (uint32_t(slot[t]) - s0) * LI.bytes(); src[t] = source_of(uint32_t(slot[t]) - s0); }
-                        auto emit = [&](int t, float v) { if (G == 0) otile[uint32_t(slot[t]) * 16 + col] = bf(v); };
-                        ZC_RUN_TILE(I / 128, w_row, s_row, b_row, I / 128, img, src, LI, lane, nt, emit);
+                        xint_run_tile<PT, 4>(w_row, s_row, b_row, I / 128, img, src, LI, lane, 1, emit);
                     }
                 }
             }
             __syncthreads();
-            if (!MIXED && NT == 1 && SB >= slots_total && I == 1024 && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
+            if (!MIXED && SB >= slots_total && I == 1024 && rt + nwg >= H / 16) bar.arrive();   // every wave has read its slots' activations
             clock(12);
             // weighted combine of the tile (reference: qwen.metal:804-816)
             if (tid < T * 16) {
@@ -923,7 +739,7 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 float partial[8];
 #pragma unroll
                 for (int q = 0; q < 8; ++q) partial[q] = 0;
-                const bool products = !MIXED && NT == 1 && SB >= slots_total && I == 1024;   // the waves left products, not outputs
+                const bool products = !MIXED && SB >= slots_total && I == 1024;   // the waves left products, not outputs
                 if (products) {
                     for (uint32_t base = 0; base < k; base += 8) {
                         float value[8];
@@ -949,21 +765,13 @@ __global__ __launch_bounds__(decode_threads(NT)) void decode_stack_kernel(Decode
                 for (uint32_t kk = 1; kk < 8 && kk < k; ++kk) sum += partial[kk];
                 const float y = bf(bf(sum) + (products ? otile[n * 16 + c] : bf(gatev[t] * otile[(n + t) * 16 + c])));
                 const uint64_t at = uint64_t(t) * H + rt * 16 + c;
-                if constexpr (NT == 1) ZC_ST(p.tout + (layer & 1u) * H + at, (__float_as_uint(y) & 0xffff0000u) | tag);   // y is BF16-valued
-                else st_f32(p.layer_out + at, y);
+                ZC_ST(p.tout + (layer & 1u) * H + at, (__float_as_uint(y) & 0xffff0000u) | tag);   // y is BF16-valued
                 if (p.out_trace) st_f32(p.out_trace + uint64_t(layer) * p.trace_tokens * H + at, y);
                 if (layer + 1 == p.L) st_f32(p.out + at, y);
-                if constexpr (NT != 1) {   // one token: the next layer's staging finds the maximum itself
-                    uint32_t m = __float_as_uint(y) & 0x7fffffffu;
-                    if (m > 0x7f800000u) m = 0;   // NaN does not take part in the maximum
-#pragma unroll
-                    for (int o = 8; o; o >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), o)));
-                    if (c == 0) __hip_atomic_fetch_max(p.maxabs + layer * T + t, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
             }
         }
         clock_all(13);
-        if constexpr (NT == 1) __syncthreads(); else bar.wait();   // one token: the next layer polls the output words themselves
+        __syncthreads();   // the next layer polls the output words themselves
         clock(14);
     }
 }
@@ -976,7 +784,7 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
     uint32_t at = 0;
     auto take = [&](uint32_t bytes) { const uint32_t o = at; at += align16(bytes); return o; };
     lp.ids = take(NT * topk * 4); lp.weights = take(NT * topk * 4); lp.gatev = take(NT * 4);
-    lp.head = take(E * 4); lp.next = take(NT * topk * 4); lp.experts = take(E * 4); lp.misc = take(64); lp.gatew = take(H * 2);
+    lp.experts = take(E * 4); lp.misc = take(64); lp.gatew = take(H * 2);
     lp.spec = take((2 * (topk + 1) + 1) * 4);
     lp.region = at;
     lp.img_rg = lp.region; lp.xh = lp.img_rg + NT * LH.bytes();
@@ -1002,10 +810,10 @@ DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I,
 hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt, uint32_t workgroups, const DecodeLdsPlan& lp) {
 #define ZC_DECODE(MIXED)                                                                                               \
     do {                                                                                                               \
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1, MIXED>),                \
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<MIXED>),                \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lp.total));                 \
         if (e != hipSuccess) return e;                                                                                 \
-        hipLaunchKernelGGL((decode_stack_kernel<1, MIXED>), dim3(workgroups), dim3(decode_threads(1)), lp.total, s, p, lp);  \
+        hipLaunchKernelGGL((decode_stack_kernel<MIXED>), dim3(workgroups), dim3(decode_threads(1)), lp.total, s, p, lp);  \
     } while (0)
     (void)nt;   // two to eight tokens run decode_multi_kernel (zc_decode_multi.hip)
     if (p.bits_down == 4 && p.shared_bits_gate_up == 4 && p.shared_bits_down == 4) ZC_DECODE(false); else ZC_DECODE(true);
@@ -1015,14 +823,14 @@ hipError_t launch_decode_stack(hipStream_t s, const DecodeParams& p, uint32_t nt
 hipError_t decode_stack_occupancy(uint32_t nt, uint32_t lds_bytes, int* blocks_per_cu) {
     (void)nt;
     // both variants have the same launch bounds and dynamic LDS; the mixed one uses no more registers than the other
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1, false>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<1, true>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stack_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
     int plain = 0, mixed = 0;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, decode_stack_kernel<1, false>, decode_threads(1), lds_bytes);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, decode_stack_kernel<false>, decode_threads(1), lds_bytes);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&mixed, decode_stack_kernel<1, true>, decode_threads(1), lds_bytes);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&mixed, decode_stack_kernel<true>, decode_threads(1), lds_bytes);
     *blocks_per_cu = plain < mixed ? plain : mixed;
     return e;
 }

@@ -88,7 +88,7 @@ struct DecodeParams {
 };
 constexpr uint32_t kDecodeStamps = 24;
 struct DecodeLdsPlan {
-    uint32_t ids, weights, gatev, head, next, experts, misc, region, total;
+    uint32_t ids, weights, gatev, experts, misc, region, total;
     uint32_t img_rg, xh, gprod, img_d, ah, otile, slots_per_batch, gatew, spec;
 };
 DecodeLdsPlan decode_lds_plan(uint32_t H, uint32_t E, uint32_t topk, uint32_t I, uint32_t NT, uint32_t lds_limit);

@@ -33,10 +33,14 @@ constexpr int kWideBatch = 8;                // tokens whose rows and images a w
 constexpr int kWidePass = ZC_WIDE_PASS_TOKENS;
 constexpr uint32_t kWideThreads = kWidePass <= 2 ? 512 : 256, kWideWaves = kWideThreads / 64;
 
-template <class Emit>
+template <bool T32, class Emit>
 __device__ __forceinline__ void run_tile_wide(const uint8_t* w_row, const uint16_t* s_row, const uint16_t* b_row, uint32_t spans, const uint8_t* const* img,
                                               const LdsBf16* src, const XintLayout L, uint32_t lane, int nt, Emit emit) {
-    if constexpr (kWidePass == 8) xint_run_tile_upto8(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    if constexpr (T32) {   // tiles of 32 weight rows on the 32x32x32 instruction
+        if (nt <= 1) xint_run_tile32<1>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+        else if (kWidePass == 2 || nt == 2) xint_run_tile32<2>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+        else if constexpr (kWidePass >= 4) xint_run_tile32<4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
+    } else if constexpr (kWidePass == 8) xint_run_tile_upto8(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     else if (nt <= 1) xint_run_tile_tokens<1, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
     else xint_run_tile_tokens_piped<2, 4>(w_row, s_row, b_row, spans, img, src, L, lane, nt, emit);
 }
@@ -46,6 +50,8 @@ __device__ __forceinline__ void run_tile_wide(const uint8_t* w_row, const uint16
 template <bool MIXED>
 __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams p, WideLdsPlan lp) {
     constexpr int PT = kWidePass, MT = kWideBatch;
+    constexpr bool T32 = !MIXED && (kWidePass == 2 || kWidePass == 4);
+    constexpr uint32_t TR = T32 ? 16 : 8, DR = T32 ? 32 : 16;   // gate (and up) rows of a gate/up tile, rows of a down tile
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, col = lane & 15u, G = lane >> 4;
     const uint32_t wg = blockIdx.x, nwg = gridDim.x;
@@ -68,10 +74,10 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
     auto clock_all = [&]() { if (p.clocks) __syncthreads(); clock(); };
 
     auto store_act = [&](float* buffer, uint32_t slot_row, uint32_t row, float v) {   // SwiGLU of a gate/up tile as packed BF16 pairs
-        const float up = __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
+        const float up = T32 ? __shfl(v, (lane & ~31u) | ((lane & 15u) + 16u)) : __shfl(v, (lane & ~15u) | ((col & 7u) + 8u));
         const uint32_t a = __float_as_uint(swiglu_bf(v, up));
         const uint32_t other = uint32_t(__shfl_xor(int(a), 1));
-        if (lane < 8 && !(lane & 1u))
+        if (lane < TR && !(lane & 1u))
             ZC_ST(reinterpret_cast<uint32_t*>(buffer) + (uint64_t(slot_row) * I + row) / 2, (a >> 16) | (other & 0xffff0000u));
     };
     // exclusive prefix of `mine` over the threads of the workgroup, and the total; every thread calls it
@@ -315,7 +321,7 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
             const bool q8_shared = MIXED && p.shared_bits_gate_up == 8;
             const uint32_t cut = q8_shared ? 4u : 1u, routed_passes = uint32_t(cum[U]);
             auto gcum = [&](uint32_t i) { const uint32_t c = uint32_t(uniform(cum[i])); return i <= U ? c : routed_passes + cut * (c - routed_passes); };
-            const uint32_t tiles = I / 8, total = tiles * gcum(NE);
+            const uint32_t tiles = I / TR, total = tiles * gcum(NE);
             uint32_t i0, i1;
             share_of_items(wg, nwg, total, kWideWaves, i0, i1);
             uint32_t ei = 0;
@@ -360,7 +366,7 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
                         continue;
                     }
                     const uint32_t tile = (item - first) / passes, pass = pass_of_item(item - first, passes, kWideWaves);
-                    const uint32_t row = tile * 8 + (col & 7u), pr = col < 8 ? 0 : 3;
+                    const uint32_t row = T32 ? tile * 16 + (lane & 15u) : tile * 8 + (col & 7u), pr = T32 ? ((lane & 31u) < 16 ? 0 : 3) : (col < 8 ? 0 : 3);
                     const uint8_t* w_row = rec + off[pr] + uint64_t(row) * (H / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 1]) + uint64_t(row) * (H / 64);
                     const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[pr + 2]) + uint64_t(row) * (H / 64);
@@ -372,7 +378,7 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
                     auto emit = [&](int t, float v) {
                         if (routed) store_act(p.act, uint32_t(slot[t]), row, v); else store_act(p.shared_act, uint32_t(slot[t]) - n, row, v);
                     };
-                    run_tile_wide(w_row, s_row, b_row, H / 128, img, src, LH, lane, nt, emit);
+                    run_tile_wide<T32>(w_row, s_row, b_row, H / 128, img, src, LH, lane, nt, emit);
                 }
                 at = seg_end;
             }
@@ -383,7 +389,7 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
         clock();
         // ---------------- phase D: down tiles; items (entry, row tile, pass), one contiguous range per workgroup ----------------
         {
-            const uint32_t row_tiles = H / 16, total = row_tiles * uint32_t(cum[NE]);
+            const uint32_t row_tiles = H / DR, total = row_tiles * uint32_t(cum[NE]);
             uint32_t i0, i1;
             share_of_items(wg, nwg, total, kWideWaves, i0, i1);
             uint16_t* ah = reinterpret_cast<uint16_t*>(lds + lp.ah);
@@ -411,7 +417,7 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
                 const uint32_t passes = uint32_t(na + PT - 1) / PT;
                 for (uint32_t item = at + wave; item < seg_end; item += kWideWaves) {
                     const uint32_t pass = pass_of_item(item - first, passes, kWideWaves);
-                    const uint32_t row = ((item - first) / passes) * 16 + col;
+                    const uint32_t row = ((item - first) / passes) * DR + (T32 ? (lane & 31u) : col);
                     const uint8_t* w_row = rec + off[6] + uint64_t(row) * (I / 2);
                     const uint16_t* s_row = reinterpret_cast<const uint16_t*>(rec + off[7]) + uint64_t(row) * (I / 64);
                     const uint16_t* b_row = reinterpret_cast<const uint16_t*>(rec + off[8]) + uint64_t(row) * (I / 64);
@@ -430,8 +436,8 @@ __global__ __launch_bounds__(kWideThreads) void decode_wide_kernel(DecodeParams 
                     const uint8_t* img[PT]; LdsBf16 src[PT];
 #pragma unroll
                     for (int t = 0; t < PT; ++t) { img[t] = lds + lp.img_d + index[t] * LI.bytes(); src[t] = LdsBf16{ah + index[t] * I}; }
-                    auto emit = [&](int t, float v) { if (G == 0) st_f32(p.eout + uint64_t(slot[t]) * H + row, bf(v)); };
-                    run_tile_wide(w_row, s_row, b_row, I / 128, img, src, LI, lane, nt, emit);
+                    auto emit = [&](int t, float v) { if (T32 ? lane < 32 : G == 0) st_f32(p.eout + uint64_t(slot[t]) * H + row, bf(v)); };
+                    run_tile_wide<T32>(w_row, s_row, b_row, I / 128, img, src, LI, lane, nt, emit);
                 }
                 at = seg_end;
             }

@@ -699,6 +699,13 @@ __device__ __forceinline__ void xint_run_tile32(const uint8_t* w_row, const uint
 #pragma unroll
     for (int e = 0; e < 16; ++e) zero[e] = 0;
     const uint32_t info_at = L.planes_bytes() + 4 * h * 8, mask_at = L.planes_bytes() + L.info_bytes();
+    // lane q < NTOK holds where token q's BF16 row starts, in elements from src[0]'s (a select chain over the tokens would be
+    // turned into a table in memory by the compiler)
+    uint32_t row_table = 0;
+    if constexpr (Source::kRowInLds) {
+#pragma unroll
+        for (int q = 1; q < NTOK; ++q) row_table = lane == uint32_t(q) ? uint32_t(src[q].x - src[0].x) : row_table;
+    }
     for (uint32_t d0 = 0; d0 < spans; d0 += R) {
         const uint32_t sdw[4] = {sring.x, sring.y, sring.z, sring.w}, bdw[4] = {bring.x, bring.y, bring.z, bring.w};
         if (d0 + R < spans) { sring = ldg_u4(s_row, (d0 + R) / 4); bring = ldg_u4(b_row, (d0 + R) / 4); }
@@ -728,8 +735,9 @@ __device__ __forceinline__ void xint_run_tile32(const uint8_t* w_row, const uint
             float dot[NTOK][4], bsum[NTOK][4];
 #pragma unroll
             for (int t = 0; t < NTOK; ++t) {
-                const float4 f0 = *reinterpret_cast<const float4*>(img[t < nt ? t : 0] + info_at + d * 64);        // {2^e, sum} of blocks 4h, 4h+1
-                const float4 f1 = *reinterpret_cast<const float4*>(img[t < nt ? t : 0] + info_at + d * 64 + 16);   // of blocks 4h+2, 4h+3
+                const uint8_t* image = t < nt ? img[t] : img[0];   // (two fixed elements, not an index formed at run time: the array stays in registers)
+                const float4 f0 = *reinterpret_cast<const float4*>(image + info_at + d * 64);        // {2^e, sum} of blocks 4h, 4h+1
+                const float4 f1 = *reinterpret_cast<const float4*>(image + info_at + d * 64 + 16);   // of blocks 4h+2, 4h+3
                 dot[t][0] = f0.x; bsum[t][0] = f0.y; dot[t][1] = f0.z; bsum[t][1] = f0.w;
                 dot[t][2] = f1.x; bsum[t][2] = f1.y; dot[t][3] = f1.z; bsum[t][3] = f1.w;
             }
@@ -759,11 +767,11 @@ __device__ __forceinline__ void xint_run_tile32(const uint8_t* w_row, const uint
 #pragma unroll
                     for (int t = 0; t < NTOK; ++t) pending |= ((unsafe[t] >> (8 * j)) & 15u) << (4 * t);
                     while (__ballot(pending != 0) != 0) {
+                        // (every lane is active here: the row of token t is lane t's entry of the table, fetched across lanes)
+                        const uint32_t item = uint32_t(__builtin_ctz(pending | 0x80000000u)), t = (item >> 2) & uint32_t(NTOK - 1), i = item & 3u;
+                        const uint32_t row_at = uint32_t(__builtin_amdgcn_ds_bpermute(int(4 * t), int(row_table)));
                         if (pending) {
-                            const uint32_t item = uint32_t(__builtin_ctz(pending)), t = item >> 2, i = item & 3u;
-                            const uint16_t* row = src[0].x;
-#pragma unroll
-                            for (int q = 1; q < NTOK; ++q) row = t == uint32_t(q) ? src[q].x : row;
+                            const uint16_t* row = src[0].x + int32_t(row_at);   // (a signed distance)
                             uint32_t lo = words[0], hi = words[1];
 #pragma unroll
                             for (int q = 1; q < 4; ++q) { lo = i == uint32_t(q) ? words[2 * q] : lo; hi = i == uint32_t(q) ? words[2 * q + 1] : hi; }

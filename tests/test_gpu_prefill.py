@@ -159,12 +159,12 @@ def test_prefill_full_size_unskewed(ctx):
         ctx.free(b)
 
 
-def test_prefill_reports_unroutable_rows(ctx):
+@pytest.mark.parametrize("T", [70, 300])   # 300 tokens: the router on bounds with the selection in its launch, and the one-launch dispatch sort
+def test_prefill_reports_unroutable_rows(ctx, T):
     # A NaN row gives that token no selectable expert (ids -1): its sorted positions are not covered by any tile.  The
     # call must end normally and the check must report "invalid router output", as the exact path does.
     cfg = workload.tiny_config(512, 32, 4, 128)
     weights = workload.LayerWeights(ctx, cfg, 94, ("normal", 0.5))
-    T = 70
     ws = ctx.alloc(ctx.moe_prefill_workspace_bytes(cfg, T)); out = ctx.alloc(T * cfg.hidden * 4)
     good = workload.hidden_rows(ctx, T, cfg.hidden, 95)
     ctx.fill(ws, 0xff)                        # whatever an earlier call could have left in the recomputation map: all bits set

@@ -136,7 +136,7 @@ def prefill_workload(ctx, args):
         "metric": "moe_prefill_tokens_per_s", "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["us_per_layer"] * 1e-3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u4 codes as bf16 x bf16 inputs, fp32 accumulation", "data": "synthetic (seeded generator)",
-        "config": {"workload": "BASELINE configs[3]: one MoE layer, 2048-token prefill batch, hidden 2048, 512 experts, top-10, "
+        "config": {"workload": "BASELINE configs[2]: one MoE layer, 2048-token prefill batch, hidden 2048, 512 experts, top-10, "
                                "intermediate 512, affine Q4 group 64, no router skew", "tokens": args.prefill_tokens,
                    "with_zipf_1.1_router_offsets": {"us_per_layer": skewed["us_per_layer"], "tokens_per_s": skewed["tokens_per_s"], "TFLOPs": skewed["TFLOPs"]}},
         "roofline": {"bound": "mfma", "achieved": r["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s", "frac": r["TFLOPs"] / 2500.0,
